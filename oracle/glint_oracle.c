@@ -1,0 +1,470 @@
+/*
+ * glint_oracle.c -- CPU restatement of Glinthawk's amd64/OpenMP Llama2 KV-cache path.
+ *
+ * TEST INFRASTRUCTURE ONLY: loaded by the tests, by the smoke check and by the benchmark's
+ * cpu_baseline leg as the checker / the timed CPU baseline.  Never linked into, imported by or
+ * called from the HIP product path.
+ *
+ * The reference cannot be compiled in this build environment without writing a stand-in for its
+ * logging dependency (glog headers are absent) and its fp16 alias needs a newer GCC, so no
+ * compiled-reference binary backs this file.  The reference holds no tests, golden vectors or
+ * fixtures for this path either.  Each function is therefore pinned by what the mathematics
+ * fixes, in tests/test_oracle_*.py:
+ *
+ *   go_half_to_float / go_float_to_half   all 65536 patterns and rounding cases vs numpy.float16
+ *   go_accum, go_silu                     float64 closed forms; fp16 variant vs numpy rounding
+ *   go_rmsnorm                            float64 closed form; unit-norm invariant; eps placement
+ *                                         (all-zero row -> 0, tiny rows scale by 1/sqrt(eps))
+ *   go_argmax                             numpy.argmax incl. ties (first index), fp16 ties
+ *   go_matmul                             numpy float64 x @ W.T; identity / one-hot rows pick columns
+ *   go_gumbel                             float64 closed form with given uniforms
+ *   go_copy_kv_cache                      bit-exact vs slice assignment; empty rows untouched;
+ *                                         canaries around every row
+ *   go_apply_rope                         complex multiplication (x0 + i x1) e^{i pos theta_k} in
+ *                                         float64; norm preservation; pos 0 identity; V untouched;
+ *                                         interleaved (not half-split) pairing
+ *   go_attention_0_gemm                   numpy einsum float64; entries beyond pos untouched;
+ *                                         one-hot query picks a key column; gqa head -> kv head map
+ *   go_softmax_row / go_attention_softmax scipy.special.softmax float64; rows sum to 1; shift
+ *                                         invariance; fp16 variant within 1 half-ulp model
+ *   go_attention_2_gemm                   numpy einsum float64; uniform weights -> mean of V
+ *   go_attention_ops                      composition vs float64 end-to-end attention; pos 0 -> V row 0
+ *   go_layer_forward_f32, go_classify_f32 float64 numpy transformer block (independent einsum code)
+ *   go_rope_tables_f32                    closed form vs numpy float64
+ *   go_ctx_* addressing                   brute force enumeration on small shapes; disjointness
+ *   go_dynctx_prepare                     brute-force page model (set of committed blocks)
+ *   go_ctxman_*                           random op sequences vs a dict + deque model
+ *   go_check_finished, temperature codec  exhaustive truth table on small ranges
+ *
+ * What stays unpinned bit-for-bit: the last-ulp effect of the reference's -ffast-math build
+ * (compiler specific) and the exact fp16 rounding sequence inside softmax for DType = _Float16
+ * (read from source, arch/amd64/llama2/ops.hh:124-130; bounded by tolerance, not bit-checked).
+ */
+#include "glint_oracle.h"
+
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#if defined( __F16C__ )
+#include <immintrin.h>
+#endif
+
+/* ---------------------------------------------------------------------------------------------
+ * binary16 <-> binary32.  `static_cast<float>(_Float16)` is exact; `static_cast<_Float16>(float)`
+ * rounds to nearest, ties to even (what the reference's DType( sum ) stores do).
+ * ------------------------------------------------------------------------------------------- */
+static inline float half_bits_to_float( go_half h )
+{
+#if defined( __F16C__ )
+  return _cvtsh_ss( h );
+#else
+  const uint32_t sign = (uint32_t)( h & 0x8000u ) << 16;
+  const uint32_t exp = ( h >> 10 ) & 0x1fu;
+  uint32_t man = h & 0x3ffu;
+  uint32_t bits;
+  if ( exp == 0 ) {
+    if ( man == 0 ) {
+      bits = sign;
+    } else {
+      /* subnormal: renormalise */
+      int e = -1;
+      do {
+        man <<= 1;
+        e++;
+      } while ( ( man & 0x400u ) == 0 );
+      bits = sign | ( (uint32_t)( 127 - 15 - e ) << 23 ) | ( ( man & 0x3ffu ) << 13 );
+    }
+  } else if ( exp == 31 ) {
+    bits = sign | 0x7f800000u | ( man << 13 );
+  } else {
+    bits = sign | ( ( exp + 127 - 15 ) << 23 ) | ( man << 13 );
+  }
+  float f;
+  memcpy( &f, &bits, sizeof( f ) );
+  return f;
+#endif
+}
+
+static inline go_half float_to_half_bits( float f )
+{
+#if defined( __F16C__ )
+  return _cvtss_sh( f, _MM_FROUND_TO_NEAREST_INT | _MM_FROUND_NO_EXC );
+#else
+  uint32_t x;
+  memcpy( &x, &f, sizeof( x ) );
+  const uint32_t sign = ( x >> 16 ) & 0x8000u;
+  x &= 0x7fffffffu;
+  if ( x >= 0x7f800000u ) { /* inf / nan */
+    return (go_half)( sign | 0x7c00u | ( x > 0x7f800000u ? 0x200u | ( ( x >> 13 ) & 0x3ffu ) : 0 ) );
+  }
+  if ( x >= 0x477ff000u ) { /* rounds to >= 65520 -> inf */
+    return (go_half)( sign | 0x7c00u );
+  }
+  if ( x < 0x33000001u ) { /* <= 2^-25 -> 0 (ties to even gives 0 at exactly 2^-25) */
+    return (go_half)sign;
+  }
+  const int32_t e = (int32_t)( x >> 23 ) - 127;
+  uint32_t man = ( x & 0x7fffffu ) | 0x800000u;
+  uint32_t shift;
+  uint32_t base;
+  if ( e < -14 ) { /* subnormal half */
+    shift = (uint32_t)( 13 + ( -14 - e ) );
+    base = 0;
+  } else {
+    shift = 13;
+    base = (uint32_t)( e + 15 ) << 10;
+    man &= 0x7fffffu;
+  }
+  const uint32_t q = man >> shift;
+  const uint32_t rem = man & ( ( 1u << shift ) - 1 );
+  const uint32_t halfway = 1u << ( shift - 1 );
+  uint32_t out = base + q;
+  if ( rem > halfway || ( rem == halfway && ( out & 1u ) ) ) {
+    out++;
+  }
+  return (go_half)( sign | out );
+#endif
+}
+
+float go_half_to_float( go_half h ) { return half_bits_to_float( h ); }
+go_half go_float_to_half( float f ) { return float_to_half_bits( f ); }
+
+/* arch/amd64/llama2/ops.hh:354-368 (convert_and_copy: element-wise static_cast) */
+void go_convert_f16_to_f32( float* dst, const go_half* src, uint64_t n )
+{
+#pragma omp parallel for
+  for ( uint64_t i = 0; i < n; i++ ) {
+    dst[i] = half_bits_to_float( src[i] );
+  }
+}
+
+void go_convert_f32_to_f16( go_half* dst, const float* src, uint64_t n )
+{
+#pragma omp parallel for
+  for ( uint64_t i = 0; i < n; i++ ) {
+    dst[i] = float_to_half_bits( src[i] );
+  }
+}
+
+/* ---- storage type = float ---- */
+#define T float
+#define LD( x ) ( x )
+#define ST( f ) ( (float)( f ) )
+#define FN( name ) name##_f32
+#include "glint_oracle_ops.inc"
+#undef T
+#undef LD
+#undef ST
+#undef FN
+
+/* ---- storage type = binary16 ---- */
+#define T go_half
+#define LD( x ) half_bits_to_float( x )
+#define ST( f ) float_to_half_bits( (float)( f ) )
+#define FN( name ) name##_f16
+#include "glint_oracle_ops.inc"
+#undef T
+#undef LD
+#undef ST
+#undef FN
+
+/* tools/bin2glint.py:19-25 -- freqs = theta^(-(2k)/head_size); table[pos][k] = cos/sin(pos * freqs[k]),
+ * computed in fp32 like the converter's torch.float32 tensors. */
+void go_rope_tables_f32( float* real, float* imag, uint64_t seq_len, uint64_t head_size, float theta )
+{
+  const uint64_t half = head_size / 2;
+  for ( uint64_t k = 0; k < half; k++ ) {
+    const float freq = 1.0f / powf( theta, (float)( 2 * k ) / (float)head_size );
+    for ( uint64_t p = 0; p < seq_len; p++ ) {
+      const float angle = (float)p * freq;
+      real[p * half + k] = cosf( angle );
+      imag[p * half + k] = sinf( angle );
+    }
+  }
+}
+
+/* models/llama2/model.hh:326-427 -- one full layer in the order the reference issues the ops:
+ * rmsnorm, wq, wkv, kv append | rope, scores, softmax, weighted sum | wo, accum, rmsnorm, w1, w3,
+ * silu, w2, accum. */
+void go_layer_forward_f32( const go_config* c,
+                           const go_layer_weights_f32* w,
+                           const float* freq_cis_real,
+                           const float* freq_cis_imag,
+                           go_scratch_f32* s,
+                           float* const* layer_ctx,
+                           const uint32_t* token_positions,
+                           uint64_t batch )
+{
+  float** token_ctx = (float**)malloc( sizeof( float* ) * ( batch ? batch : 1 ) );
+  for ( uint64_t i = 0; i < batch; i++ ) {
+    token_ctx[i] = layer_ctx[i] ? layer_ctx[i] + (uint64_t)token_positions[i] * 2 * c->kv_dim : NULL;
+  }
+
+  /* pre-attention: model.hh:326-351 */
+  go_rmsnorm_f32( s->xb, s->x, w->rms_att_weight, c->dim, batch );
+  go_matmul_f32( s->q, s->xb, w->wq, c->dim, c->dim, batch );
+  go_matmul_f32( s->kv, s->xb, w->wkv, c->dim, 2 * c->kv_dim, batch );
+  go_copy_kv_cache_f32( c, token_ctx, s->kv, batch );
+
+  /* attention: model.hh:354-387 */
+  go_apply_rope_f32( c, batch, token_positions, freq_cis_real, freq_cis_imag, s->q, token_ctx );
+  go_attention_0_gemm_f32( c, s->q, (const float* const*)layer_ctx, s->att, batch, token_positions );
+  go_attention_softmax_f32( c, s->att, token_positions, batch );
+  go_attention_2_gemm_f32( c, s->att, (const float* const*)layer_ctx, s->xb, batch, token_positions );
+
+  /* post-attention: model.hh:390-427 */
+  go_matmul_f32( s->xb2, s->xb, w->wo, c->dim, c->dim, batch );
+  go_accum_f32( s->x, s->xb2, c->dim, batch );
+  go_rmsnorm_f32( s->xb, s->x, w->rms_ffn_weight, c->dim, batch );
+  go_matmul_f32( s->hb, s->xb, w->w1, c->dim, c->hidden_dim, batch );
+  go_matmul_f32( s->hb2, s->xb, w->w3, c->dim, c->hidden_dim, batch );
+  go_silu_f32( s->hb, s->hb2, c->hidden_dim, batch );
+  go_matmul_f32( s->xb, s->hb, w->w2, c->hidden_dim, c->dim, batch );
+  go_accum_f32( s->x, s->xb, c->dim, batch );
+
+  free( token_ctx );
+}
+
+/* models/llama2/model.hh:430-442 */
+void go_classify_f32( const go_config* c,
+                      const float* rms_final_weight,
+                      const float* wcls,
+                      float* x,
+                      float* logits,
+                      uint64_t batch )
+{
+  go_rmsnorm_f32( x, x, rms_final_weight, c->dim, batch );
+  go_matmul_f32( logits, x, wcls, c->dim, c->vocab_size, batch );
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * KV addressing: models/llama2/context.hh:61-190
+ * ------------------------------------------------------------------------------------------- */
+uint64_t go_ctx_layer_offset( const go_config* c, const uint8_t* hosted, uint64_t layer )
+{
+  /* Context::set_buffer, context.hh:177-189: hosted layers are packed back to back */
+  if ( !hosted[layer] ) {
+    return UINT64_MAX;
+  }
+  uint64_t before = 0;
+  for ( uint64_t l = 0; l < layer; l++ ) {
+    before += hosted[l] ? 1 : 0;
+  }
+  return before * c->seq_len * c->kv_dim * 2; /* LayerContext::max_size()/sizeof(DType), context.hh:131 */
+}
+
+uint64_t go_ctx_token_offset( const go_config* c, const uint8_t* hosted, uint64_t layer, uint64_t pos )
+{
+  const uint64_t base = go_ctx_layer_offset( c, hosted, layer );
+  return base == UINT64_MAX ? UINT64_MAX : base + pos * c->kv_dim * 2; /* context.hh:116-121 */
+}
+
+uint64_t go_ctx_key_head_offset( const go_config* c, const uint8_t* hosted, uint64_t layer, uint64_t pos, uint64_t h )
+{
+  const uint64_t base = go_ctx_token_offset( c, hosted, layer, pos );
+  return base == UINT64_MAX ? UINT64_MAX : base + h * c->head_size; /* context.hh:82-86 */
+}
+
+uint64_t go_ctx_value_head_offset( const go_config* c, const uint8_t* hosted, uint64_t layer, uint64_t pos, uint64_t h )
+{
+  const uint64_t base = go_ctx_token_offset( c, hosted, layer, pos );
+  return base == UINT64_MAX ? UINT64_MAX : base + c->kv_dim + h * c->head_size; /* context.hh:79-89 */
+}
+
+uint64_t go_ctx_max_size_bytes( const go_config* c, uint64_t n_hosted_layers, uint64_t elem_size )
+{
+  return n_hosted_layers * c->seq_len * c->kv_dim * 2 * elem_size; /* context.hh:131,174 */
+}
+
+/* DynamicContext::prepare, context.hh:221-248 */
+uint64_t go_dynctx_prepare( const go_config* c,
+                            uint64_t elem_size,
+                            uint64_t* allocated,
+                            uint64_t layer,
+                            uint64_t token_pos,
+                            int can_release,
+                            int commit_all,
+                            int* cleared )
+{
+  const uint64_t block = 2ull * 1024 * 1024;
+  if ( cleared ) {
+    *cleared = 0;
+  }
+  if ( can_release ) {
+    for ( uint64_t l = 0; l < c->n_layers; l++ ) {
+      allocated[l] = 0;
+    }
+    if ( cleared ) {
+      *cleared = 1;
+    }
+  }
+  const uint64_t needed = ( token_pos + 1 ) * c->kv_dim * 2 * elem_size;
+  uint64_t committed = 0;
+  if ( commit_all ) {
+    while ( needed > allocated[layer] ) {
+      allocated[layer] += block;
+      committed++;
+    }
+  } else if ( needed > allocated[layer] ) {
+    allocated[layer] += block;
+    committed = 1;
+  }
+  return committed;
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * PreallocatingContextManager: compute/contextman.hh:56-196
+ * free list = FIFO of slot indices (front popped on allocation); map context_id -> slot.
+ * ------------------------------------------------------------------------------------------- */
+struct go_ctxman
+{
+  uint64_t capacity;
+  int32_t* fifo; /* ring buffer of free slots */
+  uint64_t head;
+  uint64_t count;
+  uint32_t* ids;    /* ids[k], slots[k]: allocated pairs (linear search; test sizes are small) */
+  int32_t* slots;
+  uint64_t n_alloc;
+};
+
+go_ctxman* go_ctxman_new( uint64_t max_context_count )
+{
+  go_ctxman* m = (go_ctxman*)calloc( 1, sizeof( go_ctxman ) );
+  const uint64_t cap = max_context_count ? max_context_count : 1;
+  m->capacity = cap; /* ring size; never 0 so the modulo below is defined */
+  m->fifo = (int32_t*)malloc( sizeof( int32_t ) * cap );
+  m->ids = (uint32_t*)malloc( sizeof( uint32_t ) * cap );
+  m->slots = (int32_t*)malloc( sizeof( int32_t ) * cap );
+  for ( uint64_t i = 0; i < max_context_count; i++ ) {
+    m->fifo[i] = (int32_t)i; /* contextman.hh:94-96: emplace_back in construction order */
+  }
+  m->count = max_context_count;
+  return m;
+}
+
+void go_ctxman_delete( go_ctxman* m )
+{
+  if ( m ) {
+    free( m->fifo );
+    free( m->ids );
+    free( m->slots );
+    free( m );
+  }
+}
+
+uint64_t go_ctxman_free( const go_ctxman* m ) { return m->count; }
+uint64_t go_ctxman_allocated( const go_ctxman* m ) { return m->n_alloc; }
+
+static int32_t ctxman_find( const go_ctxman* m, uint32_t id )
+{
+  for ( uint64_t k = 0; k < m->n_alloc; k++ ) {
+    if ( m->ids[k] == id ) {
+      return m->slots[k];
+    }
+  }
+  return -1;
+}
+
+static int32_t ctxman_take_front( go_ctxman* m, uint32_t id )
+{
+  const int32_t slot = m->fifo[m->head];
+  m->head = ( m->head + 1 ) % m->capacity;
+  m->count--;
+  m->ids[m->n_alloc] = id;
+  m->slots[m->n_alloc] = slot;
+  m->n_alloc++;
+  return slot;
+}
+
+int go_ctxman_get_contexts( go_ctxman* m,
+                            const uint8_t* active,
+                            const uint32_t* context_id,
+                            uint64_t start,
+                            uint64_t end,
+                            int32_t* slots_out )
+{
+  /* pass 1 (contextman.hh:138-151): every active row whose id is unmapped counts, duplicates included */
+  uint64_t missing = 0;
+  for ( uint64_t i = start; i < end; i++ ) {
+    if ( active[i] && ctxman_find( m, context_id[i] ) < 0 ) {
+      missing++;
+    }
+  }
+  if ( missing > m->count ) {
+    return 0;
+  }
+  /* pass 2 (contextman.hh:153-168) */
+  for ( uint64_t i = start; i < end; i++ ) {
+    if ( !active[i] ) {
+      slots_out[i - start] = -1;
+      continue;
+    }
+    int32_t slot = ctxman_find( m, context_id[i] );
+    if ( slot < 0 ) {
+      slot = ctxman_take_front( m, context_id[i] );
+    }
+    slots_out[i - start] = slot;
+  }
+  return 1;
+}
+
+int32_t go_ctxman_get_context( go_ctxman* m, uint32_t context_id )
+{
+  const int32_t slot = ctxman_find( m, context_id );
+  if ( slot >= 0 ) {
+    return slot;
+  }
+  if ( m->count == 0 ) {
+    return -1;
+  }
+  return ctxman_take_front( m, context_id );
+}
+
+int go_ctxman_release( go_ctxman* m, uint32_t context_id )
+{
+  for ( uint64_t k = 0; k < m->n_alloc; k++ ) {
+    if ( m->ids[k] == context_id ) {
+      const int32_t slot = m->slots[k];
+      m->ids[k] = m->ids[m->n_alloc - 1];
+      m->slots[k] = m->slots[m->n_alloc - 1];
+      m->n_alloc--;
+      m->fifo[( m->head + m->count ) % m->capacity] = slot; /* push_back */
+      m->count++;
+      return 1;
+    }
+  }
+  return 0;
+}
+
+/* models/common/state.hh:621-631 */
+int go_check_finished( uint32_t token,
+                       uint32_t token_pos,
+                       uint32_t prompt_length,
+                       uint32_t max_completion_length,
+                       uint32_t token_eos,
+                       uint32_t token_eot,
+                       uint64_t seq_len )
+{
+  const int saw_end = max_completion_length == 0 && ( token == token_eos || token == token_eot );
+  const int out_of_seq = token_pos >= seq_len;
+  const int end_of_gen = max_completion_length > 0 && token_pos >= max_completion_length + prompt_length;
+  return saw_end || out_of_seq || end_of_gen;
+}
+
+/* models/common/state.hh:270,612 */
+uint8_t go_encode_temperature( float t ) { return (uint8_t)( t * 255.0f ); }
+float go_decode_temperature( uint8_t t ) { return (float)t / 255.0f; }
+
+int go_num_threads( void )
+{
+#ifdef _OPENMP
+  return omp_get_max_threads();
+#else
+  return 1;
+#endif
+}

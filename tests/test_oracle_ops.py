@@ -1,0 +1,479 @@
+"""Pins the CPU oracle's arithmetic against independent float64 numpy / scipy code, closed forms
+and invariants.  Nothing here touches the GPU.  The reference holds no golden vectors for this
+path, so these checks are what fixes the oracle (each is chosen so that a dropped term, a wrong
+index or a transposed operand fails it)."""
+import numpy as np
+import pytest
+import scipy.special
+
+import oracle as O
+
+TINY = O.Config(dim=32, n_layers=2, n_heads=4, n_kv_heads=2, hidden_dim=48, seq_len=16, vocab_size=64)
+MHA = O.Config(dim=48, n_layers=2, n_heads=6, n_kv_heads=6, hidden_dim=64, seq_len=12, vocab_size=50,
+               attention_rounds=2)
+rng = np.random.default_rng(1234)
+
+
+def f16_round(a):
+    return np.asarray(a, dtype=np.float64).astype(np.float32).astype(np.float16)
+
+
+# ------------------------------------------------------------------ half conversion
+def test_half_to_float_all_patterns():
+    bits = np.arange(65536, dtype=np.uint16)
+    ours = np.empty(65536, dtype=np.float32)
+    O.lib().go_convert_f16_to_f32(ours.ctypes.data, bits.ctypes.data, 65536)
+    ref = bits.view(np.float16).astype(np.float32)
+    assert np.array_equal(ours.view(np.uint32)[~np.isnan(ref)], ref.view(np.uint32)[~np.isnan(ref)])
+    assert np.all(np.isnan(ours[np.isnan(ref)]))
+
+
+def test_float_to_half_rounding():
+    # every half value, its neighbours' midpoints (ties), and random floats over the whole range
+    halves = np.arange(65536, dtype=np.uint16).view(np.float16).astype(np.float32)
+    halves = halves[np.isfinite(halves)]
+    mids = (halves[:-1].astype(np.float64) + halves[1:].astype(np.float64)) / 2
+    rand = rng.standard_normal(200000).astype(np.float32) * np.float32(10.0) ** rng.integers(-9, 6, 200000)
+    edge = np.array([0.0, -0.0, 65504.0, 65519.9, 65520.0, 1e6, -1e6, 2.0 ** -24, 2.0 ** -25,
+                     2.0 ** -25 * 1.0001, 2.0 ** -14, np.inf, -np.inf], dtype=np.float32)
+    x = np.concatenate([halves, mids.astype(np.float32), rand.astype(np.float32), edge])
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    ours = np.empty(x.size, dtype=np.uint16)
+    O.lib().go_convert_f32_to_f16(ours.ctypes.data, x.ctypes.data, x.size)
+    with np.errstate(over="ignore"):
+        ref = x.astype(np.float16).view(np.uint16)
+    assert np.array_equal(ours, ref)
+
+
+# ------------------------------------------------------------------ elementwise
+@pytest.mark.parametrize("dt", [np.float32, np.float16])
+def test_accum(dt):
+    a = rng.standard_normal((3, 37)).astype(dt)
+    b = rng.standard_normal((3, 37)).astype(dt)
+    want = (a.astype(np.float32) + b.astype(np.float32)).astype(dt)
+    O.accum(a, b)
+    assert np.array_equal(a, want)
+
+
+@pytest.mark.parametrize("dt,tol", [(np.float32, 2e-6), (np.float16, 1e-3)])
+def test_silu(dt, tol):
+    x = (rng.standard_normal((2, 53)) * 3).astype(dt)
+    y = rng.standard_normal((2, 53)).astype(dt)
+    x64, y64 = x.astype(np.float64), y.astype(np.float64)
+    want = x64 / (1 + np.exp(-x64)) * y64
+    O.silu(x, y)
+    np.testing.assert_allclose(x.astype(np.float64), want, rtol=tol, atol=tol)
+    # silu(0) * y == 0, silu(x) * 0 == 0
+    z = np.zeros((1, 8), dt)
+    O.silu(z, np.ones((1, 8), dt))
+    assert np.all(z == 0)
+
+
+@pytest.mark.parametrize("dt,tol", [(np.float32, 3e-6), (np.float16, 2e-3)])
+def test_rmsnorm_closed_form(dt, tol):
+    x = rng.standard_normal((4, 96)).astype(dt)
+    w = rng.standard_normal(96).astype(dt)
+    x64, w64 = x.astype(np.float64), w.astype(np.float64)
+    want = w64 * x64 / np.sqrt((x64 ** 2).mean(axis=1, keepdims=True) + 1e-5)
+    got = O.rmsnorm(x, w).astype(np.float64)
+    np.testing.assert_allclose(got, want, rtol=tol, atol=tol)
+
+
+def test_rmsnorm_eps_placement_and_invariants():
+    # all-zero row -> 0 (eps keeps it finite); tiny row scales by 1/sqrt(eps), which an eps added
+    # *inside the square root's argument after the mean* (and only that) reproduces
+    w = np.ones(64, np.float32)
+    z = O.rmsnorm(np.zeros((1, 64), np.float32), w)
+    assert np.all(z == 0) and np.all(np.isfinite(z))
+    tiny = np.full((1, 64), 1e-6, np.float32)
+    got = O.rmsnorm(tiny, w)
+    want = 1e-6 / np.sqrt(1e-12 + 1e-5)
+    np.testing.assert_allclose(got, want, rtol=1e-5)
+    # with unit weights and large inputs the output row has rms 1
+    x = (rng.standard_normal((3, 64)) * 100).astype(np.float32)
+    out = O.rmsnorm(x, w).astype(np.float64)
+    np.testing.assert_allclose(np.sqrt((out ** 2).mean(axis=1)), 1.0, rtol=1e-5)
+    # in-place use (classify_ops normalises x into x)
+    x2 = x.copy()
+    O.rmsnorm(x2, w, out=x2)
+    np.testing.assert_allclose(x2, out, rtol=1e-6)
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float16])
+def test_argmax_first_max_wins(dt):
+    v = rng.standard_normal((5, 300)).astype(dt)
+    v[1, 17] = v[1, 200] = 9.0      # tie: lowest index
+    v[2, :] = 0.0                   # all equal: index 0
+    v[3, 299] = 50.0                # last element
+    got = O.argmax(v)
+    assert got.dtype == np.uint32
+    assert np.array_equal(got, np.argmax(v.astype(np.float64), axis=1))
+    assert got[1] == 17 and got[2] == 0 and got[3] == 299
+
+
+@pytest.mark.parametrize("dt,tol", [(np.float32, 2e-5), (np.float16, 2e-3)])
+def test_matmul(dt, tol):
+    b, s, r = 5, 70, 33
+    x = rng.standard_normal((b, s)).astype(dt)
+    w = (rng.standard_normal((r, s)) * 0.2).astype(dt)
+    want = x.astype(np.float64) @ w.astype(np.float64).T
+    got = O.matmul(x, w)
+    assert got.shape == (b, r)
+    np.testing.assert_allclose(got.astype(np.float64), want, rtol=tol, atol=tol * 5)
+
+
+def test_matmul_layout_one_hot():
+    # a one-hot activation row b with a 1 at column p must return column p of W (as a row):
+    # fails if W were read as (s, r) or the output were written transposed
+    s, r = 7, 5
+    w = np.arange(r * s, dtype=np.float32).reshape(r, s)
+    x = np.zeros((3, s), np.float32)
+    x[0, 2] = x[1, 6] = x[2, 0] = 1
+    got = O.matmul(x, w)
+    assert np.array_equal(got[0], w[:, 2]) and np.array_equal(got[1], w[:, 6]) and np.array_equal(got[2], w[:, 0])
+
+
+def test_gumbel():
+    v = rng.standard_normal((3, 40)).astype(np.float32)
+    u = rng.uniform(0.01, 0.99, (3, 40)).astype(np.float32)
+    t = np.array([0.5, 0.0, 2.0], np.float32)
+    want = v.astype(np.float64).copy()
+    for b in (0, 2):
+        want[b] = want[b] / t[b] - np.log(-np.log(u[b].astype(np.float64)))
+    O.gumbel(v, u, t)
+    np.testing.assert_allclose(v, want, rtol=2e-5, atol=2e-5)   # row 1 (temperature 0) untouched
+
+
+# ------------------------------------------------------------------ KV append
+@pytest.mark.parametrize("dt", [np.float32, np.float16])
+def test_copy_kv_cache_bit_exact(dt):
+    cfg = TINY
+    batch = 4
+    cache = rng.standard_normal((batch, cfg.seq_len, 2 * cfg.kv_dim)).astype(dt)
+    before = cache.copy()
+    kv = rng.standard_normal((batch, 2 * cfg.kv_dim)).astype(dt)
+    kv.view(np.uint16 if dt == np.float16 else np.uint32)[0, 3] = 0x7e01 if dt == np.float16 else 0x7fc00123  # NaN payload
+    pos = [0, 5, 15, 7]
+    rows = [cache[i, pos[i]] for i in range(batch)]
+    rows[2] = None                                   # empty context: skipped
+    O.copy_kv_cache(cfg, rows, kv)
+    U = np.uint16 if dt == np.float16 else np.uint32
+    for i in range(batch):
+        want = before[i].copy()
+        if i != 2:
+            want[pos[i]] = kv[i]
+        assert np.array_equal(cache[i].view(U), want.view(U))
+
+
+# ------------------------------------------------------------------ RoPE
+def rope_ref64(vec, pos, head_size, theta=10000.0):
+    """(…, head_size) float64: complex rotation of interleaved pairs."""
+    k = np.arange(head_size // 2)
+    ang = pos * theta ** (-2.0 * k / head_size)
+    z = (vec[..., 0::2] + 1j * vec[..., 1::2]) * np.exp(1j * ang)
+    out = np.empty_like(vec)
+    out[..., 0::2] = z.real
+    out[..., 1::2] = z.imag
+    return out
+
+
+def test_rope_tables_closed_form():
+    re, im = O.rope_tables(64, 8)
+    k = np.arange(4)
+    ang = np.arange(64)[:, None] * 10000.0 ** (-2.0 * k / 8)[None, :]
+    np.testing.assert_allclose(re, np.cos(ang), atol=2e-5)
+    np.testing.assert_allclose(im, np.sin(ang), atol=2e-5)
+    assert re.shape == (64, 4)
+    assert np.all(re[0] == 1) and np.all(im[0] == 0)
+
+
+@pytest.mark.parametrize("cfg", [TINY, MHA])
+@pytest.mark.parametrize("dt,tol", [(np.float32, 3e-6), (np.float16, 2e-3)])
+def test_apply_rope(cfg, dt, tol):
+    batch = 3
+    hs = cfg.head_size
+    re32, im32 = O.rope_tables(cfg.seq_len, hs)
+    re, im = re32.astype(dt), im32.astype(dt)
+    cache = rng.standard_normal((batch, cfg.seq_len, 2 * cfg.kv_dim)).astype(dt)
+    before = cache.copy()
+    q = rng.standard_normal((batch, cfg.dim)).astype(dt)
+    q0 = q.copy()
+    pos = [0, 5, cfg.seq_len - 1]
+    rows = [cache[i, pos[i]] for i in range(batch)]
+    O.apply_rope(cfg, pos, re, im, q, rows)
+    for i in range(batch):
+        # tables as stored (possibly fp16-rounded) define the rotation; compare against the complex
+        # product with those stored values
+        c = re[pos[i]].astype(np.float64)
+        s = im[pos[i]].astype(np.float64)
+        rot = c + 1j * s
+
+        def rot64(v):
+            v = v.astype(np.float64).reshape(-1, hs)
+            z = (v[:, 0::2] + 1j * v[:, 1::2]) * rot
+            o = np.empty_like(v)
+            o[:, 0::2], o[:, 1::2] = z.real, z.imag
+            return o.reshape(-1)
+
+        np.testing.assert_allclose(q[i].astype(np.float64), rot64(q0[i]), rtol=tol, atol=tol)
+        np.testing.assert_allclose(cache[i, pos[i], : cfg.kv_dim].astype(np.float64),
+                                   rot64(before[i, pos[i], : cfg.kv_dim]), rtol=tol, atol=tol)
+        # V half of the row and every other row: untouched, bit for bit
+        assert np.array_equal(cache[i, pos[i], cfg.kv_dim:], before[i, pos[i], cfg.kv_dim:])
+        mask = np.ones(cfg.seq_len, bool)
+        mask[pos[i]] = False
+        assert np.array_equal(cache[i, mask], before[i, mask])
+    # position 0 is the identity, rotation preserves the norm of every pair
+    assert np.array_equal(q[0], q0[0])
+    if dt == np.float32:
+        n0 = np.hypot(q0[1, 0::2], q0[1, 1::2])
+        n1 = np.hypot(q[1, 0::2], q[1, 1::2])
+        np.testing.assert_allclose(n1, n0, rtol=1e-5)
+
+
+def test_rope_matches_closed_form_angles():
+    # against angles recomputed in float64 from theta (not from the oracle's own tables) and
+    # with interleaved pairing: a half-split pairing would fail this
+    cfg = TINY
+    hs = cfg.head_size
+    re, im = O.rope_tables(cfg.seq_len, hs)
+    q = rng.standard_normal((1, cfg.dim)).astype(np.float32)
+    q0 = q.copy()
+    row = rng.standard_normal(2 * cfg.kv_dim).astype(np.float32)
+    O.apply_rope(cfg, [9], re, im, q, [row])
+    want = rope_ref64(q0[0].astype(np.float64).reshape(-1, hs), 9, hs).reshape(-1)
+    np.testing.assert_allclose(q[0], want, atol=3e-5)
+
+
+def test_rope_skips_empty_context():
+    cfg = TINY
+    re, im = O.rope_tables(cfg.seq_len, cfg.head_size)
+    q = rng.standard_normal((2, cfg.dim)).astype(np.float32)
+    q0 = q.copy()
+    row = rng.standard_normal(2 * cfg.kv_dim).astype(np.float32)
+    O.apply_rope(cfg, [3, 3], re, im, q, [None, row])
+    assert np.array_equal(q[0], q0[0])          # empty context: its query is left alone
+    assert not np.array_equal(q[1], q0[1])
+
+
+# ------------------------------------------------------------------ attention pieces
+def attention_ref64(cfg, q, layers, pos):
+    """float64 scores / probabilities / output with independent einsum code."""
+    batch = len(layers)
+    hs, g = cfg.head_size, cfg.gqa_size
+    scores, probs, out = [], [], np.zeros((batch, cfg.dim))
+    for i in range(batch):
+        n = pos[i] + 1
+        K = layers[i][:n, : cfg.kv_dim].astype(np.float64).reshape(n, cfg.n_kv_heads, hs)
+        V = layers[i][:n, cfg.kv_dim:].astype(np.float64).reshape(n, cfg.n_kv_heads, hs)
+        Q = q[i].astype(np.float64).reshape(cfg.n_kv_heads, g, hs)
+        s = np.einsum("phd,hgd->hgp", K, Q) / np.sqrt(hs)
+        p = scipy.special.softmax(s, axis=-1)
+        o = np.einsum("hgp,phd->hgd", p, V)
+        scores.append(s.reshape(cfg.n_heads, n))
+        probs.append(p.reshape(cfg.n_heads, n))
+        out[i] = o.reshape(-1)
+    return scores, probs, out
+
+
+@pytest.mark.parametrize("cfg", [TINY, MHA])
+@pytest.mark.parametrize("dt,tol", [(np.float32, 1e-5), (np.float16, 4e-3)])
+def test_attention_0_gemm(cfg, dt, tol):
+    batch = 3
+    pos = [0, 5, cfg.seq_len - 1]
+    layers = [rng.standard_normal((cfg.seq_len, 2 * cfg.kv_dim)).astype(dt) for _ in range(batch)]
+    q = rng.standard_normal((batch, cfg.dim)).astype(dt)
+    att = np.full((batch, cfg.n_heads, cfg.seq_len), 77.0, dt)
+    O.attention_0_gemm(cfg, q, layers, att, pos)
+    scores, _, _ = attention_ref64(cfg, q, layers, pos)
+    for i in range(batch):
+        n = pos[i] + 1
+        np.testing.assert_allclose(att[i, :, :n].astype(np.float64), scores[i], rtol=tol, atol=tol)
+        assert np.all(att[i, :, n:] == 77.0)          # beyond pos: never written
+
+
+def test_attention_0_gemm_one_hot_and_head_mapping():
+    # q head (h*gqa+g) = one-hot at dim d  ->  att[h*gqa+g][p] = K[p][h][d] / sqrt(hs)
+    cfg = TINY
+    hs, g = cfg.head_size, cfg.gqa_size
+    layer = rng.standard_normal((cfg.seq_len, 2 * cfg.kv_dim)).astype(np.float32)
+    q = np.zeros((1, cfg.dim), np.float32)
+    picks = {}
+    for head in range(cfg.n_heads):
+        d = (3 * head + 1) % hs
+        q[0, head * hs + d] = 1.0
+        picks[head] = d
+    att = np.zeros((1, cfg.n_heads, cfg.seq_len), np.float32)
+    O.attention_0_gemm(cfg, q, [layer], att, [cfg.seq_len - 1])
+    for head, d in picks.items():
+        kvh = head // g
+        np.testing.assert_allclose(att[0, head], layer[:, kvh * hs + d] / np.sqrt(hs), rtol=1e-6)
+
+
+def test_attention_skips_empty_context():
+    cfg = TINY
+    layer = rng.standard_normal((cfg.seq_len, 2 * cfg.kv_dim)).astype(np.float32)
+    q = rng.standard_normal((2, cfg.dim)).astype(np.float32)
+    att = np.full((2, cfg.n_heads, cfg.seq_len), 5.0, np.float32)
+    O.attention_0_gemm(cfg, q, [None, layer], att, [4, 4])
+    assert np.all(att[0] == 5.0)
+    xb = np.full((2, cfg.dim), 6.0, np.float32)
+    O.attention_2_gemm(cfg, att, [None, layer], xb, [4, 4])
+    assert np.all(xb[0] == 6.0) and not np.any(xb[1] == 6.0)
+
+
+@pytest.mark.parametrize("dt,tol", [(np.float32, 2e-6), (np.float16, 1.5e-3)])
+def test_softmax_row(dt, tol):
+    for n in (1, 2, 17, 300):
+        x = (rng.standard_normal(n) * 4).astype(dt)
+        want = scipy.special.softmax(x.astype(np.float64))
+        O.softmax_row(x)
+        np.testing.assert_allclose(x.astype(np.float64), want, rtol=tol, atol=tol)
+        assert abs(x.astype(np.float64).sum() - 1) < max(tol * n ** 0.5, 1e-5)
+
+
+def test_softmax_shift_invariance_and_extremes():
+    x = (rng.standard_normal(50) * 3).astype(np.float32)
+    a, b = x.copy(), (x + np.float32(100.0)).copy()
+    O.softmax_row(a)
+    O.softmax_row(b)
+    np.testing.assert_allclose(a, b, rtol=2e-4, atol=1e-7)
+    big = np.array([1e4, 0.0, -1e4], np.float32)     # no overflow thanks to the max subtraction
+    O.softmax_row(big)
+    assert np.array_equal(big, np.array([1, 0, 0], np.float32))
+
+
+def test_attention_softmax_only_prefix():
+    cfg = TINY
+    att = (rng.standard_normal((2, cfg.n_heads, cfg.seq_len))).astype(np.float32)
+    before = att.copy()
+    pos = [3, cfg.seq_len - 1]
+    O.attention_softmax(cfg, att, pos)
+    for i in range(2):
+        n = pos[i] + 1
+        np.testing.assert_allclose(att[i, :, :n], scipy.special.softmax(before[i, :, :n].astype(np.float64), axis=-1),
+                                   rtol=1e-5, atol=1e-7)
+        assert np.array_equal(att[i, :, n:], before[i, :, n:])
+
+
+@pytest.mark.parametrize("cfg", [TINY, MHA])
+@pytest.mark.parametrize("dt,tol", [(np.float32, 1e-5), (np.float16, 3e-3)])
+def test_attention_2_gemm(cfg, dt, tol):
+    batch = 3
+    pos = [0, 6, cfg.seq_len - 1]
+    layers = [rng.standard_normal((cfg.seq_len, 2 * cfg.kv_dim)).astype(dt) for _ in range(batch)]
+    att = rng.uniform(0, 1, (batch, cfg.n_heads, cfg.seq_len)).astype(dt)
+    xb = np.zeros((batch, cfg.dim), dt)
+    O.attention_2_gemm(cfg, att, layers, xb, pos)
+    hs, g = cfg.head_size, cfg.gqa_size
+    for i in range(batch):
+        n = pos[i] + 1
+        V = layers[i][:n, cfg.kv_dim:].astype(np.float64).reshape(n, cfg.n_kv_heads, hs)
+        P = att[i, :, :n].astype(np.float64).reshape(cfg.n_kv_heads, g, n)
+        want = np.einsum("hgp,phd->hgd", P, V).reshape(-1)
+        np.testing.assert_allclose(xb[i].astype(np.float64), want, rtol=tol, atol=tol * 4)
+
+
+@pytest.mark.parametrize("cfg", [TINY, MHA])
+def test_attention_ops_end_to_end(cfg):
+    batch = 4
+    pos = [0, 3, 9, cfg.seq_len - 1]
+    re, im = O.rope_tables(cfg.seq_len, cfg.head_size)
+    layers = [rng.standard_normal((cfg.seq_len, 2 * cfg.kv_dim)).astype(np.float32) for _ in range(batch)]
+    q = rng.standard_normal((batch, cfg.dim)).astype(np.float32)
+    # independent float64 pipeline: rotate q and the current K row, then attend
+    q64 = q.astype(np.float64).copy()
+    l64 = [l.astype(np.float64).copy() for l in layers]
+    hs = cfg.head_size
+    for i in range(batch):
+        q64[i] = rope_ref64(q64[i].reshape(-1, hs), pos[i], hs).reshape(-1)
+        l64[i][pos[i], : cfg.kv_dim] = rope_ref64(l64[i][pos[i], : cfg.kv_dim].reshape(-1, hs), pos[i], hs).reshape(-1)
+    _, _, want = attention_ref64(cfg, q64, l64, pos)
+    xb = O.attention_ops(cfg, pos, re, im, q, layers)
+    np.testing.assert_allclose(xb, want, rtol=2e-4, atol=2e-5)
+    # pos 0: softmax over a single key is 1 -> output is exactly V row 0 (per kv head, repeated gqa times)
+    v0 = layers[0][0, cfg.kv_dim:].reshape(cfg.n_kv_heads, 1, hs)
+    assert np.array_equal(xb[0], np.broadcast_to(v0, (cfg.n_kv_heads, cfg.gqa_size, hs)).reshape(-1))
+
+
+def test_attention_uniform_values_pass_through():
+    # if every cached V row is the same vector, the output is that vector whatever the scores are
+    cfg = TINY
+    re, im = O.rope_tables(cfg.seq_len, cfg.head_size)
+    layer = rng.standard_normal((cfg.seq_len, 2 * cfg.kv_dim)).astype(np.float32)
+    v = rng.standard_normal(cfg.kv_dim).astype(np.float32)
+    layer[:, cfg.kv_dim:] = v
+    q = rng.standard_normal((1, cfg.dim)).astype(np.float32)
+    xb = O.attention_ops(cfg, [cfg.seq_len - 1], re, im, q, [layer])
+    want = np.repeat(v.reshape(cfg.n_kv_heads, 1, cfg.head_size), cfg.gqa_size, axis=1).reshape(-1)
+    np.testing.assert_allclose(xb[0], want, rtol=1e-5, atol=1e-6)
+
+
+# ------------------------------------------------------------------ whole layer / classifier
+def layer_ref64(cfg, w, x, layers, pos):
+    """Independent float64 transformer block (pre-norm Llama2), token at positions `pos`."""
+    hs = cfg.head_size
+    W = {k: v.astype(np.float64) for k, v in w.items()}
+    x = x.astype(np.float64).copy()
+
+    def rms(v, g):
+        return g * v / np.sqrt((v ** 2).mean(axis=-1, keepdims=True) + 1e-5)
+
+    h = rms(x, W["rms_att_weight"])
+    q = h @ W["wq"].T
+    kv = h @ W["wkv"].T
+    l64 = [l.astype(np.float64).copy() for l in layers]
+    for i in range(len(layers)):
+        l64[i][pos[i]] = kv[i]
+        l64[i][pos[i], : cfg.kv_dim] = rope_ref64(l64[i][pos[i], : cfg.kv_dim].reshape(-1, hs), pos[i], hs).reshape(-1)
+        q[i] = rope_ref64(q[i].reshape(-1, hs), pos[i], hs).reshape(-1)
+    _, _, att_out = attention_ref64(cfg, q, l64, pos)
+    x = x + att_out @ W["wo"].T
+    h = rms(x, W["rms_ffn_weight"])
+    a = h @ W["w1"].T
+    b = h @ W["w3"].T
+    x = x + ((a / (1 + np.exp(-a))) * b) @ W["w2"].T
+    return x, l64
+
+
+def make_layer_weights(cfg, scale=0.2, dtype=np.float32):
+    r = np.random.default_rng(7)
+    return {
+        "rms_att_weight": (1 + 0.1 * r.standard_normal(cfg.dim)).astype(dtype),
+        "wq": (scale * r.standard_normal((cfg.dim, cfg.dim))).astype(dtype),
+        "wkv": (scale * r.standard_normal((2 * cfg.kv_dim, cfg.dim))).astype(dtype),
+        "wo": (scale * r.standard_normal((cfg.dim, cfg.dim))).astype(dtype),
+        "rms_ffn_weight": (1 + 0.1 * r.standard_normal(cfg.dim)).astype(dtype),
+        "w1": (scale * r.standard_normal((cfg.hidden_dim, cfg.dim))).astype(dtype),
+        "w2": (scale * r.standard_normal((cfg.dim, cfg.hidden_dim))).astype(dtype),
+        "w3": (scale * r.standard_normal((cfg.hidden_dim, cfg.dim))).astype(dtype),
+    }
+
+
+@pytest.mark.parametrize("cfg", [TINY, MHA])
+def test_layer_forward(cfg):
+    batch = 3
+    pos = [0, 4, cfg.seq_len - 1]
+    w = make_layer_weights(cfg)
+    re, im = O.rope_tables(cfg.seq_len, cfg.head_size)
+    layers = [rng.standard_normal((cfg.seq_len, 2 * cfg.kv_dim)).astype(np.float32) for _ in range(batch)]
+    x = rng.standard_normal((batch, cfg.dim)).astype(np.float32)
+    want_x, want_layers = layer_ref64(cfg, w, x, layers, pos)
+    O.layer_forward(cfg, w, re, im, x, layers, pos)
+    np.testing.assert_allclose(x, want_x, rtol=3e-4, atol=3e-4)
+    for i in range(batch):   # the cache now holds the appended (rotated-K | raw-V) row
+        np.testing.assert_allclose(layers[i], want_layers[i], rtol=2e-4, atol=2e-5)
+
+
+def test_classify():
+    cfg = TINY
+    r = np.random.default_rng(3)
+    x = r.standard_normal((2, cfg.dim)).astype(np.float32)
+    g = (1 + 0.1 * r.standard_normal(cfg.dim)).astype(np.float32)
+    wcls = (0.2 * r.standard_normal((cfg.vocab_size, cfg.dim))).astype(np.float32)
+    x64 = x.astype(np.float64)
+    h = g * x64 / np.sqrt((x64 ** 2).mean(axis=-1, keepdims=True) + 1e-5)
+    want = h @ wcls.astype(np.float64).T
+    logits = O.classify(cfg, g, wcls, x)
+    np.testing.assert_allclose(logits, want, rtol=2e-5, atol=2e-5)
+    np.testing.assert_allclose(x, h, rtol=2e-5, atol=2e-6)   # x is normalised in place
