@@ -1,0 +1,63 @@
+"""Builds libglint_hip.so (the gfx950 kernels and their C-ABI) in-tree with hipcc.
+
+Usage: ``python -m glinthawk_amd.build``.  hipcc cross-compiles for gfx950 without a GPU.
+"""
+from __future__ import annotations
+
+import glob
+import os
+import subprocess
+import sys
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(PKG)
+CSRC = os.path.join(PKG, "csrc")
+HOST = os.path.join(PKG, "host")
+LIB_DIR = os.path.join(PKG, "lib")
+LIB = os.path.join(LIB_DIR, "libglint_hip.so")
+HOST_LIB = os.path.join(LIB_DIR, "libglint_host.so")
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+
+# packed fp32 instructions are switched off for every device compile of this library
+DEVICE_FLAGS = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+COMMON_FLAGS = ["-O3", "-fPIC", "-Wall", "-Wno-unused-function", "-I" + os.path.join(ROOT, "include"), "-I" + CSRC]
+
+
+def _run(cmd: list[str]) -> None:
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in proc.stdout.splitlines()
+                    if "is not a recognized feature for this target" not in l)
+    if proc.returncode != 0:
+        sys.stderr.write(out + "\n")
+        raise RuntimeError("build failed: " + " ".join(cmd))
+    if out.strip():
+        print(out)
+
+
+def build_kernels() -> str:
+    os.makedirs(LIB_DIR, exist_ok=True)
+    sources = sorted(glob.glob(os.path.join(CSRC, "*.hip")))
+    _run([HIPCC, *DEVICE_FLAGS, *COMMON_FLAGS, "-std=c++17", "-shared", "-o", LIB, *sources])
+    return LIB
+
+
+def build_host() -> str | None:
+    """The C++20 host layer (the reference-shaped classes) plus its C test hooks."""
+    sources = sorted(glob.glob(os.path.join(HOST, "*.cc")))
+    if not sources:
+        return None
+    os.makedirs(LIB_DIR, exist_ok=True)
+    _run([HIPCC, *COMMON_FLAGS, "-std=c++20", "-x", "c++", "-I" + HOST, "-shared", "-o", HOST_LIB, *sources,
+          "-L" + LIB_DIR, "-lglint_hip", "-Wl,-rpath,$ORIGIN", "-pthread"])
+    return HOST_LIB
+
+
+def build_all() -> None:
+    build_kernels()
+    build_host()
+
+
+if __name__ == "__main__":
+    build_all()
+    print("built", LIB)

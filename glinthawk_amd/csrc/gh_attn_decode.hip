@@ -1,0 +1,864 @@
+// Fused decode attention for one layer of a batch of contexts: scores, softmax and the weighted
+// sum over the cached rows in one pass, split over the key range (split-K) with an online
+// softmax; a second small kernel merges the per-split partials.  Replaces the reference's
+// attention_0_gemm + attention_softmax + attention_2_gemm sequence (models/llama2/model.hh:354-387)
+// and needs no (batch, n_heads, seq_len) score buffer.
+//
+// Cache layout (fixed by the reference, models/llama2/context.hh:61-133): a layer of a context is
+// seq_len rows of [K(kv_dim) | V(kv_dim)], token-major.  For kv head h the K head is head_size
+// contiguous elements at row + h*head_size, the V head at row + kv_dim + h*head_size.
+//
+// Three kernels produce the same partial format:
+//   generic  any head_size <= 256, any gqa, f16/f32 storage; one wave per (context, query head, split)
+//   valu     f16, head_size 128: one wave per (context, kv head, split); 16 lanes share a token's
+//            256-byte head row (one 16-byte load per lane), dot products with v_dot2_f32_f16,
+//            16-lane DPP reductions, four independent online-softmax streams per wave
+//   mfma     f16, head_size 128, 2 <= gqa <= 16: same wave decomposition, but the gqa query heads
+//            are a 16-wide MFMA tile: S^T = K Q^T with v_mfma_f32_16x16x32_f16 (K staged through LDS
+//            into operand order), O += P V with v_mfma_f32_16x16x16_f16 (V transposed in registers)
+//
+// Scores are kept in the log2 domain: s2 = (q . k) * scale * log2(e), weights are exp2(s2 - m).
+// Partial format per (context, query head, split): out[head_size] floats (un-normalised), then m and l.
+#include "gh_common.h"
+
+#include <algorithm>
+
+namespace gh {
+namespace {
+
+constexpr float LOG2E = 1.4426950408889634f;
+constexpr int HS = 128; // head size of the fast kernels
+
+uint32_t g_chunk_override = 0;
+
+typedef _Float16 f16x4 __attribute__( ( ext_vector_type( 4 ) ) );
+typedef _Float16 f16x8 __attribute__( ( ext_vector_type( 8 ) ) );
+typedef _Float16 f16x2 __attribute__( ( ext_vector_type( 2 ) ) );
+typedef float f32x4 __attribute__( ( ext_vector_type( 4 ) ) );
+
+struct Partials
+{
+  float* out; // [batch][n_heads][max_splits][head_size]
+  float* ml;  // [batch][n_heads][max_splits][2]
+};
+
+__device__ __forceinline__ float fast_exp2( float x ) { return __builtin_amdgcn_exp2f( x ); }
+
+// =================================================================================================
+// generic kernel
+// =================================================================================================
+template<typename T>
+__global__ __launch_bounds__( 64 ) void attn_decode_generic_kernel( const T* __restrict__ q,
+                                                                    const T* const* __restrict__ layer_rows,
+                                                                    const uint32_t* __restrict__ pos,
+                                                                    Partials part,
+                                                                    T* __restrict__ xb,
+                                                                    uint32_t n_kv_heads,
+                                                                    uint32_t gqa,
+                                                                    uint32_t head_size,
+                                                                    uint32_t chunk,
+                                                                    uint32_t max_splits,
+                                                                    float scale_log2e )
+{
+  const uint32_t head = blockIdx.x;
+  const uint32_t split = blockIdx.y;
+  const uint32_t ctx = blockIdx.z;
+  const T* base = layer_rows[ctx];
+  if ( base == nullptr ) {
+    return;
+  }
+  const uint32_t n_tok = pos[ctx] + 1;
+  const uint32_t t_begin = split * chunk;
+  if ( t_begin >= n_tok ) {
+    return;
+  }
+  const uint32_t t_end = min( n_tok, t_begin + chunk );
+  const uint32_t n_heads = n_kv_heads * gqa;
+  const uint32_t h = head / gqa;
+  const uint32_t lane = threadIdx.x;
+  const uint64_t row_elems = 2ull * n_kv_heads * head_size;
+
+  float qd[4], acc[4];
+  const T* qh = q + ( (uint64_t)ctx * n_heads + head ) * head_size;
+#pragma unroll
+  for ( int k = 0; k < 4; k++ ) {
+    const uint32_t d = lane + 64 * k;
+    qd[k] = d < head_size ? to_f32( qh[d] ) : 0.0f;
+    acc[k] = 0.0f;
+  }
+  float m = -INFINITY, l = 0.0f;
+  const T* kbase = base + (uint64_t)h * head_size;
+  const T* vbase = kbase + (uint64_t)n_kv_heads * head_size;
+
+  for ( uint32_t t = t_begin; t < t_end; t++ ) {
+    const T* kr = kbase + (uint64_t)t * row_elems;
+    const T* vr = vbase + (uint64_t)t * row_elems;
+    float partial = 0.0f;
+    float vd[4];
+#pragma unroll
+    for ( int k = 0; k < 4; k++ ) {
+      const uint32_t d = lane + 64 * k;
+      if ( d < head_size ) {
+        partial += to_f32( kr[d] ) * qd[k];
+        vd[k] = to_f32( vr[d] );
+      } else {
+        vd[k] = 0.0f;
+      }
+    }
+    const float s = wave_sum( partial ) * scale_log2e;
+    const float m_new = fmaxf( m, s );
+    const float alpha = fast_exp2( m - m_new );
+    const float p = fast_exp2( s - m_new );
+    l = l * alpha + p;
+#pragma unroll
+    for ( int k = 0; k < 4; k++ ) {
+      acc[k] = acc[k] * alpha + p * vd[k];
+    }
+    m = m_new;
+  }
+
+  if ( max_splits == 1 ) {
+    const float inv = 1.0f / l;
+    T* o = xb + ( (uint64_t)ctx * n_heads + head ) * head_size;
+#pragma unroll
+    for ( int k = 0; k < 4; k++ ) {
+      const uint32_t d = lane + 64 * k;
+      if ( d < head_size ) {
+        o[d] = from_f32<T>( acc[k] * inv );
+      }
+    }
+  } else {
+    const uint64_t slot = ( (uint64_t)ctx * n_heads + head ) * max_splits + split;
+    float* o = part.out + slot * head_size;
+#pragma unroll
+    for ( int k = 0; k < 4; k++ ) {
+      const uint32_t d = lane + 64 * k;
+      if ( d < head_size ) {
+        o[d] = acc[k];
+      }
+    }
+    if ( lane == 0 ) {
+      part.ml[slot * 2] = m;
+      part.ml[slot * 2 + 1] = l;
+    }
+  }
+}
+
+// =================================================================================================
+// merge of the split partials: block <-> (query head, context), thread <-> output dim
+// =================================================================================================
+template<typename T>
+__global__ __launch_bounds__( 256 ) void attn_merge_kernel( Partials part,
+                                                            const void* const* __restrict__ layer_rows,
+                                                            const uint32_t* __restrict__ pos,
+                                                            T* __restrict__ xb,
+                                                            uint32_t n_heads,
+                                                            uint32_t head_size,
+                                                            uint32_t chunk,
+                                                            uint32_t max_splits )
+{
+  const uint32_t head = blockIdx.x;
+  const uint32_t ctx = blockIdx.y;
+  if ( layer_rows[ctx] == nullptr ) {
+    return;
+  }
+  const uint32_t n_splits = ( pos[ctx] + chunk ) / chunk; // ceil((pos + 1) / chunk)
+  const uint64_t slot0 = ( (uint64_t)ctx * n_heads + head ) * max_splits;
+  float m = -INFINITY;
+  for ( uint32_t s = 0; s < n_splits; s++ ) {
+    m = fmaxf( m, part.ml[( slot0 + s ) * 2] );
+  }
+  float l = 0.0f;
+  for ( uint32_t s = 0; s < n_splits; s++ ) {
+    l += part.ml[( slot0 + s ) * 2 + 1] * fast_exp2( part.ml[( slot0 + s ) * 2] - m );
+  }
+  const float inv = 1.0f / l;
+  for ( uint32_t d = threadIdx.x; d < head_size; d += blockDim.x ) {
+    float acc = 0.0f;
+    for ( uint32_t s = 0; s < n_splits; s++ ) {
+      acc += part.out[( slot0 + s ) * head_size + d] * fast_exp2( part.ml[( slot0 + s ) * 2] - m );
+    }
+    xb[( (uint64_t)ctx * n_heads + head ) * head_size + d] = from_f32<T>( acc * inv );
+  }
+}
+
+// =================================================================================================
+// shared pieces of the two fast kernels
+// =================================================================================================
+struct WaveJob
+{
+  const __half* base; // layer rows of the context
+  uint32_t ctx, h, split, t_begin, t_end;
+  bool valid;
+};
+
+// block -> (group of 4 kv heads, split, context); wave -> kv head.  Adjacent blocks cover adjacent
+// head groups of the same token range so that concurrently running blocks read whole cache rows.
+__device__ __forceinline__ WaveJob wave_job( const __half* const* layer_rows,
+                                             const uint32_t* pos,
+                                             uint32_t n_kv_heads,
+                                             uint32_t chunk,
+                                             uint32_t max_splits )
+{
+  WaveJob j;
+  const uint32_t wave = threadIdx.x >> 6;
+  const uint32_t n_hg = ( n_kv_heads + 3 ) / 4;
+  uint32_t bid = blockIdx.x;
+  const uint32_t hg = bid % n_hg;
+  bid /= n_hg;
+  j.split = bid % max_splits;
+  j.ctx = bid / max_splits;
+  j.h = hg * 4 + wave;
+  j.base = layer_rows[j.ctx];
+  const uint32_t n_tok = pos[j.ctx] + 1;
+  j.t_begin = j.split * chunk;
+  j.t_end = min( n_tok, j.t_begin + chunk );
+  j.valid = j.h < n_kv_heads && j.base != nullptr && j.t_begin < n_tok;
+  return j;
+}
+
+__device__ __forceinline__ float dpp_quad_xor1( float v )
+{
+  return __builtin_bit_cast( float, __builtin_amdgcn_update_dpp( 0, __builtin_bit_cast( int, v ), 0xB1, 0xF, 0xF, true ) );
+}
+__device__ __forceinline__ float dpp_quad_xor2( float v )
+{
+  return __builtin_bit_cast( float, __builtin_amdgcn_update_dpp( 0, __builtin_bit_cast( int, v ), 0x4E, 0xF, 0xF, true ) );
+}
+__device__ __forceinline__ float dpp_half_mirror( float v )
+{
+  return __builtin_bit_cast( float, __builtin_amdgcn_update_dpp( 0, __builtin_bit_cast( int, v ), 0x141, 0xF, 0xF, true ) );
+}
+__device__ __forceinline__ float dpp_row_mirror( float v )
+{
+  return __builtin_bit_cast( float, __builtin_amdgcn_update_dpp( 0, __builtin_bit_cast( int, v ), 0x140, 0xF, 0xF, true ) );
+}
+// sum over the 16 lanes of a DPP row; every lane of the row gets the total
+__device__ __forceinline__ float row16_sum( float v )
+{
+  v += dpp_quad_xor1( v );
+  v += dpp_quad_xor2( v );
+  v += dpp_half_mirror( v );
+  v += dpp_row_mirror( v );
+  return v;
+}
+
+__device__ __forceinline__ uint4 load16( const __half* p ) { return *reinterpret_cast<const uint4*>( p ); }
+
+__device__ __forceinline__ float dot8( const uint4& a, const uint4& b, float acc )
+{
+  acc = __builtin_amdgcn_fdot2( __builtin_bit_cast( f16x2, a.x ), __builtin_bit_cast( f16x2, b.x ), acc, false );
+  acc = __builtin_amdgcn_fdot2( __builtin_bit_cast( f16x2, a.y ), __builtin_bit_cast( f16x2, b.y ), acc, false );
+  acc = __builtin_amdgcn_fdot2( __builtin_bit_cast( f16x2, a.z ), __builtin_bit_cast( f16x2, b.z ), acc, false );
+  acc = __builtin_amdgcn_fdot2( __builtin_bit_cast( f16x2, a.w ), __builtin_bit_cast( f16x2, b.w ), acc, false );
+  return acc;
+}
+
+__device__ __forceinline__ void unpack8( const uint4& v, float out[8] )
+{
+  const uint32_t w[4] = { v.x, v.y, v.z, v.w };
+#pragma unroll
+  for ( int k = 0; k < 4; k++ ) {
+    const f16x2 h2 = __builtin_bit_cast( f16x2, w[k] );
+    out[2 * k] = (float)h2.x;
+    out[2 * k + 1] = (float)h2.y;
+  }
+}
+
+// =================================================================================================
+// valu kernel: lane = (r = lane / 16: token within a group of 4, c = lane % 16: 16-byte chunk of the head row)
+// =================================================================================================
+template<int G>
+__global__ __launch_bounds__( 256 ) void attn_decode_valu_kernel( const __half* __restrict__ q,
+                                                                  const __half* const* __restrict__ layer_rows,
+                                                                  const uint32_t* __restrict__ pos,
+                                                                  Partials part,
+                                                                  __half* __restrict__ xb,
+                                                                  uint32_t n_kv_heads,
+                                                                  uint32_t chunk,
+                                                                  uint32_t max_splits,
+                                                                  float scale_log2e )
+{
+  const WaveJob job = wave_job( layer_rows, pos, n_kv_heads, chunk, max_splits );
+  if ( !job.valid ) {
+    return; // wave-uniform; the kernel has no block-level barrier
+  }
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t c = lane & 15;
+  const uint32_t r = lane >> 4;
+  const uint32_t n_heads = n_kv_heads * G;
+  const uint64_t row_elems = 2ull * n_kv_heads * HS;
+  const uint32_t v_off = n_kv_heads * HS;
+
+  uint4 qr[G];
+  {
+    const __half* qp = q + ( (uint64_t)job.ctx * n_heads + (uint64_t)job.h * G ) * HS + 8 * c;
+#pragma unroll
+    for ( int g = 0; g < G; g++ ) {
+      qr[g] = load16( qp + g * HS );
+    }
+  }
+
+  float m[G], l[G], acc[G][8];
+#pragma unroll
+  for ( int g = 0; g < G; g++ ) {
+    m[g] = -INFINITY;
+    l[g] = 0.0f;
+#pragma unroll
+    for ( int e = 0; e < 8; e++ ) {
+      acc[g][e] = 0.0f;
+    }
+  }
+
+  const __half* kp = job.base + (uint64_t)job.h * HS + 8 * c;
+  const uint4 zero4 = make_uint4( 0, 0, 0, 0 );
+
+  uint4 kn[4], vn[4]; // prefetched block
+#pragma unroll
+  for ( int j = 0; j < 4; j++ ) {
+    const uint32_t tok = job.t_begin + 4 * j + r;
+    const bool ok = tok < job.t_end;
+    const __half* row = kp + (uint64_t)tok * row_elems;
+    kn[j] = ok ? load16( row ) : zero4;
+    vn[j] = ok ? load16( row + v_off ) : zero4;
+  }
+
+  for ( uint32_t t0 = job.t_begin; t0 < job.t_end; t0 += 16 ) {
+    uint4 kc[4], vc[4];
+#pragma unroll
+    for ( int j = 0; j < 4; j++ ) {
+      kc[j] = kn[j];
+      vc[j] = vn[j];
+    }
+    // prefetch the next 16 tokens while this block is processed
+#pragma unroll
+    for ( int j = 0; j < 4; j++ ) {
+      const uint32_t tok = t0 + 16 + 4 * j + r;
+      const bool ok = tok < job.t_end;
+      const __half* row = kp + (uint64_t)tok * row_elems;
+      kn[j] = ok ? load16( row ) : zero4;
+      vn[j] = ok ? load16( row + v_off ) : zero4;
+    }
+
+    float s[4][G];
+#pragma unroll
+    for ( int j = 0; j < 4; j++ ) {
+      const bool ok = t0 + 4 * j + r < job.t_end;
+#pragma unroll
+      for ( int g = 0; g < G; g++ ) {
+        const float d = row16_sum( dot8( kc[j], qr[g], 0.0f ) );
+        s[j][g] = ok ? d * scale_log2e : -INFINITY;
+      }
+    }
+
+#pragma unroll
+    for ( int g = 0; g < G; g++ ) {
+      float m_new = fmaxf( fmaxf( s[0][g], s[1][g] ), fmaxf( s[2][g], s[3][g] ) );
+      m_new = fmaxf( m_new, m[g] );
+      const float m_safe = m_new == -INFINITY ? 0.0f : m_new; // a row that has seen no token yet
+      const float alpha = fast_exp2( m[g] - m_safe );
+      float p[4];
+#pragma unroll
+      for ( int j = 0; j < 4; j++ ) {
+        p[j] = fast_exp2( s[j][g] - m_safe );
+      }
+      l[g] = l[g] * alpha + ( p[0] + p[1] ) + ( p[2] + p[3] );
+      m[g] = m_new;
+#pragma unroll
+      for ( int e = 0; e < 8; e++ ) {
+        acc[g][e] *= alpha;
+      }
+#pragma unroll
+      for ( int j = 0; j < 4; j++ ) {
+        float v[8];
+        unpack8( vc[j], v );
+#pragma unroll
+        for ( int e = 0; e < 8; e++ ) {
+          acc[g][e] += p[j] * v[e];
+        }
+      }
+    }
+  }
+
+  // merge the four token streams (lane rows) of the wave
+#pragma unroll
+  for ( int g = 0; g < G; g++ ) {
+    float mm = fmaxf( m[g], __shfl_xor( m[g], 16, WAVE ) );
+    mm = fmaxf( mm, __shfl_xor( mm, 32, WAVE ) );
+    const float f = m[g] == -INFINITY ? 0.0f : fast_exp2( m[g] - mm );
+    float ll = l[g] * f;
+    ll += __shfl_xor( ll, 16, WAVE );
+    ll += __shfl_xor( ll, 32, WAVE );
+#pragma unroll
+    for ( int e = 0; e < 8; e++ ) {
+      float a = acc[g][e] * f;
+      a += __shfl_xor( a, 16, WAVE );
+      a += __shfl_xor( a, 32, WAVE );
+      acc[g][e] = a;
+    }
+    m[g] = mm;
+    l[g] = ll;
+  }
+
+  if ( r == 0 ) {
+#pragma unroll
+    for ( int g = 0; g < G; g++ ) {
+      const uint64_t head = (uint64_t)job.ctx * n_heads + (uint64_t)job.h * G + g;
+      if ( max_splits == 1 ) {
+        const float inv = 1.0f / l[g];
+        union
+        {
+          uint4 raw;
+          __half h[8];
+        } o;
+#pragma unroll
+        for ( int e = 0; e < 8; e++ ) {
+          o.h[e] = __float2half_rn( acc[g][e] * inv );
+        }
+        *reinterpret_cast<uint4*>( xb + head * HS + 8 * c ) = o.raw;
+      } else {
+        const uint64_t slot = head * max_splits + job.split;
+        float4* o = reinterpret_cast<float4*>( part.out + slot * HS + 8 * c );
+        o[0] = make_float4( acc[g][0], acc[g][1], acc[g][2], acc[g][3] );
+        o[1] = make_float4( acc[g][4], acc[g][5], acc[g][6], acc[g][7] );
+        if ( c == 0 ) {
+          part.ml[slot * 2] = m[g];
+          part.ml[slot * 2 + 1] = l[g];
+        }
+      }
+    }
+  }
+}
+
+// =================================================================================================
+// mfma kernel: a tile is 16 tokens x 16 (padded) query heads.
+//   lane = (g4 = lane / 16, c = lane % 16)
+//   global loads: lane (g4, c) reads the 16-byte chunk c of tokens 4*g4 + i, i = 0..3, for K and V
+//   K goes through a wave-private LDS tile (XOR-swizzled 16-byte chunks) and comes back as
+//     A[m = token c][k-group g4] fragments of v_mfma_f32_16x16x32_f16; B = Q^T fragments in registers
+//   S^T[token 4*g4+i][head c] lands in lane (g4, c) -- exactly the A-operand order of
+//     v_mfma_f32_16x16x16_f16 for P (m = head c, k = 4*g4+i)
+//   V fragments B[k = token 4*g4+i][n = c] for output column (dim 8*c + nn) are byte-permuted out of
+//     the four 16-byte registers; acc[nn][i] = O[head 4*g4+i][dim 8*c+nn]
+// =================================================================================================
+template<int G>
+__global__ __launch_bounds__( 256 ) void attn_decode_mfma_kernel( const __half* __restrict__ q,
+                                                                  const __half* const* __restrict__ layer_rows,
+                                                                  const uint32_t* __restrict__ pos,
+                                                                  Partials part,
+                                                                  __half* __restrict__ xb,
+                                                                  uint32_t n_kv_heads,
+                                                                  uint32_t chunk,
+                                                                  uint32_t max_splits,
+                                                                  float scale_log2e )
+{
+  __shared__ uint4 s_k[4][16 * 16]; // per wave: 16 tokens x 16 chunks of 16 bytes
+
+  const WaveJob job = wave_job( layer_rows, pos, n_kv_heads, chunk, max_splits );
+  if ( !job.valid ) {
+    return; // wave-uniform; only wave-private LDS is used, no block barrier
+  }
+  const uint32_t wave = threadIdx.x >> 6;
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t c = lane & 15;
+  const uint32_t g4 = lane >> 4;
+  const uint32_t n_heads = n_kv_heads * G;
+  const uint64_t row_elems = 2ull * n_kv_heads * HS;
+  const uint32_t v_off = n_kv_heads * HS;
+  uint4* tile = s_k[wave];
+
+  // B fragments of Q^T: head c (zero for the padding heads), dims of chunk 4*kk + g4
+  f16x8 qb[4];
+  {
+    const __half* qp = q + ( (uint64_t)job.ctx * n_heads + (uint64_t)job.h * G + ( c < G ? c : 0 ) ) * HS;
+#pragma unroll
+    for ( int kk = 0; kk < 4; kk++ ) {
+      uint4 v = load16( qp + 8 * ( 4 * kk + g4 ) );
+      if ( c >= G ) {
+        v = make_uint4( 0, 0, 0, 0 );
+      }
+      qb[kk] = __builtin_bit_cast( f16x8, v );
+    }
+  }
+
+  f32x4 acc[8];
+#pragma unroll
+  for ( int nn = 0; nn < 8; nn++ ) {
+    acc[nn] = f32x4 { 0.0f, 0.0f, 0.0f, 0.0f };
+  }
+  float m = -INFINITY; // running max of head c (log2 domain), identical in the 4 lanes that share c
+  float l = 0.0f;      // this lane's share of the running sum of head c
+
+  const __half* kp = job.base + (uint64_t)job.h * HS + 8 * c;
+  const uint4 zero4 = make_uint4( 0, 0, 0, 0 );
+
+  uint4 kn[4], vn[4];
+#pragma unroll
+  for ( int i = 0; i < 4; i++ ) {
+    const uint32_t tok = job.t_begin + 4 * g4 + i;
+    const bool ok = tok < job.t_end;
+    const __half* row = kp + (uint64_t)tok * row_elems;
+    kn[i] = ok ? load16( row ) : zero4;
+    vn[i] = ok ? load16( row + v_off ) : zero4;
+  }
+
+  for ( uint32_t t0 = job.t_begin; t0 < job.t_end; t0 += 16 ) {
+    uint4 vc[4];
+    // K tile into LDS: token 4*g4+i, chunk c, stored at chunk position c ^ token
+#pragma unroll
+    for ( int i = 0; i < 4; i++ ) {
+      const uint32_t tl = 4 * g4 + i;
+      tile[tl * 16 + ( c ^ tl )] = kn[i];
+      vc[i] = vn[i];
+    }
+    // prefetch the next tile
+#pragma unroll
+    for ( int i = 0; i < 4; i++ ) {
+      const uint32_t tok = t0 + 16 + 4 * g4 + i;
+      const bool ok = tok < job.t_end;
+      const __half* row = kp + (uint64_t)tok * row_elems;
+      kn[i] = ok ? load16( row ) : zero4;
+      vn[i] = ok ? load16( row + v_off ) : zero4;
+    }
+    __builtin_amdgcn_fence( __ATOMIC_RELEASE, "wavefront" );
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence( __ATOMIC_ACQUIRE, "wavefront" );
+
+    // S^T = K Q^T : A fragment = token c, chunk 4*kk + g4
+    f32x4 st = f32x4 { 0.0f, 0.0f, 0.0f, 0.0f };
+#pragma unroll
+    for ( int kk = 0; kk < 4; kk++ ) {
+      const uint4 kf = tile[c * 16 + ( ( 4 * kk + g4 ) ^ c )];
+      st = __builtin_amdgcn_mfma_f32_16x16x32_f16( __builtin_bit_cast( f16x8, kf ), qb[kk], st, 0, 0, 0 );
+    }
+    __builtin_amdgcn_fence( __ATOMIC_RELEASE, "wavefront" );
+    __builtin_amdgcn_wave_barrier(); // the tile is rewritten at the top of the next iteration
+
+    // st[i] = score of token t0 + 4*g4 + i for head c
+    float s[4];
+    float mt = -INFINITY;
+#pragma unroll
+    for ( int i = 0; i < 4; i++ ) {
+      const bool ok = t0 + 4 * g4 + i < job.t_end;
+      s[i] = ok ? st[i] * scale_log2e : -INFINITY;
+      mt = fmaxf( mt, s[i] );
+    }
+    mt = fmaxf( mt, __shfl_xor( mt, 16, WAVE ) );
+    mt = fmaxf( mt, __shfl_xor( mt, 32, WAVE ) );
+    const float m_new = fmaxf( m, mt ); // finite: the first token of every tile is inside the range
+    const float alpha = fast_exp2( m - m_new );
+    float p[4];
+#pragma unroll
+    for ( int i = 0; i < 4; i++ ) {
+      p[i] = fast_exp2( s[i] - m_new );
+    }
+    l = l * alpha + ( p[0] + p[1] ) + ( p[2] + p[3] );
+    m = m_new;
+
+    // rescale the accumulators when some head's maximum moved: acc[.][i] belongs to head 4*g4 + i
+    if ( __builtin_amdgcn_ballot_w64( alpha != 1.0f ) != 0 ) {
+#pragma unroll
+      for ( int i = 0; i < 4; i++ ) {
+        const float a = __shfl( alpha, (int)( 4 * g4 + i ), WAVE );
+#pragma unroll
+        for ( int nn = 0; nn < 8; nn++ ) {
+          acc[nn][i] *= a;
+        }
+      }
+    }
+
+    // P as A fragment: head c, tokens 4*g4 .. 4*g4+3
+    const f16x4 pa = f16x4 { (_Float16)p[0], (_Float16)p[1], (_Float16)p[2], (_Float16)p[3] };
+
+    // V fragments: for output column nn = 2*w + hl take half `hl` of word w of the four token registers
+    const uint32_t vw[4][4] = { { vc[0].x, vc[0].y, vc[0].z, vc[0].w },
+                                { vc[1].x, vc[1].y, vc[1].z, vc[1].w },
+                                { vc[2].x, vc[2].y, vc[2].z, vc[2].w },
+                                { vc[3].x, vc[3].y, vc[3].z, vc[3].w } };
+#pragma unroll
+    for ( int w = 0; w < 4; w++ ) {
+      // low halves: bytes 0,1 of the first source then bytes 0,1 of the second
+      const uint2 lo = make_uint2( __builtin_amdgcn_perm( vw[1][w], vw[0][w], 0x05040100u ),
+                                   __builtin_amdgcn_perm( vw[3][w], vw[2][w], 0x05040100u ) );
+      const uint2 hi = make_uint2( __builtin_amdgcn_perm( vw[1][w], vw[0][w], 0x07060302u ),
+                                   __builtin_amdgcn_perm( vw[3][w], vw[2][w], 0x07060302u ) );
+      acc[2 * w] = __builtin_amdgcn_mfma_f32_16x16x16f16( pa, __builtin_bit_cast( f16x4, lo ), acc[2 * w], 0, 0, 0 );
+      acc[2 * w + 1] = __builtin_amdgcn_mfma_f32_16x16x16f16( pa, __builtin_bit_cast( f16x4, hi ), acc[2 * w + 1], 0, 0, 0 );
+    }
+  }
+
+  // total sum of head c over the four lane groups
+  l += __shfl_xor( l, 16, WAVE );
+  l += __shfl_xor( l, 32, WAVE );
+
+  // the accumulators of this lane belong to heads 4*g4 + i; fetch their m and l from lanes c' = 4*g4 + i
+#pragma unroll
+  for ( int i = 0; i < 4; i++ ) {
+    const uint32_t hd = 4 * g4 + i;
+    const float mh = __shfl( m, (int)hd, WAVE );
+    const float lh = __shfl( l, (int)hd, WAVE );
+    if ( hd < G ) {
+      const uint64_t head = (uint64_t)job.ctx * n_heads + (uint64_t)job.h * G + hd;
+      if ( max_splits == 1 ) {
+        const float inv = 1.0f / lh;
+        union
+        {
+          uint4 raw;
+          __half h[8];
+        } o;
+#pragma unroll
+        for ( int nn = 0; nn < 8; nn++ ) {
+          o.h[nn] = __float2half_rn( acc[nn][i] * inv );
+        }
+        *reinterpret_cast<uint4*>( xb + head * HS + 8 * c ) = o.raw;
+      } else {
+        const uint64_t slot = head * max_splits + job.split;
+        float4* o = reinterpret_cast<float4*>( part.out + slot * HS + 8 * c );
+        o[0] = make_float4( acc[0][i], acc[1][i], acc[2][i], acc[3][i] );
+        o[1] = make_float4( acc[4][i], acc[5][i], acc[6][i], acc[7][i] );
+        if ( c == 0 ) {
+          part.ml[slot * 2] = mh;
+          part.ml[slot * 2 + 1] = lh;
+        }
+      }
+    }
+  }
+}
+
+// =================================================================================================
+// host side
+// =================================================================================================
+struct Plan
+{
+  int variant;
+  uint32_t chunk;       // tokens per split
+  uint32_t max_splits;  // splits of the longest context
+  uint32_t split_bound; // upper bound of max_splits for any shorter longest context (sizes the workspace)
+};
+
+bool fast_ok( const gh_shape* s, gh_dtype dt ) { return dt == GH_F16 && s->head_size == HS; }
+bool valu_gqa_ok( uint32_t g ) { return g == 1 || g == 2 || g == 4 || g == 8; }
+bool mfma_gqa_ok( uint32_t g ) { return g == 2 || g == 4 || g == 8 || g == 16; }
+
+Plan make_plan( uint64_t batch, uint32_t max_pos, const gh_shape* s, gh_dtype dt, int variant )
+{
+  Plan p;
+  p.variant = variant;
+  if ( variant == GH_ATTN_AUTO ) {
+    if ( fast_ok( s, dt ) && mfma_gqa_ok( s->gqa_size ) && s->gqa_size >= 4 ) {
+      p.variant = GH_ATTN_MFMA;
+    } else if ( fast_ok( s, dt ) && valu_gqa_ok( s->gqa_size ) ) {
+      p.variant = GH_ATTN_VALU;
+    } else {
+      p.variant = GH_ATTN_GENERIC;
+    }
+  }
+  const uint32_t n_tok = max_pos + 1;
+  uint32_t chunk;
+  uint64_t split_cap = 0;
+  if ( g_chunk_override ) {
+    chunk = g_chunk_override;
+  } else {
+    // enough independent waves to fill 256 CUs several times over, but splits no shorter than 256
+    // tokens so that the partial traffic stays a few percent of the cache traffic
+    const uint64_t streams = batch * ( p.variant == GH_ATTN_GENERIC ? s->n_heads : s->n_kv_heads );
+    const uint64_t want_waves = 4096;
+    uint64_t splits = ( want_waves + streams - 1 ) / ( streams ? streams : 1 );
+    if ( splits < 1 ) {
+      splits = 1;
+    }
+    chunk = (uint32_t)( ( n_tok + splits - 1 ) / splits );
+    if ( chunk < 256 ) {
+      chunk = 256;
+    }
+    split_cap = std::min<uint64_t>( splits, ( n_tok + 255 ) / 256 );
+  }
+  chunk = ( chunk + 15 ) / 16 * 16;
+  p.chunk = chunk;
+  p.max_splits = ( n_tok + chunk - 1 ) / chunk;
+  if ( p.max_splits < 1 ) {
+    p.max_splits = 1;
+  }
+  p.split_bound = (uint32_t)std::max<uint64_t>( p.max_splits, split_cap );
+  return p;
+}
+
+uint64_t partial_floats( uint64_t batch, const gh_shape* s, uint32_t max_splits )
+{
+  return batch * s->n_heads * (uint64_t)max_splits * ( s->head_size + 2ull );
+}
+
+template<int G>
+void launch_valu( dim3 grid, hipStream_t st, const void* q, const void* const* rows, const uint32_t* pos, Partials part, void* xb,
+                  const gh_shape* s, const Plan& p, float scale )
+{
+  attn_decode_valu_kernel<G><<<grid, 256, 0, st>>>( static_cast<const __half*>( q ), reinterpret_cast<const __half* const*>( rows ), pos, part,
+                                                   static_cast<__half*>( xb ), s->n_kv_heads, p.chunk, p.max_splits, scale );
+}
+
+template<int G>
+void launch_mfma( dim3 grid, hipStream_t st, const void* q, const void* const* rows, const uint32_t* pos, Partials part, void* xb,
+                  const gh_shape* s, const Plan& p, float scale )
+{
+  attn_decode_mfma_kernel<G><<<grid, 256, 0, st>>>( static_cast<const __half*>( q ), reinterpret_cast<const __half* const*>( rows ), pos, part,
+                                                   static_cast<__half*>( xb ), s->n_kv_heads, p.chunk, p.max_splits, scale );
+}
+
+} // namespace
+} // namespace gh
+
+using namespace gh;
+
+extern "C" {
+
+int gh_attn_set_chunk( uint32_t tokens_per_split )
+{
+  g_chunk_override = tokens_per_split;
+  return GH_OK;
+}
+
+uint64_t gh_attn_decode_workspace( uint64_t batch, uint32_t max_pos, const gh_shape* shape )
+{
+  if ( shape == nullptr || batch == 0 ) {
+    return 0;
+  }
+  // the generic kernel splits per query head and may use more splits than the fast ones; size for the larger
+  const Plan a = make_plan( batch, max_pos, shape, GH_F16, GH_ATTN_AUTO );
+  const Plan b = make_plan( batch, max_pos, shape, GH_F32, GH_ATTN_GENERIC );
+  const uint32_t splits = std::max( a.split_bound, b.split_bound );
+  return partial_floats( batch, shape, splits ) * sizeof( float ) + 256;
+}
+
+int gh_attn_decode( const void* q, const void* const* layer_rows_dev, const uint32_t* pos_dev, void* xb, uint64_t batch,
+                    uint32_t max_pos, const gh_shape* shape, gh_dtype dt, void* workspace, uint64_t workspace_bytes,
+                    int variant, gh_stream stream )
+{
+  if ( int rc = ensure_init() ) {
+    return rc;
+  }
+  if ( batch == 0 ) {
+    return GH_OK;
+  }
+  GH_REQUIRE( shape != nullptr, "gh_attn_decode: NULL shape" );
+  GH_REQUIRE( q && layer_rows_dev && pos_dev && xb, "gh_attn_decode: NULL pointer" );
+  GH_REQUIRE( dt == GH_F16 || dt == GH_F32, "gh_attn_decode: unsupported dtype %d", (int)dt );
+  GH_REQUIRE( shape->n_kv_heads > 0 && shape->gqa_size > 0 && shape->head_size > 0 && shape->seq_len > 0, "gh_attn_decode: zero dimension" );
+  GH_REQUIRE( shape->n_heads == shape->n_kv_heads * shape->gqa_size, "gh_attn_decode: n_heads != n_kv_heads * gqa_size" );
+  GH_REQUIRE( shape->kv_dim == shape->n_kv_heads * shape->head_size, "gh_attn_decode: kv_dim != n_kv_heads * head_size" );
+  GH_REQUIRE( shape->head_size <= 256, "gh_attn_decode: head_size %u > 256", shape->head_size );
+  GH_REQUIRE( max_pos < shape->seq_len, "gh_attn_decode: max_pos %u outside seq_len %u", max_pos, shape->seq_len );
+  GH_REQUIRE( batch <= 65535, "gh_attn_decode: batch too large" );
+  GH_REQUIRE( variant >= GH_ATTN_AUTO && variant <= GH_ATTN_MFMA, "gh_attn_decode: unknown variant %d", variant );
+  if ( variant == GH_ATTN_VALU ) {
+    GH_REQUIRE( fast_ok( shape, dt ) && valu_gqa_ok( shape->gqa_size ), "gh_attn_decode: the valu kernel needs f16, head_size 128, gqa in {1,2,4,8}" );
+  }
+  if ( variant == GH_ATTN_MFMA ) {
+    GH_REQUIRE( fast_ok( shape, dt ) && mfma_gqa_ok( shape->gqa_size ), "gh_attn_decode: the mfma kernel needs f16, head_size 128, gqa in {2,4,8,16}" );
+  }
+  if ( dt == GH_F16 && shape->head_size == HS ) {
+    GH_REQUIRE( ( reinterpret_cast<uintptr_t>( q ) & 15u ) == 0 && ( reinterpret_cast<uintptr_t>( xb ) & 15u ) == 0,
+                "gh_attn_decode: q and xb must be 16-byte aligned" );
+  }
+
+  const Plan plan = make_plan( batch, max_pos, shape, dt, variant );
+  Partials part { nullptr, nullptr };
+  if ( plan.max_splits > 1 ) {
+    const uint64_t need = partial_floats( batch, shape, plan.max_splits ) * sizeof( float );
+    GH_REQUIRE( workspace != nullptr, "gh_attn_decode: workspace required (%llu bytes)", (unsigned long long)need );
+    if ( workspace_bytes < need ) {
+      return fail( GH_ERR_WORKSPACE, "gh_attn_decode: workspace of %llu bytes, %llu needed", (unsigned long long)workspace_bytes,
+                   (unsigned long long)need );
+    }
+    GH_REQUIRE( ( reinterpret_cast<uintptr_t>( workspace ) & 15u ) == 0, "gh_attn_decode: workspace must be 16-byte aligned" );
+    part.out = static_cast<float*>( workspace );
+    part.ml = part.out + batch * shape->n_heads * (uint64_t)plan.max_splits * shape->head_size;
+  }
+
+  hipStream_t st = as_stream( stream );
+  const float scale = LOG2E / sqrtf( (float)shape->head_size );
+  int timer = -1;
+  if ( int rc = timer_begin( st, &timer ) ) {
+    return rc;
+  }
+
+  if ( plan.variant == GH_ATTN_GENERIC ) {
+    const dim3 grid( shape->n_heads, plan.max_splits, (unsigned)batch );
+    if ( dt == GH_F16 ) {
+      attn_decode_generic_kernel<__half><<<grid, 64, 0, st>>>( static_cast<const __half*>( q ), reinterpret_cast<const __half* const*>( layer_rows_dev ),
+                                                              pos_dev, part, static_cast<__half*>( xb ), shape->n_kv_heads, shape->gqa_size,
+                                                              shape->head_size, plan.chunk, plan.max_splits, scale );
+    } else {
+      attn_decode_generic_kernel<float><<<grid, 64, 0, st>>>( static_cast<const float*>( q ), reinterpret_cast<const float* const*>( layer_rows_dev ),
+                                                             pos_dev, part, static_cast<float*>( xb ), shape->n_kv_heads, shape->gqa_size,
+                                                             shape->head_size, plan.chunk, plan.max_splits, scale );
+    }
+  } else {
+    const uint64_t n_blocks = batch * plan.max_splits * ( ( shape->n_kv_heads + 3 ) / 4 );
+    GH_REQUIRE( n_blocks <= 0x7fffffffull, "gh_attn_decode: grid too large" );
+    const dim3 grid( (unsigned)n_blocks );
+    if ( plan.variant == GH_ATTN_VALU ) {
+      switch ( shape->gqa_size ) {
+        case 1: launch_valu<1>( grid, st, q, layer_rows_dev, pos_dev, part, xb, shape, plan, scale ); break;
+        case 2: launch_valu<2>( grid, st, q, layer_rows_dev, pos_dev, part, xb, shape, plan, scale ); break;
+        case 4: launch_valu<4>( grid, st, q, layer_rows_dev, pos_dev, part, xb, shape, plan, scale ); break;
+        default: launch_valu<8>( grid, st, q, layer_rows_dev, pos_dev, part, xb, shape, plan, scale ); break;
+      }
+    } else {
+      switch ( shape->gqa_size ) {
+        case 2: launch_mfma<2>( grid, st, q, layer_rows_dev, pos_dev, part, xb, shape, plan, scale ); break;
+        case 4: launch_mfma<4>( grid, st, q, layer_rows_dev, pos_dev, part, xb, shape, plan, scale ); break;
+        case 8: launch_mfma<8>( grid, st, q, layer_rows_dev, pos_dev, part, xb, shape, plan, scale ); break;
+        default: launch_mfma<16>( grid, st, q, layer_rows_dev, pos_dev, part, xb, shape, plan, scale ); break;
+      }
+    }
+  }
+  GH_LAUNCH_CHECK();
+
+  if ( plan.max_splits > 1 ) {
+    const dim3 grid( shape->n_heads, (unsigned)batch );
+    const unsigned threads = shape->head_size <= 64 ? 64 : ( shape->head_size <= 128 ? 128 : 256 );
+    if ( dt == GH_F16 ) {
+      attn_merge_kernel<__half><<<grid, threads, 0, st>>>( part, layer_rows_dev, pos_dev, static_cast<__half*>( xb ), shape->n_heads,
+                                                          shape->head_size, plan.chunk, plan.max_splits );
+    } else {
+      attn_merge_kernel<float><<<grid, threads, 0, st>>>( part, layer_rows_dev, pos_dev, static_cast<float*>( xb ), shape->n_heads,
+                                                         shape->head_size, plan.chunk, plan.max_splits );
+    }
+    GH_LAUNCH_CHECK();
+  }
+  return timer_end( st, timer );
+}
+
+int gh_attn_decode_host( const void* q, const void* const* layer_rows_host, const uint32_t* pos_host, void* xb, uint64_t batch,
+                         const gh_shape* shape, gh_dtype dt, void* workspace, uint64_t workspace_bytes, int variant, gh_stream stream )
+{
+  if ( int rc = ensure_init() ) {
+    return rc;
+  }
+  if ( batch == 0 ) {
+    return GH_OK;
+  }
+  GH_REQUIRE( layer_rows_host && pos_host, "gh_attn_decode_host: NULL table" );
+  GH_REQUIRE( batch <= MAX_BATCH, "gh_attn_decode_host: batch %llu > %llu", (unsigned long long)batch, (unsigned long long)MAX_BATCH );
+  uint32_t max_pos = 0;
+  for ( uint64_t i = 0; i < batch; i++ ) {
+    if ( layer_rows_host[i] != nullptr ) {
+      max_pos = std::max( max_pos, pos_host[i] );
+    }
+  }
+  void* d_rows = nullptr;
+  void* d_pos = nullptr;
+  if ( int rc = stage_table( layer_rows_host, batch * sizeof( void* ), as_stream( stream ), &d_rows ) ) {
+    return rc;
+  }
+  if ( int rc = stage_table( pos_host, batch * sizeof( uint32_t ), as_stream( stream ), &d_pos ) ) {
+    return rc;
+  }
+  if ( int rc = gh_attn_decode( q, static_cast<const void* const*>( d_rows ), static_cast<const uint32_t*>( d_pos ), xb, batch, max_pos, shape, dt,
+                                workspace, workspace_bytes, variant, stream ) ) {
+    return rc;
+  }
+  return stage_fence( as_stream( stream ) );
+}
+
+} // extern "C"

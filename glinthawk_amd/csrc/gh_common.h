@@ -1,0 +1,110 @@
+// Internal helpers shared by the HIP translation units of libglint_hip.so (gfx950 only).
+#pragma once
+
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+
+#include "glint_hip.h"
+
+namespace gh {
+
+// ---- error plumbing ---------------------------------------------------------------------------
+void set_error( const char* fmt, ... ) __attribute__( ( format( printf, 1, 2 ) ) );
+int fail( int status, const char* fmt, ... ) __attribute__( ( format( printf, 2, 3 ) ) );
+
+#define GH_HIP( expr )                                                                                                 \
+  do {                                                                                                                 \
+    hipError_t gh_err_ = ( expr );                                                                                     \
+    if ( gh_err_ != hipSuccess ) {                                                                                     \
+      return ::gh::fail( gh_err_ == hipErrorOutOfMemory ? GH_ERR_OOM : GH_ERR_DEVICE,                                  \
+                         "%s failed: %s (%s:%d)",                                                                      \
+                         #expr,                                                                                        \
+                         hipGetErrorString( gh_err_ ),                                                                 \
+                         __FILE__,                                                                                     \
+                         __LINE__ );                                                                                   \
+    }                                                                                                                  \
+  } while ( 0 )
+
+#define GH_REQUIRE( cond, ... )                                                                                        \
+  do {                                                                                                                 \
+    if ( !( cond ) ) {                                                                                                 \
+      return ::gh::fail( GH_ERR_INVALID, __VA_ARGS__ );                                                                \
+    }                                                                                                                  \
+  } while ( 0 )
+
+// after a kernel launch: surface launch-configuration errors
+#define GH_LAUNCH_CHECK() GH_HIP( hipGetLastError() )
+
+int ensure_init();
+
+inline hipStream_t as_stream( gh_stream s ) { return reinterpret_cast<hipStream_t>( s ); }
+
+inline size_t dtype_size( gh_dtype dt ) { return dt == GH_F32 ? 4 : 2; }
+
+// ---- staging of host-side pointer / position tables ------------------------------------------
+// Copies `bytes` from a host array into a slot of a device-side ring (via pinned memory) on
+// `stream` and returns the device address.  A slot is reused only after the work that was queued
+// behind its previous use has finished.
+int stage_table( const void* host_src, size_t bytes, hipStream_t stream, void** dev_out );
+// Marks the end of the work that reads the most recently staged slots on this stream.
+int stage_fence( hipStream_t stream );
+
+// Event pair around a kernel sequence when the benchmark's timer is enabled (pair == -1: off).
+int timer_begin( hipStream_t stream, int* pair_out );
+int timer_end( hipStream_t stream, int pair );
+
+constexpr size_t STAGE_SLOT_BYTES = 16 * 1024; // 1024 rows x (8-byte pointer + 4-byte position) fits
+constexpr uint64_t MAX_BATCH = 1024;           // models/llama2/base.hh:26
+
+// ---- device helpers ---------------------------------------------------------------------------
+constexpr int WAVE = 64;
+
+__device__ __forceinline__ float wave_sum( float v )
+{
+#pragma unroll
+  for ( int off = 32; off > 0; off >>= 1 ) {
+    v += __shfl_xor( v, off, WAVE );
+  }
+  return v;
+}
+
+__device__ __forceinline__ float wave_max( float v )
+{
+#pragma unroll
+  for ( int off = 32; off > 0; off >>= 1 ) {
+    v = fmaxf( v, __shfl_xor( v, off, WAVE ) );
+  }
+  return v;
+}
+
+template<typename T>
+__device__ __forceinline__ float to_f32( T v );
+template<>
+__device__ __forceinline__ float to_f32<float>( float v )
+{
+  return v;
+}
+template<>
+__device__ __forceinline__ float to_f32<__half>( __half v )
+{
+  return __half2float( v );
+}
+
+template<typename T>
+__device__ __forceinline__ T from_f32( float v );
+template<>
+__device__ __forceinline__ float from_f32<float>( float v )
+{
+  return v;
+}
+template<>
+__device__ __forceinline__ __half from_f32<__half>( float v )
+{
+  return __float2half_rn( v );
+}
+
+} // namespace gh

@@ -1,0 +1,277 @@
+// Dense projection GEMM of the stage: xout(b, r) = sum_p w(r, p) * x(b, p), w row-major (r, s),
+// fp32 accumulate (Operations::matmul / untemplated_matmul, arch/amd64/common/ops.hh:74-93,212-271).
+//
+// f16: MFMA kernel.  The weight matrix is the streamed operand (read exactly once), the
+// activations are the small operand.  A work-group owns a 64-row slab of w and a 64-column slab of
+// the batch, walks K in steps of 128, stages both tiles in LDS with 16-byte chunks XOR-swizzled so
+// that the MFMA-operand reads are bank-conflict free, and keeps 4 x (16x16) fp32 accumulators per
+// wave (v_mfma_f32_16x16x32_f16).  When r / 64 is too small to fill the chip K is split across
+// work-groups and an fp32 partial buffer is reduced by a second kernel.
+//
+// f32: plain wave-per-row kernel (only the tiny fp32 configuration uses it).
+#include "gh_common.h"
+
+#include <mutex>
+
+namespace gh {
+namespace {
+
+typedef _Float16 f16x8 __attribute__( ( ext_vector_type( 8 ) ) );
+typedef float f32x4 __attribute__( ( ext_vector_type( 4 ) ) );
+
+constexpr int BM = 64;  // weight rows per work-group
+constexpr int BN = 64;  // batch columns per work-group
+constexpr int BK = 128; // k per stage (16 chunks of 8 halves)
+
+std::mutex g_ws_mutex;
+float* g_ws = nullptr; // split-K partials, grow-only
+uint64_t g_ws_bytes = 0;
+
+int ensure_workspace( uint64_t bytes, float** out )
+{
+  std::lock_guard<std::mutex> lock( g_ws_mutex );
+  if ( bytes > g_ws_bytes ) {
+    if ( g_ws ) {
+      GH_HIP( hipDeviceSynchronize() );
+      GH_HIP( hipFree( g_ws ) );
+      g_ws = nullptr;
+      g_ws_bytes = 0;
+    }
+    const uint64_t want = std::max<uint64_t>( bytes, 64ull << 20 );
+    GH_HIP( hipMalloc( reinterpret_cast<void**>( &g_ws ), want ) );
+    g_ws_bytes = want;
+  }
+  *out = g_ws;
+  return GH_OK;
+}
+
+// Loads one (64 x 128) f16 tile, rows [row0, row0+64) x k [k0, k0+128) of a row-major matrix with
+// leading dimension ld, into registers: thread t handles chunk (t % 16) of rows t/16 + 16*i.
+// Rows >= n_rows and k >= k_end read as zero.
+struct TileRegs
+{
+  uint4 v[4];
+};
+
+__device__ __forceinline__ TileRegs load_tile( const __half* __restrict__ mat, uint64_t ld, uint32_t row0, uint32_t n_rows, uint32_t k0, uint32_t k_end, bool k_vec_ok )
+{
+  TileRegs t;
+  const uint32_t chunk = threadIdx.x & 15;
+  const uint32_t k = k0 + chunk * 8;
+#pragma unroll
+  for ( int i = 0; i < 4; i++ ) {
+    const uint32_t row = row0 + ( threadIdx.x >> 4 ) + 16 * i;
+    uint4 v = make_uint4( 0, 0, 0, 0 );
+    if ( row < n_rows && k < k_end ) {
+      const __half* p = mat + (uint64_t)row * ld + k;
+      if ( k_vec_ok && k + 8 <= k_end ) {
+        v = *reinterpret_cast<const uint4*>( p );
+      } else {
+        union
+        {
+          uint4 raw;
+          __half h[8];
+        } u;
+        u.raw = make_uint4( 0, 0, 0, 0 );
+        for ( int e = 0; e < 8; e++ ) {
+          if ( k + e < k_end ) {
+            u.h[e] = p[e];
+          }
+        }
+        v = u.raw;
+      }
+    }
+    t.v[i] = v;
+  }
+  return t;
+}
+
+__device__ __forceinline__ void store_tile( uint4* lds, const TileRegs& t )
+{
+  const uint32_t chunk = threadIdx.x & 15;
+#pragma unroll
+  for ( int i = 0; i < 4; i++ ) {
+    const uint32_t row = ( threadIdx.x >> 4 ) + 16 * i;
+    lds[row * 16 + ( chunk ^ ( row & 15 ) )] = t.v[i];
+  }
+}
+
+// grid: (ceil(r / 64), ceil(b / 64), k_splits)
+template<bool SPLIT>
+__global__ __launch_bounds__( 256 ) void gemm_f16_kernel( __half* __restrict__ xout,
+                                                          float* __restrict__ partial,
+                                                          const __half* __restrict__ x,
+                                                          const __half* __restrict__ w,
+                                                          uint32_t s,
+                                                          uint32_t r,
+                                                          uint32_t b,
+                                                          uint32_t k_per_split,
+                                                          bool k_vec_ok )
+{
+  __shared__ uint4 s_w[2][BM * 16];
+  __shared__ uint4 s_x[2][BN * 16];
+
+  const uint32_t row0 = blockIdx.x * BM;
+  const uint32_t col0 = blockIdx.y * BN;
+  const uint32_t k_begin = blockIdx.z * k_per_split;
+  const uint32_t k_end = min( s, k_begin + k_per_split );
+  const uint32_t wave = threadIdx.x >> 6;
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t c = lane & 15;
+  const uint32_t g4 = lane >> 4;
+
+  f32x4 acc[4];
+#pragma unroll
+  for ( int j = 0; j < 4; j++ ) {
+    acc[j] = f32x4 { 0.0f, 0.0f, 0.0f, 0.0f };
+  }
+
+  TileRegs tw = load_tile( w, s, row0, r, k_begin, k_end, k_vec_ok );
+  TileRegs tx = load_tile( x, s, col0, b, k_begin, k_end, k_vec_ok );
+  int buf = 0;
+  for ( uint32_t k0 = k_begin; k0 < k_end; k0 += BK ) {
+    store_tile( s_w[buf], tw );
+    store_tile( s_x[buf], tx );
+    __syncthreads();
+    if ( k0 + BK < k_end ) {
+      tw = load_tile( w, s, row0, r, k0 + BK, k_end, k_vec_ok );
+      tx = load_tile( x, s, col0, b, k0 + BK, k_end, k_vec_ok );
+    }
+    const uint4* lw = s_w[buf];
+    const uint4* lx = s_x[buf];
+    const uint32_t arow = wave * 16 + c;
+#pragma unroll
+    for ( int kk = 0; kk < 4; kk++ ) {
+      const uint32_t ch = 4 * kk + g4;
+      const f16x8 a = __builtin_bit_cast( f16x8, lw[arow * 16 + ( ch ^ ( arow & 15 ) )] );
+#pragma unroll
+      for ( int j = 0; j < 4; j++ ) {
+        const uint32_t brow = 16 * j + c;
+        const f16x8 bb = __builtin_bit_cast( f16x8, lx[brow * 16 + ( ch ^ ( brow & 15 ) )] );
+        acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16( a, bb, acc[j], 0, 0, 0 );
+      }
+    }
+    buf ^= 1; // the other buffer is free: its readers passed the barrier of this iteration
+  }
+
+  // acc[j][i] = out(row0 + 16*wave + 4*g4 + i, col0 + 16*j + c)
+#pragma unroll
+  for ( int j = 0; j < 4; j++ ) {
+    const uint32_t col = col0 + 16 * j + c;
+    if ( col >= b ) {
+      continue;
+    }
+#pragma unroll
+    for ( int i = 0; i < 4; i++ ) {
+      const uint32_t row = row0 + 16 * wave + 4 * g4 + i;
+      if ( row < r ) {
+        if ( SPLIT ) {
+          partial[( (uint64_t)blockIdx.z * b + col ) * r + row] = acc[j][i];
+        } else {
+          xout[(uint64_t)col * r + row] = __float2half_rn( acc[j][i] );
+        }
+      }
+    }
+  }
+}
+
+__global__ __launch_bounds__( 256 ) void gemm_reduce_kernel( __half* __restrict__ xout, const float* __restrict__ partial, uint64_t n, uint32_t splits )
+{
+  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  for ( uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride ) {
+    float sum = 0.0f;
+    for ( uint32_t k = 0; k < splits; k++ ) {
+      sum += partial[(uint64_t)k * n + i];
+    }
+    xout[i] = __float2half_rn( sum );
+  }
+}
+
+// f32: one wave per weight row, batch columns looped
+__global__ __launch_bounds__( 256 ) void gemm_f32_kernel( float* __restrict__ xout, const float* __restrict__ x, const float* __restrict__ w, uint32_t s, uint32_t r, uint32_t b )
+{
+  const uint32_t row = blockIdx.x * 4 + ( threadIdx.x >> 6 );
+  if ( row >= r ) {
+    return;
+  }
+  const uint32_t lane = threadIdx.x & 63;
+  const float* wr = w + (uint64_t)row * s;
+  for ( uint32_t col = 0; col < b; col++ ) {
+    const float* xc = x + (uint64_t)col * s;
+    float sum = 0.0f;
+    for ( uint32_t p = lane; p < s; p += 64 ) {
+      sum += wr[p] * xc[p];
+    }
+    sum = wave_sum( sum );
+    if ( lane == 0 ) {
+      xout[(uint64_t)col * r + row] = sum;
+    }
+  }
+}
+
+} // namespace
+} // namespace gh
+
+using namespace gh;
+
+extern "C" {
+
+int gh_matmul( void* xout, const void* x, const void* w, uint64_t s, uint64_t r, uint64_t b, gh_dtype dt, gh_stream stream )
+{
+  if ( int rc = ensure_init() ) {
+    return rc;
+  }
+  if ( b == 0 || r == 0 ) {
+    return GH_OK;
+  }
+  GH_REQUIRE( xout && x && w, "gh_matmul: NULL pointer" );
+  GH_REQUIRE( s > 0 && s <= 0x7fffffffull && r <= 0x7fffffffull && b <= 0x7fffffffull, "gh_matmul: bad shape" );
+  hipStream_t st = as_stream( stream );
+
+  if ( dt == GH_F32 ) {
+    gemm_f32_kernel<<<(unsigned)( ( r + 3 ) / 4 ), 256, 0, st>>>( static_cast<float*>( xout ), static_cast<const float*>( x ), static_cast<const float*>( w ),
+                                                                 (uint32_t)s, (uint32_t)r, (uint32_t)b );
+    GH_LAUNCH_CHECK();
+    return GH_OK;
+  }
+  GH_REQUIRE( dt == GH_F16, "gh_matmul: unsupported dtype %d", (int)dt );
+
+  const bool k_vec_ok = ( s % 8 == 0 ) && ( ( reinterpret_cast<uintptr_t>( x ) | reinterpret_cast<uintptr_t>( w ) ) & 15u ) == 0;
+  const uint32_t grid_m = (uint32_t)( ( r + BM - 1 ) / BM );
+  const uint32_t grid_n = (uint32_t)( ( b + BN - 1 ) / BN );
+  GH_REQUIRE( grid_n <= 65535, "gh_matmul: batch too large" );
+  // split K until there are about 1024 work-groups (4 per CU), keeping at least 1024 k per split
+  uint32_t splits = 1;
+  const uint64_t tiles = (uint64_t)grid_m * grid_n;
+  if ( tiles < 1024 ) {
+    splits = (uint32_t)( ( 1024 + tiles - 1 ) / tiles );
+    const uint32_t max_by_k = (uint32_t)std::max<uint64_t>( 1, s / 1024 );
+    splits = std::min( splits, max_by_k );
+    splits = std::min<uint32_t>( splits, 16 );
+  }
+  uint32_t k_per_split = (uint32_t)( ( s + splits - 1 ) / splits );
+  k_per_split = ( k_per_split + BK - 1 ) / BK * BK;
+  splits = (uint32_t)( ( s + k_per_split - 1 ) / k_per_split );
+
+  const dim3 grid( grid_m, grid_n, splits );
+  if ( splits == 1 ) {
+    gemm_f16_kernel<false><<<grid, 256, 0, st>>>( static_cast<__half*>( xout ), nullptr, static_cast<const __half*>( x ), static_cast<const __half*>( w ),
+                                                 (uint32_t)s, (uint32_t)r, (uint32_t)b, k_per_split, k_vec_ok );
+    GH_LAUNCH_CHECK();
+    return GH_OK;
+  }
+  float* ws = nullptr;
+  if ( int rc = ensure_workspace( (uint64_t)splits * b * r * sizeof( float ), &ws ) ) {
+    return rc;
+  }
+  gemm_f16_kernel<true><<<grid, 256, 0, st>>>( nullptr, ws, static_cast<const __half*>( x ), static_cast<const __half*>( w ), (uint32_t)s, (uint32_t)r,
+                                              (uint32_t)b, k_per_split, k_vec_ok );
+  GH_LAUNCH_CHECK();
+  const uint64_t n = b * r;
+  const unsigned blocks = (unsigned)std::min<uint64_t>( ( n + 255 ) / 256, 4096 );
+  gemm_reduce_kernel<<<blocks, 256, 0, st>>>( static_cast<__half*>( xout ), ws, n, splits );
+  GH_LAUNCH_CHECK();
+  return GH_OK;
+}
+
+} // extern "C"

@@ -1,0 +1,426 @@
+// Runtime half of libglint_hip.so: device selection, error text, allocation and copies, the
+// staging ring for host-side tables, the paged (virtual-memory) KV arena and the event-based
+// kernel timer used by the benchmark.
+#include "gh_common.h"
+
+#include <cstdarg>
+#include <mutex>
+#include <vector>
+
+namespace gh {
+
+namespace {
+
+thread_local char g_error[512] = "";
+
+std::mutex g_mutex;
+bool g_ready = false;
+int g_device = -1;
+char g_arch[128] = "";
+
+// ---- staging ring ------------------------------------------------------------------------------
+constexpr int STAGE_SLOTS = 64;
+struct StageSlot
+{
+  char* pinned = nullptr;
+  char* device = nullptr;
+  hipEvent_t done = nullptr;
+  bool in_flight = false;
+};
+StageSlot g_slots[STAGE_SLOTS];
+int g_next_slot = 0;
+std::vector<int> g_unfenced;
+
+// ---- attention kernel timer ----------------------------------------------------------------
+constexpr int TIMER_PAIRS = 8192;
+bool g_timing = false;
+std::vector<hipEvent_t> g_ev_begin, g_ev_end;
+int g_ev_used = 0;
+
+} // namespace
+
+void set_error( const char* fmt, ... )
+{
+  va_list ap;
+  va_start( ap, fmt );
+  vsnprintf( g_error, sizeof( g_error ), fmt, ap );
+  va_end( ap );
+}
+
+int fail( int status, const char* fmt, ... )
+{
+  va_list ap;
+  va_start( ap, fmt );
+  vsnprintf( g_error, sizeof( g_error ), fmt, ap );
+  va_end( ap );
+  return status;
+}
+
+static int init_locked( int device )
+{
+  int count = 0;
+  hipError_t err = hipGetDeviceCount( &count );
+  if ( err != hipSuccess || count == 0 ) {
+    (void)hipGetLastError();
+    return fail( GH_ERR_NO_DEVICE, "no HIP device visible (%s)", err == hipSuccess ? "count is 0" : hipGetErrorString( err ) );
+  }
+  if ( device < 0 || device >= count ) {
+    return fail( GH_ERR_INVALID, "device %d out of range (0..%d)", device, count - 1 );
+  }
+  GH_HIP( hipSetDevice( device ) );
+  hipDeviceProp_t prop;
+  GH_HIP( hipGetDeviceProperties( &prop, device ) );
+  snprintf( g_arch, sizeof( g_arch ), "%s", prop.gcnArchName );
+  if ( strncmp( prop.gcnArchName, "gfx950", 6 ) != 0 ) {
+    return fail( GH_ERR_NO_DEVICE, "device %d is %s; this library holds gfx950 code only", device, prop.gcnArchName );
+  }
+  for ( int i = 0; i < STAGE_SLOTS; i++ ) {
+    GH_HIP( hipHostMalloc( reinterpret_cast<void**>( &g_slots[i].pinned ), STAGE_SLOT_BYTES, hipHostMallocDefault ) );
+    GH_HIP( hipMalloc( reinterpret_cast<void**>( &g_slots[i].device ), STAGE_SLOT_BYTES ) );
+    GH_HIP( hipEventCreateWithFlags( &g_slots[i].done, hipEventDisableTiming ) );
+  }
+  g_device = device;
+  g_ready = true;
+  return GH_OK;
+}
+
+int ensure_init()
+{
+  std::lock_guard<std::mutex> lock( g_mutex );
+  if ( g_ready ) {
+    return GH_OK;
+  }
+  return init_locked( 0 );
+}
+
+int stage_table( const void* host_src, size_t bytes, hipStream_t stream, void** dev_out )
+{
+  GH_REQUIRE( bytes <= STAGE_SLOT_BYTES, "table of %zu bytes exceeds the staging slot (%zu)", bytes, STAGE_SLOT_BYTES );
+  std::lock_guard<std::mutex> lock( g_mutex );
+  StageSlot& slot = g_slots[g_next_slot];
+  if ( slot.in_flight ) {
+    GH_HIP( hipEventSynchronize( slot.done ) );
+    slot.in_flight = false;
+  }
+  memcpy( slot.pinned, host_src, bytes );
+  GH_HIP( hipMemcpyAsync( slot.device, slot.pinned, bytes, hipMemcpyHostToDevice, stream ) );
+  g_unfenced.push_back( g_next_slot );
+  g_next_slot = ( g_next_slot + 1 ) % STAGE_SLOTS;
+  *dev_out = slot.device;
+  return GH_OK;
+}
+
+int stage_fence( hipStream_t stream )
+{
+  std::lock_guard<std::mutex> lock( g_mutex );
+  for ( int idx : g_unfenced ) {
+    GH_HIP( hipEventRecord( g_slots[idx].done, stream ) );
+    g_slots[idx].in_flight = true;
+  }
+  g_unfenced.clear();
+  return GH_OK;
+}
+
+// timer hooks used by gh_attn_decode
+int timer_begin( hipStream_t stream, int* pair_out )
+{
+  *pair_out = -1;
+  if ( !g_timing ) {
+    return GH_OK;
+  }
+  std::lock_guard<std::mutex> lock( g_mutex );
+  if ( g_ev_used >= TIMER_PAIRS ) {
+    return GH_OK; // silently stop sampling; the mean over the recorded pairs stays valid
+  }
+  if ( (int)g_ev_begin.size() <= g_ev_used ) {
+    hipEvent_t a, b;
+    GH_HIP( hipEventCreate( &a ) );
+    GH_HIP( hipEventCreate( &b ) );
+    g_ev_begin.push_back( a );
+    g_ev_end.push_back( b );
+  }
+  *pair_out = g_ev_used++;
+  GH_HIP( hipEventRecord( g_ev_begin[*pair_out], stream ) );
+  return GH_OK;
+}
+
+int timer_end( hipStream_t stream, int pair )
+{
+  if ( pair < 0 ) {
+    return GH_OK;
+  }
+  GH_HIP( hipEventRecord( g_ev_end[pair], stream ) );
+  return GH_OK;
+}
+
+} // namespace gh
+
+using namespace gh;
+
+extern "C" {
+
+int gh_init( int device )
+{
+  std::lock_guard<std::mutex> lock( g_mutex );
+  if ( g_ready ) {
+    if ( device != g_device ) {
+      return fail( GH_ERR_INVALID, "already initialised on device %d", g_device );
+    }
+    return GH_OK;
+  }
+  return init_locked( device );
+}
+
+const char* gh_last_error( void ) { return g_error; }
+
+int gh_device_name( char* out, size_t len )
+{
+  if ( int rc = ensure_init() ) {
+    return rc;
+  }
+  snprintf( out, len, "%s", g_arch );
+  return GH_OK;
+}
+
+int gh_sync( gh_stream stream )
+{
+  if ( int rc = ensure_init() ) {
+    return rc;
+  }
+  if ( stream == nullptr ) {
+    GH_HIP( hipDeviceSynchronize() );
+  } else {
+    GH_HIP( hipStreamSynchronize( as_stream( stream ) ) );
+  }
+  return GH_OK;
+}
+
+int gh_malloc( void** out, uint64_t bytes )
+{
+  if ( int rc = ensure_init() ) {
+    return rc;
+  }
+  GH_REQUIRE( out != nullptr, "gh_malloc: out is NULL" );
+  *out = nullptr;
+  if ( bytes == 0 ) {
+    return GH_OK;
+  }
+  GH_HIP( hipMalloc( out, bytes ) );
+  return GH_OK;
+}
+
+int gh_free( void* ptr )
+{
+  if ( ptr != nullptr ) {
+    GH_HIP( hipFree( ptr ) );
+  }
+  return GH_OK;
+}
+
+int gh_host_malloc( void** out, uint64_t bytes )
+{
+  if ( int rc = ensure_init() ) {
+    return rc;
+  }
+  GH_REQUIRE( out != nullptr, "gh_host_malloc: out is NULL" );
+  *out = nullptr;
+  if ( bytes == 0 ) {
+    return GH_OK;
+  }
+  GH_HIP( hipHostMalloc( out, bytes, hipHostMallocDefault ) );
+  return GH_OK;
+}
+
+int gh_host_free( void* ptr )
+{
+  if ( ptr != nullptr ) {
+    GH_HIP( hipHostFree( ptr ) );
+  }
+  return GH_OK;
+}
+
+int gh_memcpy( void* dst, const void* src, uint64_t bytes, gh_copy_kind kind, int async, gh_stream stream )
+{
+  if ( int rc = ensure_init() ) {
+    return rc;
+  }
+  if ( bytes == 0 ) {
+    return GH_OK;
+  }
+  GH_REQUIRE( dst != nullptr && src != nullptr, "gh_memcpy: NULL pointer" );
+  hipMemcpyKind k;
+  switch ( kind ) {
+    case GH_HOST_TO_DEVICE: k = hipMemcpyHostToDevice; break;
+    case GH_DEVICE_TO_HOST: k = hipMemcpyDeviceToHost; break;
+    case GH_DEVICE_TO_DEVICE: k = hipMemcpyDeviceToDevice; break;
+    case GH_HOST_TO_HOST: k = hipMemcpyHostToHost; break;
+    default: return fail( GH_ERR_INVALID, "gh_memcpy: bad copy kind %d", (int)kind );
+  }
+  GH_HIP( hipMemcpyAsync( dst, src, bytes, k, as_stream( stream ) ) );
+  if ( !async ) {
+    GH_HIP( hipStreamSynchronize( as_stream( stream ) ) );
+  }
+  return GH_OK;
+}
+
+// ---- paged arena ------------------------------------------------------------------------------
+struct gh_vmm
+{
+  void* base = nullptr;
+  uint64_t len = 0;
+  uint64_t granularity = 0;
+  struct Span
+  {
+    uint64_t offset;
+    uint64_t len;
+    hipMemGenericAllocationHandle_t handle;
+  };
+  std::vector<Span> spans;
+  uint64_t committed = 0;
+};
+
+static int vmm_props( hipMemAllocationProp* prop )
+{
+  memset( prop, 0, sizeof( *prop ) );
+  prop->type = hipMemAllocationTypePinned;
+  prop->location.type = hipMemLocationTypeDevice;
+  int dev = 0;
+  GH_HIP( hipGetDevice( &dev ) );
+  prop->location.id = dev;
+  return GH_OK;
+}
+
+int gh_vmm_granularity( uint64_t* out )
+{
+  if ( int rc = ensure_init() ) {
+    return rc;
+  }
+  hipMemAllocationProp prop;
+  if ( int rc = vmm_props( &prop ) ) {
+    return rc;
+  }
+  size_t g = 0;
+  GH_HIP( hipMemGetAllocationGranularity( &g, &prop, hipMemAllocationGranularityMinimum ) );
+  *out = g;
+  return GH_OK;
+}
+
+int gh_vmm_reserve( gh_vmm** out, uint64_t bytes )
+{
+  if ( int rc = ensure_init() ) {
+    return rc;
+  }
+  GH_REQUIRE( out != nullptr && bytes > 0, "gh_vmm_reserve: bad arguments" );
+  uint64_t gran = 0;
+  if ( int rc = gh_vmm_granularity( &gran ) ) {
+    return rc;
+  }
+  const uint64_t rounded = ( bytes + gran - 1 ) / gran * gran;
+  void* base = nullptr;
+  GH_HIP( hipMemAddressReserve( &base, rounded, 0, nullptr, 0 ) );
+  gh_vmm* r = new gh_vmm;
+  r->base = base;
+  r->len = rounded;
+  r->granularity = gran;
+  *out = r;
+  return GH_OK;
+}
+
+void* gh_vmm_ptr( const gh_vmm* r ) { return r ? r->base : nullptr; }
+uint64_t gh_vmm_max_len( const gh_vmm* r ) { return r ? r->len : 0; }
+uint64_t gh_vmm_committed_bytes( const gh_vmm* r ) { return r ? r->committed : 0; }
+
+int gh_vmm_commit( gh_vmm* r, uint64_t offset, uint64_t len )
+{
+  GH_REQUIRE( r != nullptr, "gh_vmm_commit: NULL region" );
+  GH_REQUIRE( len > 0 && offset + len <= r->len, "gh_vmm_commit: span [%llu, +%llu) outside the %llu-byte region",
+              (unsigned long long)offset, (unsigned long long)len, (unsigned long long)r->len );
+  GH_REQUIRE( offset % r->granularity == 0 && len % r->granularity == 0,
+              "gh_vmm_commit: span must be a multiple of the %llu-byte granularity", (unsigned long long)r->granularity );
+  hipMemAllocationProp prop;
+  if ( int rc = vmm_props( &prop ) ) {
+    return rc;
+  }
+  hipMemGenericAllocationHandle_t handle;
+  GH_HIP( hipMemCreate( &handle, len, &prop, 0 ) );
+  void* at = static_cast<char*>( r->base ) + offset;
+  hipError_t err = hipMemMap( at, len, 0, handle, 0 );
+  if ( err != hipSuccess ) {
+    (void)hipMemRelease( handle );
+    return fail( GH_ERR_DEVICE, "hipMemMap failed: %s", hipGetErrorString( err ) );
+  }
+  hipMemAccessDesc access;
+  memset( &access, 0, sizeof( access ) );
+  access.location = prop.location;
+  access.flags = hipMemAccessFlagsProtReadWrite;
+  err = hipMemSetAccess( at, len, &access, 1 );
+  if ( err != hipSuccess ) {
+    (void)hipMemUnmap( at, len );
+    (void)hipMemRelease( handle );
+    return fail( GH_ERR_DEVICE, "hipMemSetAccess failed: %s", hipGetErrorString( err ) );
+  }
+  r->spans.push_back( { offset, len, handle } );
+  r->committed += len;
+  return GH_OK;
+}
+
+int gh_vmm_clear( gh_vmm* r )
+{
+  GH_REQUIRE( r != nullptr, "gh_vmm_clear: NULL region" );
+  for ( auto& s : r->spans ) {
+    GH_HIP( hipMemUnmap( static_cast<char*>( r->base ) + s.offset, s.len ) );
+    GH_HIP( hipMemRelease( s.handle ) );
+  }
+  r->spans.clear();
+  r->committed = 0;
+  return GH_OK;
+}
+
+int gh_vmm_free( gh_vmm* r )
+{
+  if ( r == nullptr ) {
+    return GH_OK;
+  }
+  if ( int rc = gh_vmm_clear( r ) ) {
+    return rc;
+  }
+  GH_HIP( hipMemAddressFree( r->base, r->len ) );
+  delete r;
+  return GH_OK;
+}
+
+// ---- kernel timer ------------------------------------------------------------------------------
+int gh_attn_timing_enable( int on )
+{
+  std::lock_guard<std::mutex> lock( g_mutex );
+  g_timing = on != 0;
+  return GH_OK;
+}
+
+int gh_attn_timing_reset( void )
+{
+  std::lock_guard<std::mutex> lock( g_mutex );
+  g_ev_used = 0;
+  return GH_OK;
+}
+
+int gh_attn_timing_read( double* total_ms, uint64_t* launches )
+{
+  std::lock_guard<std::mutex> lock( g_mutex );
+  double total = 0.0;
+  for ( int i = 0; i < g_ev_used; i++ ) {
+    GH_HIP( hipEventSynchronize( g_ev_end[i] ) );
+    float ms = 0.0f;
+    GH_HIP( hipEventElapsedTime( &ms, g_ev_begin[i], g_ev_end[i] ) );
+    total += ms;
+  }
+  if ( total_ms ) {
+    *total_ms = total;
+  }
+  if ( launches ) {
+    *launches = (uint64_t)g_ev_used;
+  }
+  return GH_OK;
+}
+
+} // extern "C"

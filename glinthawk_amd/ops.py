@@ -1,0 +1,211 @@
+"""Thin torch-tensor front-end over the C-ABI, for the tests and the benchmark.
+
+torch is used for device memory and the current stream only; every function below ends in exactly
+one call into libglint_hip.so.  Names follow the reference's op names
+(models/common/ops/concept.hh, models/llama2/ops/concept.hh).
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional, Sequence
+
+import torch
+
+from . import _lib
+from ._lib import GH_ATTN_AUTO, GH_F16, GH_F32, Shape, check, lib
+
+
+def _dt(t: torch.Tensor) -> int:
+    if t.dtype == torch.float16:
+        return GH_F16
+    if t.dtype == torch.float32:
+        return GH_F32
+    raise TypeError(f"unsupported dtype {t.dtype}")
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _p(t: Optional[torch.Tensor]) -> Optional[int]:
+    if t is None:
+        return None
+    assert t.is_contiguous()
+    return t.data_ptr()
+
+
+def init(device: int = 0) -> None:
+    check(lib().gh_init(device), "gh_init")
+
+
+def device_name() -> str:
+    buf = C.create_string_buffer(128)
+    check(lib().gh_device_name(buf, 128), "gh_device_name")
+    return buf.value.decode()
+
+
+# ---- tables -------------------------------------------------------------------------------------
+def row_table(ptrs: Sequence[int], device="cuda") -> torch.Tensor:
+    """Device-resident table of row / layer base addresses (0 = empty context)."""
+    return torch.tensor([int(p) for p in ptrs], dtype=torch.int64, device=device)
+
+
+def host_ptr_array(ptrs: Sequence[int]):
+    arr = (C.c_void_p * max(1, len(ptrs)))()
+    for i, p in enumerate(ptrs):
+        arr[i] = p if p else None
+    return arr
+
+
+def host_u32_array(vals: Sequence[int]):
+    arr = (C.c_uint32 * max(1, len(vals)))()
+    for i, v in enumerate(vals):
+        arr[i] = int(v)
+    return arr
+
+
+# ---- common ops ---------------------------------------------------------------------------------
+def accum(a: torch.Tensor, b: torch.Tensor) -> None:
+    batch, size = a.shape
+    check(lib().gh_accum(_p(a), _p(b), size, batch, _dt(a), _stream()), "gh_accum")
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    batch, size = x.shape
+    out = torch.empty_like(x) if out is None else out
+    check(lib().gh_rmsnorm(_p(out), _p(x), _p(weight), size, batch, _dt(x), _stream()), "gh_rmsnorm")
+    return out
+
+
+def silu(hb: torch.Tensor, hb2: torch.Tensor) -> None:
+    batch, hidden = hb.shape
+    check(lib().gh_silu(_p(hb), _p(hb2), hidden, batch, _dt(hb), _stream()), "gh_silu")
+
+
+def argmax(v: torch.Tensor, to_host: bool = True):
+    batch, n = v.shape
+    out_dev = torch.empty(batch, dtype=torch.int32, device=v.device)
+    host = (C.c_uint32 * batch)() if to_host else None
+    check(lib().gh_argmax(host, _p(out_dev), _p(v), n, batch, _dt(v), _stream()), "gh_argmax")
+    return list(host) if to_host else out_dev
+
+
+def matmul(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    b, s = x.shape
+    r, s2 = w.shape
+    assert s == s2
+    out = torch.empty((b, r), dtype=x.dtype, device=x.device) if out is None else out
+    check(lib().gh_matmul(_p(out), _p(x), _p(w), s, r, b, _dt(x), _stream()), "gh_matmul")
+    return out
+
+
+def soft_sample(v: torch.Tensor, temperatures: Sequence[float], seed: int = 0) -> None:
+    batch, vocab = v.shape
+    temps = (C.c_float * batch)(*[float(t) for t in temperatures])
+    check(lib().gh_soft_sample(_p(v), temps, vocab, batch, seed, _dt(v), _stream()), "gh_soft_sample")
+
+
+def fill_normal(t: torch.Tensor, mean: float, std: float, seed: int) -> None:
+    check(lib().gh_fill_normal(_p(t), t.numel(), mean, std, seed, _dt(t), _stream()), "gh_fill_normal")
+
+
+def fill_uniform(t: torch.Tensor, lo: float, hi: float, seed: int) -> None:
+    check(lib().gh_fill_uniform(_p(t), t.numel(), lo, hi, seed, _dt(t), _stream()), "gh_fill_uniform")
+
+
+# ---- llama2 ops ---------------------------------------------------------------------------------
+def kv_append(token_rows: torch.Tensor, state_kv: torch.Tensor, kv_dim: int) -> None:
+    """token_rows: int64 device table of row addresses."""
+    batch = token_rows.numel()
+    check(lib().gh_kv_append(_p(token_rows), _p(state_kv), batch, kv_dim, _dt(state_kv), _stream()), "gh_kv_append")
+
+
+def kv_append_host(token_rows: Sequence[int], state_kv: torch.Tensor, kv_dim: int) -> None:
+    arr = host_ptr_array(token_rows)
+    check(lib().gh_kv_append_host(arr, _p(state_kv), len(token_rows), kv_dim, _dt(state_kv), _stream()),
+          "gh_kv_append_host")
+
+
+def rope(pos: torch.Tensor, freq_real: torch.Tensor, freq_imag: torch.Tensor, q: torch.Tensor,
+         token_rows: torch.Tensor, shape: Shape) -> None:
+    batch = token_rows.numel()
+    check(lib().gh_rope(batch, _p(pos), _p(freq_real), _p(freq_imag), _p(q), _p(token_rows),
+                        shape.n_kv_heads, shape.gqa_size, shape.head_size, _dt(q), _stream()), "gh_rope")
+
+
+def rope_host(pos: Sequence[int], freq_real: torch.Tensor, freq_imag: torch.Tensor, q: torch.Tensor,
+              token_rows: Sequence[int], shape: Shape) -> None:
+    check(lib().gh_rope_host(len(token_rows), host_u32_array(pos), _p(freq_real), _p(freq_imag), _p(q),
+                             host_ptr_array(token_rows), shape.n_kv_heads, shape.gqa_size, shape.head_size,
+                             _dt(q), _stream()), "gh_rope_host")
+
+
+def attn_scores(q, layer_rows: torch.Tensor, att, pos: torch.Tensor, shape: Shape) -> None:
+    s = shape.c()
+    check(lib().gh_attn_scores(_p(q), _p(layer_rows), _p(att), layer_rows.numel(), _p(pos), C.byref(s), _dt(q),
+                               _stream()), "gh_attn_scores")
+
+
+def attn_softmax(att, pos: torch.Tensor, shape: Shape) -> None:
+    s = shape.c()
+    check(lib().gh_attn_softmax(_p(att), _p(pos), pos.numel(), C.byref(s), _dt(att), _stream()), "gh_attn_softmax")
+
+
+def attn_pv(att, layer_rows: torch.Tensor, xb, pos: torch.Tensor, shape: Shape) -> None:
+    s = shape.c()
+    check(lib().gh_attn_pv(_p(att), _p(layer_rows), _p(xb), layer_rows.numel(), _p(pos), C.byref(s), _dt(att),
+                           _stream()), "gh_attn_pv")
+
+
+def attn_scores_host(q, layer_rows: Sequence[int], att, pos: Sequence[int], shape: Shape) -> None:
+    s = shape.c()
+    check(lib().gh_attn_scores_host(_p(q), host_ptr_array(layer_rows), _p(att), len(layer_rows), host_u32_array(pos),
+                                    C.byref(s), _dt(q), _stream()), "gh_attn_scores_host")
+
+
+def attn_softmax_host(att, pos: Sequence[int], shape: Shape) -> None:
+    s = shape.c()
+    check(lib().gh_attn_softmax_host(_p(att), host_u32_array(pos), len(pos), C.byref(s), _dt(att), _stream()),
+          "gh_attn_softmax_host")
+
+
+def attn_pv_host(att, layer_rows: Sequence[int], xb, pos: Sequence[int], shape: Shape) -> None:
+    s = shape.c()
+    check(lib().gh_attn_pv_host(_p(att), host_ptr_array(layer_rows), _p(xb), len(layer_rows), host_u32_array(pos),
+                                C.byref(s), _dt(att), _stream()), "gh_attn_pv_host")
+
+
+def attn_decode_workspace(batch: int, max_pos: int, shape: Shape) -> int:
+    s = shape.c()
+    return int(lib().gh_attn_decode_workspace(batch, max_pos, C.byref(s)))
+
+
+def attn_decode(q, layer_rows: torch.Tensor, pos: torch.Tensor, xb, max_pos: int, shape: Shape,
+                workspace: Optional[torch.Tensor] = None, variant: int = GH_ATTN_AUTO) -> None:
+    s = shape.c()
+    batch = layer_rows.numel()
+    if workspace is None:
+        workspace = torch.empty(attn_decode_workspace(batch, max_pos, shape), dtype=torch.uint8, device=q.device)
+    check(lib().gh_attn_decode(_p(q), _p(layer_rows), _p(pos), _p(xb), batch, max_pos, C.byref(s), _dt(q),
+                               _p(workspace), workspace.numel() * workspace.element_size(), variant, _stream()),
+          "gh_attn_decode")
+
+
+def attn_decode_host(q, layer_rows: Sequence[int], pos: Sequence[int], xb, shape: Shape,
+                     workspace: Optional[torch.Tensor] = None, variant: int = GH_ATTN_AUTO) -> None:
+    s = shape.c()
+    batch = len(layer_rows)
+    if workspace is None:
+        workspace = torch.empty(attn_decode_workspace(batch, shape.seq_len - 1, shape), dtype=torch.uint8,
+                                device=q.device)
+    check(lib().gh_attn_decode_host(_p(q), host_ptr_array(layer_rows), host_u32_array(pos), _p(xb), batch,
+                                    C.byref(s), _dt(q), _p(workspace), workspace.numel(), variant, _stream()),
+          "gh_attn_decode_host")
+
+
+def attn_set_chunk(tokens: int) -> None:
+    check(lib().gh_attn_set_chunk(tokens), "gh_attn_set_chunk")
+
+
+def sync() -> None:
+    check(lib().gh_sync(None), "gh_sync")

@@ -1,0 +1,202 @@
+/*
+ * glint_hip.h -- C-ABI of libglint_hip.so, the MI355X (gfx950) backend for Glinthawk's per-stage
+ * Llama2 KV-cache path.
+ *
+ * This is the boundary a `hip` target of the reference binds to: its C++ `Operations` /
+ * `LlamaOperations` / `Context` / `VirtualMemoryRegion` classes (glinthawk_amd/host/) are thin
+ * wrappers over these entry points, one per method of the reference's compile-time interface
+ * (models/common/ops/concept.hh:16-40, models/llama2/ops/concept.hh:15-36, models/llama2/context.hh:17-45).
+ * Each declaration cites the reference method it replaces (paths relative to the reference root).
+ *
+ * Conventions
+ *  - plain pointers and sizes only; no C++ or torch types.  Device pointers are raw HIP device
+ *    addresses, `gh_stream` is a `hipStream_t` (NULL = the default stream).
+ *  - every function returns GH_OK (0) or a negative gh_status; gh_last_error() gives the text for
+ *    the calling thread.  The reference aborts on any device error (arch/cuda/common/ops.cu:5-19);
+ *    the C++ wrappers do the same on a non-zero status.
+ *  - launches are asynchronous on `stream` unless stated; gh_sync() waits.
+ *  - "row" = one token's [K | V] = 2 * kv_dim elements, token-major inside a layer
+ *    (models/llama2/context.hh:61-133).  A NULL row / layer pointer is the reference's *empty*
+ *    context: that batch entry is skipped, exactly like the reference's ops do.
+ *  - ops that take per-context tables come in two forms: `*_host` receives HOST arrays of device
+ *    pointers / positions (what the reference's ops receive: models/llama2/base.hh:199-202) and
+ *    stages them itself; the plain form takes tables that already live in device memory (what the
+ *    stage driver and the benchmark use; one upload per step instead of one per op).
+ *  - nothing here falls back to the CPU: if no gfx950 device is present every call fails.
+ */
+#ifndef GLINT_HIP_H
+#define GLINT_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* gh_stream;
+
+/* values equal glinthawk::DataType (models/types.hh:19-24) */
+typedef enum gh_dtype
+{
+  GH_F16 = 0,
+  GH_F32 = 1,
+  GH_BF16 = 2 /* declared for wire compatibility; no kernel accepts it (the reference's amd64 bf16 is an alias of fp16, arch/float.hh:13) */
+} gh_dtype;
+
+/* values equal glinthawk::CopyType (models/types.hh:127-133) */
+typedef enum gh_copy_kind
+{
+  GH_HOST_TO_DEVICE = 0,
+  GH_DEVICE_TO_HOST = 1,
+  GH_DEVICE_TO_DEVICE = 2,
+  GH_HOST_TO_HOST = 3
+} gh_copy_kind;
+
+typedef enum gh_status
+{
+  GH_OK = 0,
+  GH_ERR_INVALID = -1,     /* bad argument / unsupported shape */
+  GH_ERR_DEVICE = -2,      /* a HIP call failed */
+  GH_ERR_NO_DEVICE = -3,   /* no gfx950 GPU visible */
+  GH_ERR_OOM = -4,
+  GH_ERR_WORKSPACE = -5    /* caller-provided workspace too small */
+} gh_status;
+
+/* Llama2 shape: the constants of models/llama2/variants.hh:9-32 as run-time values */
+typedef struct gh_shape
+{
+  uint32_t dim;
+  uint32_t kv_dim;
+  uint32_t hidden_dim;
+  uint32_t n_layers;
+  uint32_t head_size;
+  uint32_t n_heads;
+  uint32_t n_kv_heads;
+  uint32_t gqa_size;
+  uint32_t vocab_size;
+  uint32_t seq_len;
+} gh_shape;
+
+/* ---- runtime ------------------------------------------------------------------------------ */
+int gh_init( int device );              /* selects the device, checks it is gfx950, creates staging; idempotent */
+const char* gh_last_error( void );
+int gh_device_name( char* out, size_t len );
+int gh_sync( gh_stream stream );        /* hipStreamSynchronize (NULL: whole device) */
+
+/* Operations::device_allocate / DeviceUniquePtr deleter (arch/cuda/common/ops.cuh:27-35,748-756) */
+int gh_malloc( void** out, uint64_t bytes );
+int gh_free( void* ptr );
+/* pinned host memory for the staging buffers of a caller (hipHostMalloc) */
+int gh_host_malloc( void** out, uint64_t bytes );
+int gh_host_free( void* ptr );
+/* Operations::copy (arch/cuda/common/ops.cuh:758-780): byte copy; `async` != 0 returns before completion */
+int gh_memcpy( void* dst, const void* src, uint64_t bytes, gh_copy_kind kind, int async, gh_stream stream );
+int gh_memset_zero( void* dst, uint64_t bytes, gh_stream stream ); /* fill kernel, graph-capture safe */
+
+/* Operations::randomize_device_buffer (arch/cuda/common/ops.cuh:782-792): uniform [lo, hi), counter-based, seeded */
+int gh_fill_uniform( void* dst, uint64_t n, float lo, float hi, uint64_t seed, gh_dtype dt, gh_stream stream );
+/* synthetic inputs of the benchmark configs: N(mean, std) */
+int gh_fill_normal( void* dst, uint64_t n, float mean, float std, uint64_t seed, gh_dtype dt, gh_stream stream );
+
+/* LlamaOperations::convert_and_copy (arch/cuda/llama2/ops.cuh:455-492): n elements, static_cast per
+ * element; dst/src may each be host or device as `kind` says.  Synchronous (the reference's is). */
+int gh_convert_and_copy( void* dst, gh_dtype dst_dt, const void* src, gh_dtype src_dt, uint64_t n, gh_copy_kind kind );
+/* same conversion, device to device, asynchronous */
+int gh_convert( void* dst, gh_dtype dst_dt, const void* src, gh_dtype src_dt, uint64_t n, gh_stream stream );
+
+/* ---- paged KV arena: common::cuda::VirtualMemoryRegion (arch/cuda/common/vmem.cuh:22-160),
+ *      amd64 semantics in arch/amd64/common/vmem.hh:43-79 ---------------------------------- */
+typedef struct gh_vmm gh_vmm;
+int gh_vmm_granularity( uint64_t* out );                       /* minimum commit size of the device */
+int gh_vmm_reserve( gh_vmm** out, uint64_t bytes );            /* VirtualMemoryRegion(len): address range only */
+void* gh_vmm_ptr( const gh_vmm* r );                           /* ptr() */
+uint64_t gh_vmm_max_len( const gh_vmm* r );                    /* max_len() */
+int gh_vmm_commit( gh_vmm* r, uint64_t offset, uint64_t len ); /* allocate_span(ptr()+offset, len): out of range -> GH_ERR_INVALID */
+int gh_vmm_clear( gh_vmm* r );                                 /* clear(): unmap + release every committed span */
+uint64_t gh_vmm_committed_bytes( const gh_vmm* r );
+int gh_vmm_free( gh_vmm* r );
+
+/* ---- common ops: models/common/ops/concept.hh:28-39 --------------------------------------- */
+/* Operations::accum<size>    arch/amd64/common/ops.hh:124-137 : a = DType(float(a) + float(b)) over batch*size */
+int gh_accum( void* a, const void* b, uint64_t size, uint64_t batch, gh_dtype dt, gh_stream stream );
+/* Operations::rmsnorm<size>  arch/amd64/common/ops.hh:139-169 : eps 1e-5 after the mean; out may alias x */
+int gh_rmsnorm( void* out, const void* x, const void* weight, uint64_t size, uint64_t batch, gh_dtype dt, gh_stream stream );
+/* Operations::silu<hidden>   arch/amd64/common/ops.hh:194-210 : hb = DType(x / (1 + exp(-x)) * hb2) */
+int gh_silu( void* hb, const void* hb2, uint64_t hidden_dim, uint64_t batch, gh_dtype dt, gh_stream stream );
+/* Operations::argmax<n>      arch/amd64/common/ops.hh:171-192 : first index of the row maximum.
+ * `out_dev` (batch uint32, device) receives the indices; if `out_host` is non-NULL they are also
+ * copied there and the call synchronises (the reference writes a host array: arch/cuda/common/ops.cuh:646-650) */
+int gh_argmax( uint32_t* out_host, uint32_t* out_dev, const void* v, uint64_t n, uint64_t batch, gh_dtype dt, gh_stream stream );
+/* Operations::matmul<s,r> / untemplated_matmul  arch/amd64/common/ops.hh:74-93,212-271 :
+ * xout(b, r) = sum_p w(r, p) * x(b, p); w row-major (r, s); fp32 accumulate */
+int gh_matmul( void* xout, const void* x, const void* w, uint64_t s, uint64_t r, uint64_t b, gh_dtype dt, gh_stream stream );
+/* Operations::soft_sample    arch/amd64/common/ops.hh:97-107,273-283 : rows with temperature > 0 get
+ * v / T - log(-log(u)), u from a counter-based generator keyed by (seed, row, column).
+ * `temperatures` is a HOST array (batch floats), as in the reference. */
+int gh_soft_sample( void* v, const float* temperatures, uint64_t vocab, uint64_t batch, uint64_t seed, gh_dtype dt, gh_stream stream );
+
+/* ---- llama2 ops: models/llama2/ops/concept.hh:29-35 ---------------------------------------- */
+/* LlamaOperations::copy_kv_cache  arch/amd64/llama2/ops.hh:335-352 : row_i <- state_kv[i] (2*kv_dim elems), bit copy */
+int gh_kv_append( void* const* token_rows_dev, const void* state_kv, uint64_t batch, uint32_t kv_dim, gh_dtype dt, gh_stream stream );
+int gh_kv_append_host( void* const* token_rows_host, const void* state_kv, uint64_t batch, uint32_t kv_dim, gh_dtype dt, gh_stream stream );
+
+/* LlamaOperations::apply_rope  arch/amd64/llama2/ops.hh:138-164,300-333 : rotates the K half of each
+ * row in place and the query heads in `q` (batch, n_kv_heads*gqa*head_size); tables are (seq_len, head_size/2) */
+int gh_rope( uint64_t batch, const uint32_t* pos_dev, const void* freq_real, const void* freq_imag, void* q,
+             void* const* token_rows_dev, uint32_t n_kv_heads, uint32_t gqa_size, uint32_t head_size, gh_dtype dt, gh_stream stream );
+int gh_rope_host( uint64_t batch, const uint32_t* pos_host, const void* freq_real, const void* freq_imag, void* q,
+                  void* const* token_rows_host, uint32_t n_kv_heads, uint32_t gqa_size, uint32_t head_size, gh_dtype dt, gh_stream stream );
+
+/* LlamaOperations::attention_0_gemm  arch/amd64/llama2/ops.hh:170-223 : att (batch, n_heads, seq_len),
+ * entries [0, pos_i] written, the rest untouched */
+int gh_attn_scores( const void* q, const void* const* layer_rows_dev, void* att, uint64_t batch, const uint32_t* pos_dev,
+                    const gh_shape* shape, gh_dtype dt, gh_stream stream );
+int gh_attn_scores_host( const void* q, const void* const* layer_rows_host, void* att, uint64_t batch, const uint32_t* pos_host,
+                         const gh_shape* shape, gh_dtype dt, gh_stream stream );
+/* LlamaOperations::attention_softmax  arch/amd64/llama2/ops.hh:110-132,283-298 : over [0, pos_i] of every head row */
+int gh_attn_softmax( void* att, const uint32_t* pos_dev, uint64_t batch, const gh_shape* shape, gh_dtype dt, gh_stream stream );
+int gh_attn_softmax_host( void* att, const uint32_t* pos_host, uint64_t batch, const gh_shape* shape, gh_dtype dt, gh_stream stream );
+/* LlamaOperations::attention_2_gemm  arch/amd64/llama2/ops.hh:225-281 : xb (batch, dim) */
+int gh_attn_pv( const void* att, const void* const* layer_rows_dev, void* xb, uint64_t batch, const uint32_t* pos_dev,
+                const gh_shape* shape, gh_dtype dt, gh_stream stream );
+int gh_attn_pv_host( const void* att, const void* const* layer_rows_host, void* xb, uint64_t batch, const uint32_t* pos_host,
+                     const gh_shape* shape, gh_dtype dt, gh_stream stream );
+
+/* Fused decode attention = attention_0_gemm + attention_softmax + attention_2_gemm of
+ * Llama2::attention_ops (models/llama2/model.hh:354-387) without the `att` scratch: split-K over the
+ * cached rows with an online softmax, partial (max, sum, out) per split merged by a second kernel.
+ * q must already be rotated (gh_rope) and the current row appended (gh_kv_append).
+ *   layer_rows_dev[i]  base of context i's rows for this layer (NULL: skipped, xb row untouched)
+ *   pos_dev[i]         position of the current token; keys [0, pos_i] are attended
+ *   max_pos            host-side upper bound of pos (sizes the grid; seq_len - 1 if unknown)
+ *   workspace          device scratch of at least gh_attn_decode_workspace() bytes
+ *   variant            GH_ATTN_AUTO, or force a kernel (tests / measurements) */
+typedef enum gh_attn_variant
+{
+  GH_ATTN_AUTO = 0,
+  GH_ATTN_GENERIC = 1, /* any head_size <= 256, any gqa, f16 / f32 */
+  GH_ATTN_VALU = 2,    /* f16, head_size 128, wave-per-kv-head dot2/DPP kernel */
+  GH_ATTN_MFMA = 3     /* f16, head_size 128, gqa in [2, 16]: MFMA score / weighted-sum tiles */
+} gh_attn_variant;
+
+/* tokens per split of the fused kernel; 0 (default) lets the library choose from the batch shape */
+int gh_attn_set_chunk( uint32_t tokens_per_split );
+uint64_t gh_attn_decode_workspace( uint64_t batch, uint32_t max_pos, const gh_shape* shape );
+int gh_attn_decode( const void* q, const void* const* layer_rows_dev, const uint32_t* pos_dev, void* xb, uint64_t batch,
+                    uint32_t max_pos, const gh_shape* shape, gh_dtype dt, void* workspace, uint64_t workspace_bytes,
+                    int variant, gh_stream stream );
+int gh_attn_decode_host( const void* q, const void* const* layer_rows_host, const uint32_t* pos_host, void* xb, uint64_t batch,
+                         const gh_shape* shape, gh_dtype dt, void* workspace, uint64_t workspace_bytes, int variant, gh_stream stream );
+
+/* Timing hooks for the benchmark: HIP events recorded on `stream` around the attention kernels of
+ * gh_attn_decode (split + merge).  gh_attn_timing_read() synchronises and returns the accumulated
+ * kernel milliseconds and launch count since gh_attn_timing_reset(). */
+int gh_attn_timing_enable( int on );
+int gh_attn_timing_reset( void );
+int gh_attn_timing_read( double* total_ms, uint64_t* launches );
+
+#ifdef __cplusplus
+}
+#endif
+#endif

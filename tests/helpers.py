@@ -1,0 +1,59 @@
+"""Shared plumbing of the GPU parity tests: seeded inputs, KV arenas on the device with their
+address tables, and the error measures the tolerances are stated in."""
+from __future__ import annotations
+
+import numpy as np
+
+import oracle as O
+
+# north-star tolerances for attention outputs and logits against the fp32 CPU path
+MAX_ABS_TOL = 2e-2
+MEAN_REL_TOL = 1e-3
+
+
+def errors(got: np.ndarray, want: np.ndarray):
+    got = np.asarray(got, dtype=np.float64)
+    want = np.asarray(want, dtype=np.float64)
+    max_abs = float(np.max(np.abs(got - want))) if got.size else 0.0
+    denom = float(np.mean(np.abs(want))) if want.size else 1.0
+    mean_rel = float(np.mean(np.abs(got - want)) / max(denom, 1e-30)) if got.size else 0.0
+    return max_abs, mean_rel
+
+
+def assert_close(got, want, max_abs=MAX_ABS_TOL, mean_rel=MEAN_REL_TOL, what=""):
+    a, r = errors(got, want)
+    assert a <= max_abs and r <= mean_rel, f"{what}: max_abs {a:.3e} (tol {max_abs}), mean_rel {r:.3e} (tol {mean_rel})"
+
+
+def oracle_cfg(shape) -> O.Config:
+    return O.Config(dim=shape.dim, n_layers=shape.n_layers, n_heads=shape.n_heads, n_kv_heads=shape.n_kv_heads,
+                    hidden_dim=shape.hidden_dim, seq_len=shape.seq_len, vocab_size=shape.vocab_size)
+
+
+class Arena:
+    """`n_ctx` contexts x one layer of (seq_len, 2*kv_dim) rows in one device tensor, plus a host
+    (numpy) mirror for the oracle."""
+
+    def __init__(self, shape, n_ctx: int, dtype, seed: int, std: float = 1.0):
+        import torch
+        self.shape = shape
+        self.n_ctx = n_ctx
+        rng = np.random.default_rng(seed)
+        np_dt = np.float16 if dtype == torch.float16 else np.float32
+        self.host = (rng.standard_normal((n_ctx, shape.seq_len, 2 * shape.kv_dim)) * std).astype(np_dt)
+        self.dev = torch.from_numpy(self.host).cuda()
+        self.row_bytes = 2 * shape.kv_dim * self.dev.element_size()
+
+    def layer_ptr(self, i):
+        return self.dev.data_ptr() + i * self.shape.seq_len * self.row_bytes
+
+    def row_ptr(self, i, pos):
+        return self.layer_ptr(i) + pos * self.row_bytes
+
+    def host_layers_f32(self, present):
+        """fp32 copies (exact) of the host mirror for the oracle; None where the context is empty."""
+        return [np.ascontiguousarray(self.host[i].astype(np.float32)) if present[i] else None
+                for i in range(self.n_ctx)]
+
+    def refresh_host(self):
+        self.host = self.dev.cpu().numpy()

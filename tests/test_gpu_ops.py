@@ -1,0 +1,401 @@
+"""GPU parity tests, op by op, through the C-ABI against the CPU oracle on the same seeded inputs.
+
+Bit-exact: KV append.  Everything floating point: the north-star tolerance (2e-2 max-abs, 1e-3
+mean-relative) against the oracle's fp32 path, and tighter self-consistency bounds where stated."""
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from glinthawk_amd import Shape, ops
+from glinthawk_amd._lib import GH_ATTN_AUTO, GH_ATTN_GENERIC, GH_ATTN_MFMA, GH_ATTN_VALU, GlintError
+from helpers import Arena, assert_close, errors, oracle_cfg
+
+pytestmark = pytest.mark.gpu
+
+TINY = Shape(dim=32, n_layers=2, n_heads=4, n_kv_heads=2, hidden_dim=48, seq_len=16, vocab_size=64)
+STORIES = Shape(dim=288, n_layers=6, n_heads=6, n_kv_heads=6, hidden_dim=768, seq_len=256)      # config 1 shape
+MHA128 = Shape(dim=512, n_layers=1, n_heads=4, n_kv_heads=4, hidden_dim=64, seq_len=640)          # 7B-like heads
+MHA128_ODD = Shape(dim=768, n_layers=1, n_heads=6, n_kv_heads=6, hidden_dim=64, seq_len=300)      # kv heads % 4 != 0
+GQA8 = Shape(dim=2048, n_layers=1, n_heads=16, n_kv_heads=2, hidden_dim=64, seq_len=700)          # 70B-like heads
+GQA4 = Shape(dim=1536, n_layers=1, n_heads=12, n_kv_heads=3, hidden_dim=64, seq_len=330)
+GQA2 = Shape(dim=1024, n_layers=1, n_heads=8, n_kv_heads=4, hidden_dim=64, seq_len=280)
+GQA16 = Shape(dim=2048, n_layers=1, n_heads=16, n_kv_heads=1, hidden_dim=64, seq_len=300)
+
+
+def tdt(name):
+    return torch.float16 if name == "f16" else torch.float32
+
+
+def ndt(name):
+    return np.float16 if name == "f16" else np.float32
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _init():
+    ops.init(0)
+    assert ops.device_name().startswith("gfx950")
+    yield
+    ops.attn_set_chunk(0)
+
+
+# ------------------------------------------------------------------ elementwise
+@pytest.mark.parametrize("dt", ["f16", "f32"])
+@pytest.mark.parametrize("batch,size", [(1, 8), (3, 37), (4, 288), (64, 8192)])
+def test_accum(dt, batch, size):
+    rng = np.random.default_rng(1)
+    a = rng.standard_normal((batch, size)).astype(ndt(dt))
+    b = rng.standard_normal((batch, size)).astype(ndt(dt))
+    da, db = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()
+    ops.accum(da, db)
+    O.accum(a, b)
+    # one fp32 add and one rounding on both sides: identical bits
+    assert np.array_equal(da.cpu().numpy().view(np.uint8), a.view(np.uint8))
+
+
+@pytest.mark.parametrize("dt,tol", [("f16", 2e-3), ("f32", 2e-6)])
+@pytest.mark.parametrize("batch,size", [(1, 8), (4, 288), (5, 100), (64, 8192)])
+def test_rmsnorm(dt, tol, batch, size):
+    rng = np.random.default_rng(2)
+    x = rng.standard_normal((batch, size)).astype(ndt(dt))
+    w = (1 + 0.1 * rng.standard_normal(size)).astype(ndt(dt))
+    dx, dw = torch.from_numpy(x).cuda(), torch.from_numpy(w).cuda()
+    got = ops.rmsnorm(dx, dw).cpu().numpy()
+    want = O.rmsnorm(x, w)
+    np.testing.assert_allclose(got.astype(np.float64), want.astype(np.float64), rtol=tol, atol=tol)
+    want32 = O.rmsnorm(x.astype(np.float32), w.astype(np.float32))
+    assert_close(got, want32, what="rmsnorm vs fp32 path")
+    # in place
+    ops.rmsnorm(dx, dw, out=dx)
+    assert np.array_equal(dx.cpu().numpy(), got)
+
+
+@pytest.mark.parametrize("dt,tol", [("f16", 2e-3), ("f32", 3e-6)])
+@pytest.mark.parametrize("batch,hidden", [(1, 8), (4, 768), (3, 1001), (64, 28672)])
+def test_silu(dt, tol, batch, hidden):
+    rng = np.random.default_rng(3)
+    x = (2 * rng.standard_normal((batch, hidden))).astype(ndt(dt))
+    y = rng.standard_normal((batch, hidden)).astype(ndt(dt))
+    dx, dy = torch.from_numpy(x).cuda(), torch.from_numpy(y).cuda()
+    ops.silu(dx, dy)
+    O.silu(x, y)
+    np.testing.assert_allclose(dx.cpu().numpy().astype(np.float64), x.astype(np.float64), rtol=tol, atol=tol)
+
+
+@pytest.mark.parametrize("dt", ["f16", "f32"])
+def test_argmax_bit_exact(dt):
+    rng = np.random.default_rng(4)
+    v = rng.standard_normal((7, 32000)).astype(ndt(dt))
+    v[1, 17] = v[1, 20000] = 9.0     # tie across waves: first index
+    v[2, :] = 0.5                    # all equal
+    v[3, 31999] = 50.0
+    v[4, 0] = 50.0
+    v[5, 255] = v[5, 256] = 11.0     # tie across neighbouring threads
+    dv = torch.from_numpy(v).cuda()
+    got = ops.argmax(dv)
+    assert got == O.argmax(v).tolist()
+    small = rng.standard_normal((3, 5)).astype(ndt(dt))
+    assert ops.argmax(torch.from_numpy(small).cuda()) == O.argmax(small).tolist()
+
+
+def test_soft_sample_only_touches_warm_rows():
+    rng = np.random.default_rng(5)
+    v = rng.standard_normal((3, 1000)).astype(np.float32)
+    dv = torch.from_numpy(v).cuda()
+    ops.soft_sample(dv, [0.0, 0.7, 0.0], seed=9)
+    got = dv.cpu().numpy()
+    assert np.array_equal(got[0], v[0]) and np.array_equal(got[2], v[2])
+    # row 1 = v / T - log(-log(u)) for some u in (0,1): recover u and check its range and spread
+    noise = v[1].astype(np.float64) / 0.7 - got[1]
+    u = np.exp(-np.exp(noise))
+    assert np.all((u > 0) & (u < 1)) and 0.4 < u.mean() < 0.6
+    # greedy batches are a no-op
+    dv2 = torch.from_numpy(v).cuda()
+    ops.soft_sample(dv2, [0.0, 0.0, 0.0])
+    assert np.array_equal(dv2.cpu().numpy(), v)
+
+
+def test_fill_is_seeded_and_distributed():
+    t = torch.empty(1 << 20, dtype=torch.float16, device="cuda")
+    ops.fill_normal(t, 0.0, 1.0, seed=42)
+    a = t.float().cpu().numpy()
+    ops.fill_normal(t, 0.0, 1.0, seed=42)
+    assert np.array_equal(a, t.float().cpu().numpy())
+    ops.fill_normal(t, 0.0, 1.0, seed=43)
+    assert not np.array_equal(a, t.float().cpu().numpy())
+    assert abs(a.mean()) < 0.01 and abs(a.std() - 1) < 0.01
+    u = torch.empty(100003, dtype=torch.float32, device="cuda")
+    ops.fill_uniform(u, -2.0, 3.0, seed=1)
+    un = u.cpu().numpy()
+    assert un.min() >= -2.0 and un.max() <= 3.0 and abs(un.mean() - 0.5) < 0.05
+
+
+# ------------------------------------------------------------------ matmul
+@pytest.mark.parametrize("dt", ["f16", "f32"])
+@pytest.mark.parametrize("b,s,r", [(1, 8, 8), (4, 288, 288), (4, 288, 768), (3, 100, 37), (64, 1024, 512),
+                                   (5, 768, 1000), (70, 512, 130), (32, 4096, 256)])
+def test_matmul(dt, b, s, r):
+    rng = np.random.default_rng(6)
+    x = rng.standard_normal((b, s)).astype(ndt(dt))
+    w = (rng.standard_normal((r, s)) / np.sqrt(s)).astype(ndt(dt))
+    got = ops.matmul(torch.from_numpy(x).cuda(), torch.from_numpy(w).cuda()).cpu().numpy()
+    want = O.matmul(x.astype(np.float32), w.astype(np.float32))
+    assert got.shape == (b, r)
+    assert_close(got, want, what=f"matmul {dt} {b}x{s}x{r}")
+    if dt == "f32":
+        np.testing.assert_allclose(got, want, rtol=2e-5, atol=2e-5)
+
+
+def test_matmul_layout_one_hot():
+    s, r = 256, 192
+    w = torch.arange(r * s, dtype=torch.float32).reshape(r, s).remainder(1000).half().cuda()
+    x = torch.zeros((3, s), dtype=torch.float16, device="cuda")
+    x[0, 2] = x[1, 255] = x[2, 128] = 1
+    got = ops.matmul(x, w)
+    assert torch.equal(got[0], w[:, 2]) and torch.equal(got[1], w[:, 255]) and torch.equal(got[2], w[:, 128])
+
+
+# ------------------------------------------------------------------ KV append (bit exact)
+@pytest.mark.parametrize("dt", ["f16", "f32"])
+@pytest.mark.parametrize("shape", [TINY, STORIES, GQA8], ids=["tiny", "stories15m", "gqa8"])
+@pytest.mark.parametrize("host_tables", [False, True])
+def test_kv_append_bit_exact(dt, shape, host_tables):
+    batch = 5
+    arena = Arena(shape, batch, tdt(dt), seed=7)
+    rng = np.random.default_rng(8)
+    kv = rng.standard_normal((batch, 2 * shape.kv_dim)).astype(ndt(dt))
+    U = np.uint16 if dt == "f16" else np.uint32
+    kv.view(U)[0, 1] = 0x7e01 if dt == "f16" else 0x7fc00123      # NaN payload must survive
+    pos = [0, 3, shape.seq_len - 1, 7, 1]
+    present = [True, True, True, False, True]
+    rows = [arena.row_ptr(i, pos[i]) if present[i] else 0 for i in range(batch)]
+    dkv = torch.from_numpy(kv).cuda()
+    if host_tables:
+        ops.kv_append_host(rows, dkv, shape.kv_dim)
+    else:
+        ops.kv_append(ops.row_table(rows), dkv, shape.kv_dim)
+    want = arena.host.copy()
+    O.copy_kv_cache(oracle_cfg(shape), [want[i, pos[i]] if present[i] else None for i in range(batch)], kv)
+    got = arena.dev.cpu().numpy()
+    assert np.array_equal(got.view(U), want.view(U))
+
+
+# ------------------------------------------------------------------ RoPE
+@pytest.mark.parametrize("dt,tol", [("f16", 2e-3), ("f32", 3e-6)])
+@pytest.mark.parametrize("shape", [TINY, STORIES, GQA8, MHA128], ids=["tiny", "stories15m", "gqa8", "mha128"])
+@pytest.mark.parametrize("host_tables", [False, True])
+def test_rope(dt, tol, shape, host_tables):
+    batch = 4
+    arena = Arena(shape, batch, tdt(dt), seed=9)
+    re32, im32 = O.rope_tables(shape.seq_len, shape.head_size)
+    re, im = re32.astype(ndt(dt)), im32.astype(ndt(dt))
+    rng = np.random.default_rng(10)
+    q = rng.standard_normal((batch, shape.dim)).astype(ndt(dt))
+    pos = [0, 5, shape.seq_len - 1, 2]
+    present = [True, True, True, False]
+    rows = [arena.row_ptr(i, pos[i]) if present[i] else 0 for i in range(batch)]
+    dq = torch.from_numpy(q).cuda()
+    dre, dim_ = torch.from_numpy(re).cuda(), torch.from_numpy(im).cuda()
+    if host_tables:
+        ops.rope_host(pos, dre, dim_, dq, rows, shape)
+    else:
+        ops.rope(torch.tensor(pos, dtype=torch.int32, device="cuda"), dre, dim_, dq, ops.row_table(rows), shape)
+    want_cache = arena.host.copy()
+    O.apply_rope(oracle_cfg(shape), pos, re, im, q, [want_cache[i, pos[i]] if present[i] else None for i in range(batch)])
+    got_cache = arena.dev.cpu().numpy()
+    np.testing.assert_allclose(dq.cpu().numpy().astype(np.float64), q.astype(np.float64), rtol=tol, atol=tol)
+    np.testing.assert_allclose(got_cache.astype(np.float64), want_cache.astype(np.float64), rtol=tol, atol=tol)
+    # V halves and all other rows are untouched bit for bit
+    U = np.uint16 if dt == "f16" else np.uint32
+    mask = np.ones(got_cache.shape, bool)
+    for i in range(batch):
+        if present[i]:
+            mask[i, pos[i], : shape.kv_dim] = False
+    assert np.array_equal(got_cache.view(U)[mask], arena.host.view(U)[mask])
+
+
+# ------------------------------------------------------------------ unfused attention ops
+@pytest.mark.parametrize("dt", ["f16", "f32"])
+@pytest.mark.parametrize("shape", [TINY, STORIES, GQA8], ids=["tiny", "stories15m", "gqa8"])
+@pytest.mark.parametrize("host_tables", [False, True])
+def test_unfused_attention_ops(dt, shape, host_tables):
+    batch = 4
+    cfg = oracle_cfg(shape)
+    arena = Arena(shape, batch, tdt(dt), seed=11)
+    rng = np.random.default_rng(12)
+    q = rng.standard_normal((batch, shape.dim)).astype(ndt(dt))
+    pos = [0, min(37, shape.seq_len - 2), shape.seq_len - 1, 3]
+    present = [True, True, True, False]
+    layers = [arena.layer_ptr(i) if present[i] else 0 for i in range(batch)]
+    att0 = np.full((batch, shape.n_heads, shape.seq_len), 3.0, ndt(dt))
+    datt = torch.from_numpy(att0).cuda()
+    dq = torch.from_numpy(q).cuda()
+    dpos = torch.tensor(pos, dtype=torch.int32, device="cuda")
+    dxb = torch.full((batch, shape.dim), 5.0, dtype=tdt(dt), device="cuda")
+
+    host_layers = [arena.host[i] if present[i] else None for i in range(batch)]
+    att = att0.copy()
+    O.attention_0_gemm(cfg, q, host_layers, att, pos)
+    if host_tables:
+        ops.attn_scores_host(dq, layers, datt, pos, shape)
+    else:
+        ops.attn_scores(dq, ops.row_table(layers), datt, dpos, shape)
+    got = datt.cpu().numpy()
+    tol = 4e-3 if dt == "f16" else 2e-5
+    np.testing.assert_allclose(got.astype(np.float64), att.astype(np.float64), rtol=tol, atol=tol)
+    for i in range(batch):       # beyond pos and empty contexts: untouched
+        n = pos[i] + 1 if present[i] else 0
+        assert np.all(got[i, :, n:] == 3.0)
+
+    # softmax on identical inputs (the oracle's scores) so that only the softmax is compared
+    datt = torch.from_numpy(att).cuda()
+    O.attention_softmax(cfg, att, pos)
+    if host_tables:
+        ops.attn_softmax_host(datt, pos, shape)
+    else:
+        ops.attn_softmax(datt, dpos, shape)
+    got = datt.cpu().numpy()
+    tol = 2e-3 if dt == "f16" else 3e-6
+    for i in range(batch):
+        n = pos[i] + 1
+        np.testing.assert_allclose(got[i, :, :n].astype(np.float64), att[i, :, :n].astype(np.float64), rtol=tol, atol=tol)
+        assert np.array_equal(got[i, :, n:], att[i, :, n:])
+
+    datt = torch.from_numpy(att).cuda()
+    xb = np.full((batch, shape.dim), 5.0, ndt(dt))
+    O.attention_2_gemm(cfg, att, host_layers, xb, pos)
+    if host_tables:
+        ops.attn_pv_host(datt, layers, dxb, pos, shape)
+    else:
+        ops.attn_pv(datt, ops.row_table(layers), dxb, dpos, shape)
+    got = dxb.cpu().numpy()
+    tol = 3e-3 if dt == "f16" else 2e-5
+    np.testing.assert_allclose(got.astype(np.float64), xb.astype(np.float64), rtol=tol, atol=tol)
+    assert np.all(got[3] == 5.0)
+
+
+# ------------------------------------------------------------------ fused decode attention
+def run_fused_case(shape, dt, variant, pos, present, chunk, seed=13, host_tables=False, std=1.0):
+    batch = len(pos)
+    cfg = oracle_cfg(shape)
+    arena = Arena(shape, batch, tdt(dt), seed=seed, std=std)
+    rng = np.random.default_rng(seed + 1)
+    q = rng.standard_normal((batch, shape.dim)).astype(ndt(dt))
+    layers = [arena.layer_ptr(i) if present[i] else 0 for i in range(batch)]
+    dq = torch.from_numpy(q).cuda()
+    dxb = torch.full((batch, shape.dim), 5.0, dtype=tdt(dt), device="cuda")
+    ops.attn_set_chunk(chunk)
+    try:
+        if host_tables:
+            ops.attn_decode_host(dq, layers, pos, dxb, shape, variant=variant)
+        else:
+            max_pos = max([p for p, ok in zip(pos, present) if ok] + [0])
+            ops.attn_decode(dq, ops.row_table(layers), torch.tensor(pos, dtype=torch.int32, device="cuda"), dxb,
+                            max_pos, shape, variant=variant)
+        got = dxb.cpu().numpy()
+    finally:
+        ops.attn_set_chunk(0)
+
+    # oracle: the reference's fp32 CPU path on the same (exactly converted) inputs
+    q32 = q.astype(np.float32)
+    l32 = arena.host_layers_f32(present)
+    att = np.zeros((batch, shape.n_heads, shape.seq_len), np.float32)
+    xb = np.full((batch, shape.dim), 5.0, np.float32)
+    O.attention_0_gemm(cfg, q32, l32, att, pos)
+    O.attention_softmax(cfg, att, pos)
+    O.attention_2_gemm(cfg, att, l32, xb, pos)
+    live = [i for i in range(batch) if present[i]]
+    assert_close(got[live], xb[live], what=f"fused attention {dt} variant {variant} chunk {chunk}")
+    for i in range(batch):
+        if not present[i]:
+            assert np.all(got[i] == 5.0), "row of an empty context must stay untouched"
+    return got, xb
+
+
+RAGGED = [0, 1, 15, 16, 17, 63, 64, 255, 256, 257]
+
+
+@pytest.mark.parametrize("dt", ["f16", "f32"])
+@pytest.mark.parametrize("shape", [TINY, STORIES], ids=["tiny", "stories15m"])
+@pytest.mark.parametrize("chunk", [0, 16, 48])
+def test_fused_generic(dt, shape, chunk):
+    pos = [p for p in RAGGED if p < shape.seq_len] + [shape.seq_len - 1, 2]
+    present = [True] * (len(pos) - 1) + [False]
+    got, want = run_fused_case(shape, dt, GH_ATTN_GENERIC, pos, present, chunk)
+    if dt == "f32":
+        np.testing.assert_allclose(got[:-1], want[:-1], rtol=1e-4, atol=2e-5)
+
+
+@pytest.mark.parametrize("shape", [MHA128, MHA128_ODD, GQA2, GQA4, GQA8], ids=["mha", "mha6", "gqa2", "gqa4", "gqa8"])
+@pytest.mark.parametrize("chunk", [0, 16, 80, 256])
+def test_fused_valu(shape, chunk):
+    pos = [p for p in RAGGED if p < shape.seq_len] + [shape.seq_len - 1, 2]
+    present = [True] * (len(pos) - 1) + [False]
+    run_fused_case(shape, "f16", GH_ATTN_VALU, pos, present, chunk)
+
+
+@pytest.mark.parametrize("shape", [GQA2, GQA4, GQA8, GQA16], ids=["gqa2", "gqa4", "gqa8", "gqa16"])
+@pytest.mark.parametrize("chunk", [0, 16, 80, 256])
+def test_fused_mfma(shape, chunk):
+    pos = [p for p in RAGGED if p < shape.seq_len] + [shape.seq_len - 1, 2]
+    present = [True] * (len(pos) - 1) + [False]
+    run_fused_case(shape, "f16", GH_ATTN_MFMA, pos, present, chunk)
+
+
+@pytest.mark.parametrize("shape", [TINY, MHA128, GQA8], ids=["tiny", "mha", "gqa8"])
+def test_fused_auto_and_host_tables(shape):
+    pos = [0, 5, shape.seq_len - 1, shape.seq_len // 2]
+    run_fused_case(shape, "f16", GH_ATTN_AUTO, pos, [True, True, True, True], 0, host_tables=True)
+    run_fused_case(shape, "f16", GH_ATTN_AUTO, pos, [True, False, True, True], 32, host_tables=True)
+
+
+def test_fused_variants_agree():
+    # the three kernels on the same input: differences are rounding only
+    shape = GQA8
+    pos = [699, 300, 17]
+    outs = [run_fused_case(shape, "f16", v, pos, [True] * 3, 64, seed=21)[0]
+            for v in (GH_ATTN_GENERIC, GH_ATTN_VALU, GH_ATTN_MFMA)]
+    for o in outs[1:]:
+        a, r = errors(o, outs[0])
+        assert a < 4e-3 and r < 1e-3
+
+
+def test_fused_large_scores_are_stable():
+    # scores of magnitude ~ +-60 (std 6 K rows): exp() without the running max would overflow fp16/fp32 sums
+    run_fused_case(GQA8, "f16", GH_ATTN_MFMA, [699, 256], [True, True], 64, seed=31, std=6.0)
+    run_fused_case(MHA128, "f16", GH_ATTN_VALU, [639, 256], [True, True], 64, seed=32, std=6.0)
+
+
+def test_fused_properties_uniform_values_and_single_key():
+    shape = GQA8
+    batch = 3
+    arena = Arena(shape, batch, torch.float16, seed=41)
+    v = torch.randn(shape.kv_dim, dtype=torch.float16, device="cuda")
+    arena.dev[:, :, shape.kv_dim:] = v                     # every cached V row identical
+    q = torch.randn((batch, shape.dim), dtype=torch.float16, device="cuda")
+    pos = [0, 333, 699]
+    want = v.reshape(shape.n_kv_heads, 1, shape.head_size).expand(-1, shape.gqa_size, -1).reshape(-1).float()
+    for variant in (GH_ATTN_GENERIC, GH_ATTN_VALU, GH_ATTN_MFMA):
+        xb = torch.zeros((batch, shape.dim), dtype=torch.float16, device="cuda")
+        ops.attn_decode(q, ops.row_table([arena.layer_ptr(i) for i in range(batch)]),
+                        torch.tensor(pos, dtype=torch.int32, device="cuda"), xb, max(pos), shape, variant=variant)
+        assert torch.equal(xb[0].float(), want)            # one key: weight exactly 1
+        assert torch.allclose(xb.float(), want.expand(batch, -1), atol=2e-3, rtol=2e-3)
+
+
+def test_fused_rejects_bad_arguments():
+    shape = GQA8
+    q = torch.zeros((1, shape.dim), dtype=torch.float16, device="cuda")
+    xb = torch.zeros_like(q)
+    rows = ops.row_table([0])
+    pos = torch.zeros(1, dtype=torch.int32, device="cuda")
+    with pytest.raises(GlintError):
+        ops.attn_decode(q, rows, pos, xb, shape.seq_len, shape)            # max_pos outside seq_len
+    with pytest.raises(GlintError):
+        ops.attn_decode(q.float(), rows, pos, xb.float(), 5, shape, variant=GH_ATTN_MFMA)   # f32 on the f16 kernel
+    with pytest.raises(GlintError):                                         # workspace too small
+        ops.attn_set_chunk(16)
+        try:
+            ops.attn_decode(q, rows, pos, xb, 500, shape, workspace=torch.empty(64, dtype=torch.uint8, device="cuda"))
+        finally:
+            ops.attn_set_chunk(0)
