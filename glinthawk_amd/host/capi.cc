@@ -1,0 +1,386 @@
+// C entry points over the C++ host layer (libglint_host.so): a stage harness -- model driver +
+// context manager + one batched state -- for the benchmark and the tests, and host-only hooks that
+// exercise the slot bookkeeping and the paging rule without a GPU.
+#include <cstring>
+#include <deque>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "glint/contextman.hh"
+#include "glint/model.hh"
+
+using namespace glint;
+
+namespace {
+
+// ---------------------------------------------------------------------------------------------
+// type-erased stage harness
+// ---------------------------------------------------------------------------------------------
+struct StageBase
+{
+  virtual ~StageBase() = default;
+  virtual void set_layer_tensor( size_t layer, size_t k, const void* host, uint64_t n ) = 0;
+  virtual void set_base_tensor( size_t k, const void* host, uint64_t n ) = 0;
+  virtual void new_state( uint32_t batch, uint32_t next_layer, int next_stage ) = 0;
+  virtual void set_prompt( size_t i, uint32_t context_id, uint32_t token, uint32_t pos, float temp, uint32_t plen, uint32_t mcl ) = 0;
+  virtual void discard( size_t i ) = 0;
+  virtual int acquire_contexts() = 0;
+  virtual int forward( int which ) = 0;
+  virtual void* buffer( int which, uint64_t* bytes, bool allocate ) = 0;
+  virtual void row_info( size_t i, uint32_t out[6] ) = 0;
+  virtual void state_info( uint32_t out[4] ) = 0;
+  virtual void* context_layer_ptr( size_t row, size_t layer ) = 0;
+  virtual int32_t context_slot( size_t row ) = 0;
+  virtual void slot_counts( uint64_t out[3] ) = 0;
+  virtual void* scratch( int which ) = 0;
+  virtual int release_context( uint32_t id ) = 0;
+  virtual void paging_info( size_t row, size_t layer, uint64_t out[3] ) = 0;
+  virtual void sync() = 0;
+};
+
+template<typename Config, typename DType, typename Ctx>
+struct StageImpl : StageBase
+{
+  using Model = Llama2<Config, DType, hip::LlamaOperations<Config, DType, Ctx>, Ctx>;
+  using State = typename Model::StateType;
+
+  Model model;
+  PreallocatingContextManager<Model> contexts;
+  State state {};
+  typename Model::ContextVector held {};
+
+  StageImpl( const StageSettings<Config>& s, const ModelOptions& o )
+    : model( s, o )
+    , contexts( s )
+  {
+  }
+
+  void set_layer_tensor( size_t layer, size_t k, const void* host, uint64_t n ) override
+  {
+    model.set_layer_tensor( layer, k, static_cast<const DType*>( host ), n );
+  }
+  void set_base_tensor( size_t k, const void* host, uint64_t n ) override { model.set_base_tensor( k, static_cast<const DType*>( host ), n ); }
+
+  void new_state( uint32_t batch, uint32_t next_layer, int next_stage ) override
+  {
+    state = State( batch, dtype_of<DType>() );
+    state.set_next_layer( next_layer );
+    state.set_next_stage( static_cast<InferenceStage>( next_stage ) );
+    held.clear();
+  }
+  void set_prompt( size_t i, uint32_t context_id, uint32_t token, uint32_t pos, float temp, uint32_t plen, uint32_t mcl ) override
+  {
+    state.set_prompt( i, context_id, token, pos, temp, plen, mcl );
+  }
+  void discard( size_t i ) override { state.discard( i ); }
+
+  int acquire_contexts() override
+  {
+    auto got = contexts.get_contexts( state );
+    if ( !got.has_value() ) {
+      return -1; // not enough free slots: nothing was allocated
+    }
+    held = std::move( *got );
+    return 0;
+  }
+
+  // which: 0 forward (all hosted stages), 1 pre-attention, 2 attention, 3 post-attention, 4 classify
+  int forward( int which ) override
+  {
+    if ( which == 0 || which == 2 ) {
+      if ( acquire_contexts() != 0 ) {
+        return -1;
+      }
+    }
+    switch ( which ) {
+      case 0: model.forward( state, held ); break;
+      case 1: model.forward_pre_attention( state ); break;
+      case 2: model.forward_attention( state, held ); break;
+      case 3: model.forward_post_attention( state ); break;
+      case 4: model.forward_classify( state ); break;
+      default: return -2;
+    }
+    return 0;
+  }
+
+  // which: 0 activations, 1 queries, 2 kvs (host buffers of the state)
+  void* buffer( int which, uint64_t* bytes, bool allocate ) override
+  {
+    DataBuffer* b = which == 0 ? &state.activations() : which == 1 ? &state.queries() : &state.kvs();
+    if ( allocate && b->len() == 0 ) {
+      if ( which == 0 ) {
+        state.allocate_activations();
+      } else if ( which == 1 ) {
+        state.allocate_queries();
+      } else {
+        state.allocate_kvs();
+      }
+    }
+    *bytes = b->len();
+    return b->data();
+  }
+
+  void row_info( size_t i, uint32_t out[6] ) override
+  {
+    out[0] = state.active( i );
+    out[1] = state.context_id( i );
+    out[2] = state.token( i );
+    out[3] = state.token_pos( i );
+    out[4] = state.finished( i );
+    out[5] = static_cast<uint32_t>( state.temperature( i ) * 255.0f + 0.5f );
+  }
+  void state_info( uint32_t out[4] ) override
+  {
+    out[0] = state.batch_size();
+    out[1] = state.next_layer();
+    out[2] = static_cast<uint32_t>( state.next_stage() );
+    out[3] = ( state.has_activations() ? 1u : 0u ) | ( state.has_queries() ? 2u : 0u ) | ( state.has_kvs() ? 4u : 0u );
+  }
+
+  void* context_layer_ptr( size_t row, size_t layer ) override { return row < held.size() ? held[row]->layer( layer ).data() : nullptr; }
+  int32_t context_slot( size_t row ) override { return row < held.size() ? contexts.slot_index( held[row] ) : -2; }
+  void slot_counts( uint64_t out[3] ) override
+  {
+    out[0] = contexts.free();
+    out[1] = contexts.allocated();
+    out[2] = contexts.total();
+  }
+  int release_context( uint32_t id ) override { return contexts.release_context( id ) ? 1 : 0; }
+
+  void paging_info( size_t row, size_t layer, uint64_t out[3] ) override
+  {
+    out[0] = out[1] = out[2] = 0;
+    if constexpr ( requires( Ctx c ) { c.allocated_bytes( 0 ); } ) {
+      if ( row < held.size() ) {
+        out[0] = held[row]->allocated_bytes( layer );
+        out[1] = held[row]->blocks_committed();
+        out[2] = held[row]->clears();
+      }
+    }
+  }
+
+  // which: 0 x, 1 xb, 2 q, 3 kv, 4 logits
+  void* scratch( int which ) override
+  {
+    switch ( which ) {
+      case 0: return model.scratch_x();
+      case 1: return model.scratch_xb();
+      case 2: return model.scratch_q();
+      case 3: return model.scratch_kv();
+      default: return model.scratch_logits();
+    }
+  }
+  void sync() override { model.ops().synchronize(); }
+};
+
+template<typename Config>
+StageBase* make_for_config( int dtype, bool paged, const StageSettings<Config>& s, const ModelOptions& o )
+{
+  if ( dtype == 0 ) {
+    if ( paged ) {
+      return new StageImpl<Config, float16_t, hip::DynamicContext<Config, float16_t>>( s, o );
+    }
+    return new StageImpl<Config, float16_t, hip::Context<Config, float16_t>>( s, o );
+  }
+  if ( paged ) {
+    return new StageImpl<Config, float32_t, hip::DynamicContext<Config, float32_t>>( s, o );
+  }
+  return new StageImpl<Config, float32_t, hip::Context<Config, float32_t>>( s, o );
+}
+
+template<typename Config>
+StageBase* make_stage( int dtype, uint32_t first_layer, uint32_t n_hosted, uint32_t concurrency, uint32_t max_contexts, uint32_t flags, uint64_t seed, float std )
+{
+  const bool with_cls = flags & 2u;
+  auto s = StageSettings<Config>::slice( first_layer, n_hosted, concurrency, max_contexts, with_cls );
+  ModelOptions o;
+  o.fused_attention = flags & 1u;
+  o.seed = seed;
+  o.weight_std = std;
+  return make_for_config<Config>( dtype, flags & 4u, s, o );
+}
+
+// ---------------------------------------------------------------------------------------------
+// host-only stand-ins for the bookkeeping tests (no device memory involved)
+// ---------------------------------------------------------------------------------------------
+struct CountingRegion // VirtualMemoryRegion surface without memory: records what would be committed
+{
+  size_t len_;
+  std::vector<std::pair<size_t, size_t>> spans_ {};
+  size_t clears_ { 0 };
+  explicit CountingRegion( size_t len )
+    : len_( len )
+  {
+  }
+  void allocate_span( const void* ptr, size_t len )
+  {
+    const size_t off = reinterpret_cast<uintptr_t>( ptr ) - reinterpret_cast<uintptr_t>( this->ptr() );
+    GLINT_CHECK( off + len <= len_ );
+    spans_.emplace_back( off, len );
+  }
+  void* ptr() const { return reinterpret_cast<void*>( uintptr_t { 1 } << 40 ); } // fake, never dereferenced
+  size_t max_len() const { return len_; }
+  void clear()
+  {
+    spans_.clear();
+    clears_++;
+  }
+};
+
+using BookConfig = configs::Llama2_70B_Chat_4K;
+
+struct HostOnlyContext : glint::Context<BookConfig, float16_t>
+{
+  HostOnlyContext() = default;
+  template<typename Settings>
+  explicit HostOnlyContext( const Settings& s, bool make_empty = false )
+  {
+    this->set_buffer( s, make_empty ? nullptr : reinterpret_cast<float16_t*>( uintptr_t { 1 } << 40 ) );
+  }
+};
+
+struct BookModel
+{
+  using ConfigType = BookConfig;
+  using ContextType = HostOnlyContext;
+  using SettingsType = StageSettings<BookConfig>;
+};
+
+struct BookManager
+{
+  PreallocatingContextManager<BookModel> man;
+  explicit BookManager( uint64_t n )
+    : man( StageSettings<BookConfig>::slice( 0, 1, 1024, n ) )
+  {
+  }
+};
+
+using PagedBookContext = glint::DynamicContext<BookConfig, float16_t, CountingRegion>;
+
+} // namespace
+
+extern "C" {
+
+// ---- stage harness --------------------------------------------------------------------------
+// flags: 1 fused attention, 2 host the classifier, 4 paged (virtual-memory) contexts
+void* glint_stage_create( const char* config, int dtype, uint32_t first_layer, uint32_t n_hosted, uint32_t concurrency, uint32_t max_contexts,
+                          uint32_t flags, uint64_t seed, float weight_std )
+{
+  const std::string name( config );
+#define GLINT_CASE( NAME, CFG )                                                                                        \
+  if ( name == NAME ) {                                                                                                \
+    return make_stage<configs::CFG>( dtype, first_layer, n_hosted, concurrency, max_contexts, flags, seed, weight_std ); \
+  }
+  GLINT_CASE( "llama2-70b-4k", Llama2_70B_Chat_4K )
+  GLINT_CASE( "llama2-70b-8k", Llama2_70B_Chat_8K )
+  GLINT_CASE( "llama2-13b-4k", Llama2_13B_Chat_4K )
+  GLINT_CASE( "llama2-7b", Llama2_7B_Chat )
+  GLINT_CASE( "stories15m", Stories_15M )
+  GLINT_CASE( "test-gqa4", Test_GQA4 )
+  GLINT_CASE( "test-mha", Test_MHA )
+  GLINT_CASE( "test-tiny", Test_Tiny )
+#undef GLINT_CASE
+  return nullptr;
+}
+
+void glint_stage_destroy( void* h ) { delete static_cast<StageBase*>( h ); }
+void glint_stage_set_layer_tensor( void* h, uint32_t layer, uint32_t k, const void* host, uint64_t n ) { static_cast<StageBase*>( h )->set_layer_tensor( layer, k, host, n ); }
+void glint_stage_set_base_tensor( void* h, uint32_t k, const void* host, uint64_t n ) { static_cast<StageBase*>( h )->set_base_tensor( k, host, n ); }
+void glint_stage_new_state( void* h, uint32_t batch, uint32_t next_layer, int next_stage ) { static_cast<StageBase*>( h )->new_state( batch, next_layer, next_stage ); }
+void glint_stage_set_prompt( void* h, uint32_t row, uint32_t context_id, uint32_t token, uint32_t pos, float temperature, uint32_t prompt_length,
+                             uint32_t max_completion_length )
+{
+  static_cast<StageBase*>( h )->set_prompt( row, context_id, token, pos, temperature, prompt_length, max_completion_length );
+}
+void glint_stage_discard( void* h, uint32_t row ) { static_cast<StageBase*>( h )->discard( row ); }
+int glint_stage_acquire_contexts( void* h ) { return static_cast<StageBase*>( h )->acquire_contexts(); }
+int glint_stage_forward( void* h, int which ) { return static_cast<StageBase*>( h )->forward( which ); }
+void* glint_stage_buffer( void* h, int which, uint64_t* bytes, int allocate ) { return static_cast<StageBase*>( h )->buffer( which, bytes, allocate != 0 ); }
+void glint_stage_row_info( void* h, uint32_t row, uint32_t out[6] ) { static_cast<StageBase*>( h )->row_info( row, out ); }
+void glint_stage_state_info( void* h, uint32_t out[4] ) { static_cast<StageBase*>( h )->state_info( out ); }
+void* glint_stage_context_layer_ptr( void* h, uint32_t row, uint32_t layer ) { return static_cast<StageBase*>( h )->context_layer_ptr( row, layer ); }
+int32_t glint_stage_context_slot( void* h, uint32_t row ) { return static_cast<StageBase*>( h )->context_slot( row ); }
+void glint_stage_slot_counts( void* h, uint64_t out[3] ) { static_cast<StageBase*>( h )->slot_counts( out ); }
+int glint_stage_release_context( void* h, uint32_t id ) { return static_cast<StageBase*>( h )->release_context( id ); }
+void glint_stage_paging_info( void* h, uint32_t row, uint32_t layer, uint64_t out[3] ) { static_cast<StageBase*>( h )->paging_info( row, layer, out ); }
+void* glint_stage_scratch( void* h, int which ) { return static_cast<StageBase*>( h )->scratch( which ); }
+void glint_stage_sync( void* h ) { static_cast<StageBase*>( h )->sync(); }
+
+// ---- host-only bookkeeping hooks ---------------------------------------------------------------
+void* glint_book_manager_new( uint64_t max_context_count ) { return new BookManager( max_context_count ); }
+void glint_book_manager_delete( void* m ) { delete static_cast<BookManager*>( m ); }
+uint64_t glint_book_manager_free( void* m ) { return static_cast<BookManager*>( m )->man.free(); }
+uint64_t glint_book_manager_allocated( void* m ) { return static_cast<BookManager*>( m )->man.allocated(); }
+
+// rows [start, end) of a state described by active[] / context_id[]; slots_out gets creation indices (-1 = empty context)
+int glint_book_manager_get_contexts( void* m, const uint8_t* active, const uint32_t* context_id, uint64_t batch, uint64_t start, uint64_t end, int32_t* slots_out )
+{
+  auto& man = static_cast<BookManager*>( m )->man;
+  BatchedInferenceState<BookConfig> st( static_cast<uint32_t>( batch ), DataType::Float16 );
+  for ( uint64_t i = 0; i < batch; i++ ) {
+    if ( active[i] ) {
+      st.set_prompt( i, context_id[i], 1, 0, 0.0f, 1, 0 );
+    } else {
+      st.set_context_id( i, context_id[i] );
+    }
+  }
+  auto got = man.get_contexts( st, start, end );
+  if ( !got.has_value() ) {
+    return 0;
+  }
+  for ( size_t k = 0; k < got->size(); k++ ) {
+    slots_out[k] = man.slot_index( ( *got )[k] );
+  }
+  return 1;
+}
+
+int32_t glint_book_manager_get_context( void* m, uint32_t context_id )
+{
+  auto& man = static_cast<BookManager*>( m )->man;
+  auto ctx = man.get_context( context_id );
+  return ctx ? man.slot_index( ctx ) : -1;
+}
+
+int glint_book_manager_release( void* m, uint32_t context_id ) { return static_cast<BookManager*>( m )->man.release_context( context_id ) ? 1 : 0; }
+
+// paged context over a counting region: hosts `n_hosted` layers of the 70B-4K shape
+void* glint_book_paged_new( uint32_t n_hosted ) { return new PagedBookContext( StageSettings<BookConfig>::slice( 0, n_hosted, 1, 1 ) ); }
+void glint_book_paged_delete( void* c ) { delete static_cast<PagedBookContext*>( c ); }
+// returns the committed bytes of `layer` after the call; out[0] = blocks committed so far, out[1] = clears so far
+uint64_t glint_book_paged_prepare( void* c, uint32_t layer, uint32_t token_pos, int can_release, uint64_t out[2] )
+{
+  auto* ctx = static_cast<PagedBookContext*>( c );
+  GLINT_CHECK( ctx->prepare( layer, token_pos, can_release != 0 ) );
+  out[0] = ctx->blocks_committed();
+  out[1] = ctx->clears();
+  return ctx->allocated_bytes( layer );
+}
+
+// KV addressing of the host layer, in elements from the context base (UINT64_MAX: layer not hosted)
+uint64_t glint_book_key_head_offset( const uint8_t* hosted, uint32_t layer, uint32_t pos, uint32_t head, int value )
+{
+  StageSettings<BookConfig>::HostingTable t {};
+  for ( size_t l = 0; l < BookConfig::n_layers; l++ ) {
+    t[l][static_cast<size_t>( InferenceStage::Attention )] = hosted[l] != 0;
+    t[l][0] = t[l][0] || hosted[l] != 0;
+  }
+  bool any = false;
+  for ( size_t l = 0; l < BookConfig::n_layers; l++ ) {
+    any = any || hosted[l];
+  }
+  if ( !any ) {
+    return UINT64_MAX;
+  }
+  StageSettings<BookConfig> s( t, 1, 1 );
+  auto* base = reinterpret_cast<float16_t*>( uintptr_t { 1 } << 40 );
+  glint::Context<BookConfig, float16_t> ctx( s, base );
+  auto lc = ctx.layer( layer );
+  if ( lc.empty() ) {
+    return UINT64_MAX;
+  }
+  auto tc = lc.token( pos );
+  return static_cast<uint64_t>( ( value ? tc.value_head( head ) : tc.key_head( head ) ) - base );
+}
+
+} // extern "C"

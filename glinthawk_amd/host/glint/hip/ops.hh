@@ -1,0 +1,316 @@
+// The `hip` target: Operations<DType> and LlamaOperations<Config, DType, Ctx>, the two classes a
+// Glinthawk backend provides (models/common/ops/concept.hh:16-40, models/llama2/ops/concept.hh:15-42),
+// with the method names, argument order and meaning of the amd64 / cuda targets
+// (arch/amd64/common/ops.hh:13-63, arch/amd64/llama2/ops.hh:23-68).  Every method is one call into
+// libglint_hip.so; a non-zero status aborts, as every device error does in the reference.
+#pragma once
+
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "glint/config.hh"
+#include "glint/context.hh"
+#include "glint/types.hh"
+#include "glint_hip.h"
+
+namespace glint::hip {
+
+#define GLINT_GH( call )                                                                                               \
+  do {                                                                                                                 \
+    if ( ( call ) != GH_OK ) {                                                                                         \
+      ::glint::fatal( __FILE__, __LINE__, #call, gh_last_error() );                                                    \
+    }                                                                                                                  \
+  } while ( 0 )
+
+template<typename DType>
+constexpr gh_dtype gh_type()
+{
+  return sizeof( DType ) == 2 ? GH_F16 : GH_F32;
+}
+
+inline gh_copy_kind gh_kind( const CopyType t )
+{
+  switch ( t ) {
+    case CopyType::HostToDevice: return GH_HOST_TO_DEVICE;
+    case CopyType::DeviceToHost: return GH_DEVICE_TO_HOST;
+    case CopyType::DeviceToDevice: return GH_DEVICE_TO_DEVICE;
+    default: return GH_HOST_TO_HOST;
+  }
+}
+
+template<typename PtrType>
+struct DeviceDeleter
+{
+  void operator()( PtrType* ptr ) const
+  {
+    if ( ptr ) {
+      GLINT_GH( gh_free( ptr ) );
+    }
+  }
+};
+
+template<typename DType>
+class Operations
+{
+public:
+  using DeviceUniquePtr = std::unique_ptr<DType, DeviceDeleter<DType>>;
+
+  Operations() { GLINT_GH( gh_init( 0 ) ); }
+  ~Operations() = default;
+  Operations( const Operations& ) = delete;
+  Operations& operator=( const Operations& ) = delete;
+  Operations( Operations&& ) = default;
+  Operations& operator=( Operations&& ) = default;
+
+  // all work is queued on this stream (NULL = the default stream)
+  void set_stream( gh_stream s ) { stream_ = s; }
+  gh_stream stream() const { return stream_; }
+  void synchronize() const { GLINT_GH( gh_sync( stream_ ) ); }
+
+  template<uint64_t size>
+  void accum( DType* a, const DType* b, const uint64_t batch_size ) const
+  {
+    GLINT_GH( gh_accum( a, b, size, batch_size, gh_type<DType>(), stream_ ) );
+  }
+
+  // `temp` is unused: the kernel reduces in registers / LDS
+  template<uint64_t size>
+  void rmsnorm( DType* o, const DType* x, float32_t*, const DType* weight, const uint64_t batch_size ) const
+  {
+    GLINT_GH( gh_rmsnorm( o, x, weight, size, batch_size, gh_type<DType>(), stream_ ) );
+  }
+
+  // `output` is a HOST array (ScratchPad::argmax_pos); `temp` is device scratch with room for batch_size uint32
+  template<uint64_t n>
+  void argmax( uint32_t* output, const DType* v, DType* temp, const uint64_t batch_size ) const
+  {
+    GLINT_GH( gh_argmax( output, reinterpret_cast<uint32_t*>( temp ), v, n, batch_size, gh_type<DType>(), stream_ ) );
+  }
+
+  template<uint64_t hidden_dim>
+  void silu( DType* hb, DType* hb2, const uint64_t batch_size ) const
+  {
+    GLINT_GH( gh_silu( hb, hb2, hidden_dim, batch_size, gh_type<DType>(), stream_ ) );
+  }
+
+  template<uint64_t s, uint64_t r>
+  void matmul( DType* xo, const DType* x, const DType* w, const uint64_t b ) const
+  {
+    GLINT_GH( gh_matmul( xo, x, w, s, r, b, gh_type<DType>(), stream_ ) );
+  }
+
+  void untemplated_matmul( DType* xo, const DType* x, const DType* w, const uint64_t s, const uint64_t r, const uint64_t b ) const
+  {
+    GLINT_GH( gh_matmul( xo, x, w, s, r, b, gh_type<DType>(), stream_ ) );
+  }
+
+  void soft_sample( DType* v, const std::vector<float>& temperatures, const size_t vocab_size ) const
+  {
+    GLINT_GH( gh_soft_sample( v, temperatures.data(), vocab_size, temperatures.size(), sample_seed_++, gh_type<DType>(), stream_ ) );
+  }
+
+  DeviceUniquePtr device_allocate( const uint64_t size_bytes ) const
+  {
+    void* p = nullptr;
+    GLINT_GH( gh_malloc( &p, size_bytes ) );
+    return DeviceUniquePtr { static_cast<DType*>( p ) };
+  }
+
+  void randomize_device_buffer( DType* buffer, const uint64_t len, const float min, const float max ) const
+  {
+    GLINT_GH( gh_fill_uniform( buffer, len, min, max, fill_seed_++, gh_type<DType>(), stream_ ) );
+  }
+
+  void copy( DType* dst, const DType* src, const uint64_t len_bytes, const CopyType type, const bool async = false ) const
+  {
+    GLINT_GH( gh_memcpy( dst, src, len_bytes, gh_kind( type ), async ? 1 : 0, stream_ ) );
+  }
+
+  void print( const DType* x, const uint64_t b, const std::string base ) const
+  {
+    std::vector<DType> host( b );
+    GLINT_GH( gh_memcpy( host.data(), x, b * sizeof( DType ), GH_DEVICE_TO_HOST, 0, stream_ ) );
+    std::printf( "%s", base.c_str() );
+    for ( uint64_t i = 0; i < b; i++ ) {
+      std::printf( "\t%.10f", static_cast<float>( host[i] ) );
+    }
+    std::printf( "\n" );
+  }
+
+protected:
+  gh_stream stream_ { nullptr };
+  mutable uint64_t sample_seed_ { 0x5eed };
+  mutable uint64_t fill_seed_ { 0xf111 };
+};
+
+// platform-specific context: storage is one device allocation owned by the context
+// (arch/cuda/llama2/ops.cuh:66-76,108-126)
+template<typename Config, typename DType>
+class Context : public glint::Context<Config, DType>
+{
+  typename Operations<DType>::DeviceUniquePtr storage_ {};
+
+public:
+  Context() = default;
+
+  template<typename Settings>
+  explicit Context( const Settings& settings, const bool make_empty = false )
+  {
+    DType* ptr = nullptr;
+    if ( !make_empty ) {
+      void* p = nullptr;
+      GLINT_GH( gh_malloc( &p, glint::Context<Config, DType>::max_size( settings.num_attention_layers_hosted() ) ) );
+      ptr = static_cast<DType*>( p );
+    }
+    storage_.reset( ptr );
+    this->set_buffer( settings, ptr );
+  }
+};
+
+// common::hip::VirtualMemoryRegion: address-space reservation with 2 MiB commits
+// (arch/cuda/common/vmem.cuh:60-160, arch/amd64/common/vmem.hh:43-79)
+class VirtualMemoryRegion
+{
+  gh_vmm* region_ { nullptr };
+
+public:
+  explicit VirtualMemoryRegion( const size_t len ) { GLINT_GH( gh_vmm_reserve( &region_, len ) ); }
+  ~VirtualMemoryRegion()
+  {
+    if ( region_ ) {
+      GLINT_GH( gh_vmm_free( region_ ) );
+    }
+  }
+  VirtualMemoryRegion( const VirtualMemoryRegion& ) = delete;
+  VirtualMemoryRegion& operator=( const VirtualMemoryRegion& ) = delete;
+  VirtualMemoryRegion( VirtualMemoryRegion&& other ) noexcept
+    : region_( other.region_ )
+  {
+    other.region_ = nullptr;
+  }
+  VirtualMemoryRegion& operator=( VirtualMemoryRegion&& other ) noexcept
+  {
+    std::swap( region_, other.region_ );
+    return *this;
+  }
+
+  // out-of-range spans abort ("Out of bounds allocation" in the reference)
+  void allocate_span( const void* ptr, const size_t len )
+  {
+    const auto offset = static_cast<uint64_t>( static_cast<const uint8_t*>( ptr ) - static_cast<const uint8_t*>( this->ptr() ) );
+    GLINT_GH( gh_vmm_commit( region_, offset, len ) );
+  }
+
+  void* ptr() const { return gh_vmm_ptr( region_ ); }
+  size_t max_len() const { return gh_vmm_max_len( region_ ); }
+  size_t committed() const { return gh_vmm_committed_bytes( region_ ); }
+  void clear() { GLINT_GH( gh_vmm_clear( region_ ) ); }
+};
+
+template<typename Config, typename DType>
+using DynamicContext = glint::DynamicContext<Config, DType, VirtualMemoryRegion>;
+
+template<typename Config, typename DType, typename Ctx = Context<Config, DType>>
+requires ModelConfig<Config> && ContextConcept<Ctx, DType>
+class LlamaOperations : public Operations<DType>
+{
+public:
+  using typename Operations<DType>::DeviceUniquePtr;
+  using ContextType = Ctx;
+
+  template<typename Settings>
+  explicit LlamaOperations( const Settings& )
+  {
+  }
+  ~LlamaOperations() = default;
+
+  static gh_shape shape()
+  {
+    return gh_shape { (uint32_t)Config::dim,     (uint32_t)Config::kv_dim,     (uint32_t)Config::hidden_dim, (uint32_t)Config::n_layers,
+                      (uint32_t)Config::head_size, (uint32_t)Config::n_heads,  (uint32_t)Config::n_kv_heads, (uint32_t)Config::gqa_size,
+                      (uint32_t)Config::vocab_size, (uint32_t)Config::seq_len };
+  }
+
+  // `layer_contexts` / `token_contexts` / `token_positions` are HOST arrays (ScratchPad members,
+  // models/llama2/base.hh:199-202) holding device addresses; the library stages them.
+  void attention_0_gemm( const DType* query,
+                         const typename ContextType::LayerContextType layer_contexts[],
+                         DType* att,
+                         const uint64_t batch_size,
+                         const uint32_t* token_positions ) const
+  {
+    const gh_shape s = shape();
+    GLINT_GH( gh_attn_scores_host( query, layer_table( layer_contexts, batch_size ), att, batch_size, token_positions, &s, gh_type<DType>(), this->stream_ ) );
+  }
+
+  void attention_2_gemm( const DType* att,
+                         const typename ContextType::LayerContextType layer_contexts[],
+                         DType* xb,
+                         const uint64_t batch_size,
+                         const uint32_t* token_positions ) const
+  {
+    const gh_shape s = shape();
+    GLINT_GH( gh_attn_pv_host( att, layer_table( layer_contexts, batch_size ), xb, batch_size, token_positions, &s, gh_type<DType>(), this->stream_ ) );
+  }
+
+  void attention_softmax( DType* att, const uint32_t* token_positions, DType*, const uint64_t batch_size ) const
+  {
+    const gh_shape s = shape();
+    GLINT_GH( gh_attn_softmax_host( att, token_positions, batch_size, &s, gh_type<DType>(), this->stream_ ) );
+  }
+
+  void apply_rope( const uint64_t batch_size,
+                   const uint32_t* token_positions,
+                   const DType* freq_cis_real,
+                   const DType* freq_cis_imag,
+                   DType* state_q,
+                   typename ContextType::TokenContextType token_contexts[] ) const
+  {
+    GLINT_GH( gh_rope_host( batch_size, token_positions, freq_cis_real, freq_cis_imag, state_q, token_table( token_contexts, batch_size ),
+                            Config::n_kv_heads, Config::gqa_size, Config::head_size, gh_type<DType>(), this->stream_ ) );
+  }
+
+  void copy_kv_cache( typename ContextType::TokenContextType token_contexts[], const DType* state_kv, const uint64_t batch_size ) const
+  {
+    GLINT_GH( gh_kv_append_host( token_table( token_contexts, batch_size ), state_kv, batch_size, Config::kv_dim, gh_type<DType>(), this->stream_ ) );
+  }
+
+  template<typename DTypeDst, typename DTypeSrc>
+  void convert_and_copy( DTypeDst* dst, const DTypeSrc* src, const uint64_t size, const CopyType type ) const
+  {
+    GLINT_GH( gh_convert_and_copy( dst, gh_type<DTypeDst>(), src, gh_type<DTypeSrc>(), size, gh_kind( type ) ) );
+  }
+
+  // Extension used by the stage driver: attention_0_gemm + attention_softmax + attention_2_gemm in
+  // one fused split-K kernel without the `att` buffer.  Tables live in device memory.
+  void attention_fused( const DType* query,
+                        const void* const* layer_rows_dev,
+                        const uint32_t* token_positions_dev,
+                        DType* xb,
+                        const uint64_t batch_size,
+                        const uint32_t max_pos,
+                        void* workspace,
+                        const uint64_t workspace_bytes ) const
+  {
+    const gh_shape s = shape();
+    GLINT_GH( gh_attn_decode( query, layer_rows_dev, token_positions_dev, xb, batch_size, max_pos, &s, gh_type<DType>(), workspace, workspace_bytes,
+                              GH_ATTN_AUTO, this->stream_ ) );
+  }
+
+private:
+  // TokenContext / LayerContext are a single pointer each, so an array of them is a pointer table
+  static_assert( sizeof( typename ContextType::TokenContextType ) == sizeof( void* ) );
+  static_assert( sizeof( typename ContextType::LayerContextType ) == sizeof( void* ) );
+
+  static void* const* token_table( typename ContextType::TokenContextType token_contexts[], uint64_t )
+  {
+    return reinterpret_cast<void* const*>( token_contexts );
+  }
+  static const void* const* layer_table( const typename ContextType::LayerContextType layer_contexts[], uint64_t )
+  {
+    return reinterpret_cast<const void* const*>( layer_contexts );
+  }
+};
+
+} // namespace glint::hip

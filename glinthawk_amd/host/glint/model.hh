@@ -1,0 +1,636 @@
+// Llama2 stage driver for the hip target: owns the hosted weights and the scratchpad, and issues the
+// ops of one stage step in the reference's order (models/llama2/model.hh:311-442, 444-808):
+//
+//   pre-attention   rmsnorm -> wq -> wkv -> KV append
+//   attention       RoPE (q and the appended K row) -> scores -> softmax -> weighted sum
+//   post-attention  wo -> residual -> rmsnorm -> w1, w3 -> SiLU gate -> w2 -> residual
+//   classification  final rmsnorm -> wcls -> (Gumbel noise if temperature > 0) -> argmax
+//
+// Two attention paths produce the same result: the fused split-K kernel (default; per-step tables
+// of row addresses are uploaded once and shared by all layers) and the three unfused ops of the
+// reference's interface with the (batch, n_heads, seq_len) score buffer.
+#pragma once
+
+#include <algorithm>
+#include <cmath>
+#include <memory>
+#include <vector>
+
+#include "glint/concepts.hh"
+#include "glint/config.hh"
+#include "glint/context.hh"
+#include "glint/hip/ops.hh"
+#include "glint/state.hh"
+
+namespace glint {
+
+constexpr size_t MAX_BATCH_SIZE = 1024; // models/llama2/base.hh:26
+
+// element counts of the weight files, in file order (models/llama2/base.hh:357-373,477-499)
+template<typename Config>
+struct WeightLayout
+{
+  // base: token_embedding_table, rms_final_weight, freq_cis_real, freq_cis_imag, wcls
+  static std::array<uint64_t, 5> base_on_disk()
+  {
+    return { Config::vocab_size * Config::dim, Config::dim, Config::seq_len * Config::head_size / 2, Config::seq_len * Config::head_size / 2,
+             Config::wcls_present ? Config::vocab_size * Config::dim : 0 };
+  }
+  // layer: rms_att_weight, wq, wkv (wk rows then wv rows), wo, rms_ffn_weight, w1, w2, w3
+  static std::array<uint64_t, 8> layer_on_disk()
+  {
+    return { Config::dim, Config::dim * Config::dim, Config::dim * Config::kv_dim * 2, Config::dim * Config::dim, Config::dim, Config::dim * Config::hidden_dim,
+             Config::dim * Config::hidden_dim, Config::dim * Config::hidden_dim };
+  }
+  // what a node keeps in memory depends on what it hosts (models/llama2/base.hh:410-433,520-545)
+  template<typename Settings>
+  static std::array<uint64_t, 5> base_in_memory( const Settings& s )
+  {
+    const bool emb = s.hosts( 0, InferenceStage::PreAttention ) || ( s.hosts_in_any_layer( InferenceStage::Classification ) && !Config::wcls_present );
+    const bool att = s.hosts_in_any_layer( InferenceStage::Attention );
+    const bool cls = s.hosts_in_any_layer( InferenceStage::Classification );
+    auto d = base_on_disk();
+    return { emb ? d[0] : 0, cls ? d[1] : 0, att ? d[2] : 0, att ? d[3] : 0, ( Config::wcls_present && cls ) ? d[4] : 0 };
+  }
+  template<typename Settings>
+  static std::array<uint64_t, 8> layer_in_memory( const Settings& s, size_t layer )
+  {
+    const bool pre = s.hosts( layer, InferenceStage::PreAttention );
+    const bool post = s.hosts( layer, InferenceStage::PostAttention );
+    auto d = layer_on_disk();
+    return { pre ? d[0] : 0, pre ? d[1] : 0, pre ? d[2] : 0, post ? d[3] : 0, post ? d[4] : 0, post ? d[5] : 0, post ? d[6] : 0, post ? d[7] : 0 };
+  }
+};
+
+template<typename DType>
+struct BaseWeights
+{
+  DType* token_embedding_table {};
+  DType* rms_final_weight {};
+  DType* freq_cis_real {};
+  DType* freq_cis_imag {};
+  DType* wcls {}; // aliases the embedding table when the model has no separate classifier
+};
+
+template<typename DType>
+struct LayerWeights
+{
+  DType* rms_att_weight {};
+  DType* wq {};
+  DType* wkv {};
+  DType* wo {};
+  DType* rms_ffn_weight {};
+  DType* w1 {};
+  DType* w2 {};
+  DType* w3 {};
+  DType* tensor( size_t k ) const
+  {
+    DType* const t[8] = { rms_att_weight, wq, wkv, wo, rms_ffn_weight, w1, w2, w3 };
+    return t[k];
+  }
+};
+
+struct ModelOptions
+{
+  bool fused_attention { true };  // false: the reference's three unfused ops + score buffer
+  bool allocate_logits { true };  // only needed when the classifier is hosted
+  uint64_t seed { 1 };            // random initialisation of weights
+  float weight_std { 0.02f };     // N(0, std) for every tensor, as the benchmark configurations say
+};
+
+template<typename Config, typename DType, typename LlamaOperations = hip::LlamaOperations<Config, DType>, typename Context = hip::Context<Config, DType>>
+requires ModelConfig<Config>
+class Llama2
+{
+public:
+  using ConfigType = Config;
+  using DataTypeT = DType;
+  using ContextType = Context;
+  using SettingsType = StageSettings<Config>;
+  using StateType = BatchedInferenceState<Config>;
+  using ContextVector = std::vector<std::shared_ptr<Context>>;
+  using DevicePtr = typename LlamaOperations::DeviceUniquePtr;
+
+  static_assert( LlamaOperationsConcept<LlamaOperations, DType, SettingsType> );
+  static_assert( ContextConcept<Context, DType> );
+
+  // weights are drawn N(0, weight_std) from `options.seed`; RoPE tables come from the closed form
+  explicit Llama2( const SettingsType& settings, const ModelOptions options = {} )
+    : settings_( settings )
+    , options_( options )
+    , ops_( settings )
+  {
+    GLINT_CHECK( settings_.concurrency_limit <= MAX_BATCH_SIZE );
+    allocate_weights();
+    allocate_scratch();
+    randomize_weights();
+    write_rope_tables();
+  }
+
+  const SettingsType& settings() const { return settings_; }
+  LlamaOperations& ops() { return ops_; }
+  const BaseWeights<DType>& base_weights() const { return base_; }
+  const LayerWeights<DType>& layer_weights( size_t l ) const { return layers_[l]; }
+
+  // copies `n` elements from host memory into tensor `k` (file order) of a hosted layer
+  void set_layer_tensor( size_t layer, size_t k, const DType* host, uint64_t n )
+  {
+    GLINT_CHECK( layer < Config::n_layers && k < 8 );
+    GLINT_CHECK( n == WeightLayout<Config>::layer_in_memory( settings_, layer )[k] );
+    ops_.copy( layers_[layer].tensor( k ), host, n * sizeof( DType ), CopyType::HostToDevice );
+  }
+  // k: 0 token_embedding_table, 1 rms_final_weight, 2 freq_cis_real, 3 freq_cis_imag, 4 wcls
+  void set_base_tensor( size_t k, const DType* host, uint64_t n )
+  {
+    DType* const t[5] = { base_.token_embedding_table, base_.rms_final_weight, base_.freq_cis_real, base_.freq_cis_imag, base_.wcls };
+    GLINT_CHECK( k < 5 && t[k] != nullptr && n == WeightLayout<Config>::base_in_memory( settings_ )[k] );
+    ops_.copy( t[k], host, n * sizeof( DType ), CopyType::HostToDevice );
+  }
+
+  // ------------------------------------------------------------------------------------------
+  // forward(): every stage of every hosted layer, starting at states.next_layer()
+  // ------------------------------------------------------------------------------------------
+  void forward( StateType& states, const ContextVector& contexts )
+  {
+    check_batch( states, contexts.size(), InferenceStage::PreAttention );
+    batch_ = states.batch_size();
+    const uint32_t first = states.next_layer();
+
+    // contexts first: position 0 on the first served layer restarts a slot (paged contexts drop their pages)
+    for ( size_t i = 0; i < contexts.size(); i++ ) {
+      GLINT_CHECK( contexts[i]->prepare( first, states.token_pos( i ), states.token_pos( i ) == 0 && settings_.first_layer_served == first ) );
+      token_positions_[i] = states.token_pos( i );
+    }
+
+    if ( first == 0 ) {
+      load_embedding( states );
+    } else {
+      ops_.copy( x_, reinterpret_cast<const DType*>( states.activations().data() ), states.activations().len(), CopyType::HostToDevice, true );
+    }
+
+    size_t last = Config::n_layers;
+    std::vector<size_t> run;
+    for ( size_t l = first; l < Config::n_layers && settings_.hosts( l, InferenceStage::PreAttention ); l++ ) {
+      run.push_back( l );
+    }
+    for ( size_t l : run ) {
+      for ( size_t i = 0; i < contexts.size(); i++ ) {
+        GLINT_CHECK( contexts[i]->prepare( l, states.token_pos( i ), false ) );
+      }
+    }
+    if ( options_.fused_attention ) {
+      upload_tables( contexts, run );
+    }
+
+    for ( size_t k = 0; k < run.size(); k++ ) {
+      const size_t l = run[k];
+      for ( size_t i = 0; i < contexts.size(); i++ ) {
+        layer_contexts_[i] = contexts[i]->layer( l );
+        token_contexts_[i] = contexts[i]->layer( l ).token( states.token_pos( i ) );
+      }
+      pre_attention_ops( l, true, k );
+      GLINT_CHECK( settings_.hosts( l, InferenceStage::Attention ) );
+      attention_ops( k );
+      GLINT_CHECK( settings_.hosts( l, InferenceStage::PostAttention ) );
+      post_attention_ops( l );
+      last = l;
+    }
+    GLINT_CHECK( last < Config::n_layers );
+
+    if ( last == Config::n_layers - 1 && settings_.hosts( last, InferenceStage::Classification ) ) {
+      classify_ops();
+      postlude( states, last, true );
+    } else {
+      postlude( states, last, false );
+    }
+  }
+
+  // ------------------------------------------------------------------------------------------
+  // stage-at-a-time entry points (disaggregated execution)
+  // ------------------------------------------------------------------------------------------
+  void forward_pre_attention( StateType& states )
+  {
+    check_batch( states, 0, InferenceStage::PreAttention );
+    batch_ = states.batch_size();
+    if ( states.next_layer() == 0 ) {
+      load_embedding( states );
+    } else {
+      ops_.copy( x_, reinterpret_cast<const DType*>( states.activations().data() ), states.activations().len(), CopyType::HostToDevice, true );
+    }
+    pre_attention_ops( states.next_layer(), false, 0 );
+    export_pre_attention( states );
+  }
+
+  void forward_attention( StateType& states, const ContextVector& contexts )
+  {
+    check_batch( states, contexts.size(), InferenceStage::Attention );
+    batch_ = states.batch_size();
+    const uint32_t l = states.next_layer();
+    for ( size_t i = 0; i < states.batch_size(); i++ ) {
+      GLINT_CHECK( contexts[i]->prepare( l, states.token_pos( i ), states.token_pos( i ) == 0 && settings_.first_layer_served == l ) );
+      token_positions_[i] = states.token_pos( i );
+      layer_contexts_[i] = contexts[i]->layer( l );
+      token_contexts_[i] = contexts[i]->layer( l ).token( states.token_pos( i ) );
+    }
+
+    // the wire dtype may differ from the attention dtype (fp16 activations, fp32 attention)
+    import_converted( q_, states.queries().data(), states.queries().len(), states.dtype() );
+    if ( states.has_kvs() ) {
+      for ( size_t i = 0; i < states.batch_size(); i++ ) {
+        if ( states.active( i ) && !token_contexts_[i].empty() ) {
+          import_converted( token_contexts_[i].key(), states.kv( i ), 2 * Config::kv_dim * DataTypeSize( states.dtype() ), states.dtype() );
+        }
+      }
+    }
+    if ( options_.fused_attention ) {
+      upload_tables( contexts, { static_cast<size_t>( l ) } );
+    }
+    attention_ops( 0 );
+
+    if ( !states.has_queries() ) {
+      states.allocate_queries();
+    }
+    export_converted( states.queries().data(), xb_, states.queries().len(), states.dtype() ); // the output travels in the query buffer
+    states.set_next_stage( InferenceStage::PostAttention );
+  }
+
+  void forward_post_attention( StateType& states, const bool fuse_to_pre = false, const bool fuse_to_cls = false )
+  {
+    check_batch( states, 0, InferenceStage::PostAttention );
+    batch_ = states.batch_size();
+    ops_.copy( x_, reinterpret_cast<const DType*>( states.activations().data() ), states.activations().len(), CopyType::HostToDevice );
+    ops_.copy( xb_, reinterpret_cast<const DType*>( states.queries().data() ), states.queries().len(), CopyType::HostToDevice );
+    post_attention_ops( states.next_layer() );
+
+    const uint32_t l = states.next_layer();
+    if ( fuse_to_cls && l == Config::n_layers - 1 && settings_.hosts( l, InferenceStage::Classification ) ) {
+      classify_ops();
+      postlude( states, l, true );
+    } else if ( fuse_to_pre && l < Config::n_layers - 1 && settings_.hosts( l + 1, InferenceStage::PreAttention ) ) {
+      states.set_next_layer( l + 1 );
+      pre_attention_ops( l + 1, false, 0 );
+      export_pre_attention( states );
+    } else {
+      postlude( states, l, false );
+    }
+  }
+
+  void forward_classify( StateType& states )
+  {
+    check_batch( states, 0, InferenceStage::Classification );
+    batch_ = states.batch_size();
+    ops_.copy( x_, reinterpret_cast<const DType*>( states.activations().data() ), states.activations().len(), CopyType::HostToDevice );
+    classify_ops();
+    postlude( states, states.next_layer(), true );
+  }
+
+  // scratch views for tests (device pointers)
+  DType* scratch_x() const { return x_; }
+  DType* scratch_xb() const { return xb_; }
+  DType* scratch_q() const { return q_; }
+  DType* scratch_kv() const { return kv_; }
+  DType* scratch_logits() const { return logits_; }
+  const uint32_t* argmax_pos() const { return argmax_pos_; }
+
+private:
+  // ---- ops of one layer ----------------------------------------------------------------------
+  void pre_attention_ops( const size_t layer, const bool update_kv_cache, const size_t table_index )
+  {
+    const auto& w = layers_[layer];
+    ops_.template rmsnorm<Config::dim>( xb_, x_, reinterpret_cast<float32_t*>( temp_ ), w.rms_att_weight, batch_ );
+    ops_.template matmul<Config::dim, Config::dim>( q_, xb_, w.wq, batch_ );
+    ops_.template matmul<Config::dim, Config::kv_dim * 2>( kv_, xb_, w.wkv, batch_ );
+    if ( update_kv_cache ) {
+      if ( options_.fused_attention ) {
+        GLINT_GH( gh_kv_append( token_rows_dev( table_index ), kv_, batch_, Config::kv_dim, hip::gh_type<DType>(), ops_.stream() ) );
+      } else {
+        ops_.copy_kv_cache( token_contexts_, kv_, batch_ );
+      }
+    }
+  }
+
+  void attention_ops( const size_t table_index )
+  {
+    if ( options_.fused_attention ) {
+      GLINT_GH( gh_rope( batch_, pos_dev(), base_.freq_cis_real, base_.freq_cis_imag, q_, token_rows_dev( table_index ), Config::n_kv_heads, Config::gqa_size,
+                         Config::head_size, hip::gh_type<DType>(), ops_.stream() ) );
+      ops_.attention_fused( q_, layer_rows_dev( table_index ), pos_dev(), xb_, batch_, max_pos_, attn_ws_.get(), attn_ws_bytes_ );
+    } else {
+      ops_.apply_rope( batch_, token_positions_, base_.freq_cis_real, base_.freq_cis_imag, q_, token_contexts_ );
+      ops_.attention_0_gemm( q_, layer_contexts_, att_, batch_, token_positions_ );
+      ops_.attention_softmax( att_, token_positions_, temp_, batch_ );
+      ops_.attention_2_gemm( att_, layer_contexts_, xb_, batch_, token_positions_ );
+    }
+  }
+
+  void post_attention_ops( const size_t layer )
+  {
+    const auto& w = layers_[layer];
+    ops_.template matmul<Config::dim, Config::dim>( xb2_, xb_, w.wo, batch_ );
+    ops_.template accum<Config::dim>( x_, xb2_, batch_ );
+    ops_.template rmsnorm<Config::dim>( xb_, x_, reinterpret_cast<float32_t*>( temp_ ), w.rms_ffn_weight, batch_ );
+    ops_.template matmul<Config::dim, Config::hidden_dim>( hb_, xb_, w.w1, batch_ );
+    ops_.template matmul<Config::dim, Config::hidden_dim>( hb2_, xb_, w.w3, batch_ );
+    ops_.template silu<Config::hidden_dim>( hb_, hb2_, batch_ );
+    ops_.template matmul<Config::hidden_dim, Config::dim>( xb_, hb_, w.w2, batch_ );
+    ops_.template accum<Config::dim>( x_, xb_, batch_ );
+  }
+
+  void classify_ops()
+  {
+    ops_.template rmsnorm<Config::dim>( x_, x_, reinterpret_cast<float32_t*>( temp_ ), base_.rms_final_weight, batch_ );
+    ops_.template matmul<Config::dim, Config::vocab_size>( logits_, x_, base_.wcls, batch_ );
+  }
+
+  // ---- staging ---------------------------------------------------------------------------------
+  void check_batch( const StateType& states, const size_t n_contexts, const InferenceStage stage ) const
+  {
+    GLINT_CHECK( states.batch_size() > 0 && states.batch_size() <= settings_.concurrency_limit );
+    GLINT_CHECK( states.next_stage() == stage );
+    GLINT_CHECK( settings_.hosts( states.next_layer(), stage ) );
+    if ( stage == InferenceStage::Attention || n_contexts != 0 ) {
+      GLINT_CHECK( n_contexts == states.batch_size() );
+    }
+    if ( stage != InferenceStage::Attention ) {
+      GLINT_CHECK( states.dtype() == dtype_of<DType>() );
+    }
+  }
+
+  void load_embedding( const StateType& states )
+  {
+    for ( size_t i = 0; i < states.batch_size(); i++ ) {
+      if ( states.active( i ) ) {
+        GLINT_CHECK( states.token( i ) < Config::vocab_size );
+        ops_.copy( x_ + i * Config::dim, base_.token_embedding_table + (uint64_t)states.token( i ) * Config::dim, Config::dim * sizeof( DType ),
+                   CopyType::DeviceToDevice, true );
+      }
+    }
+  }
+
+  void export_pre_attention( StateType& states )
+  {
+    if ( !states.has_activations() ) {
+      states.allocate_activations();
+    }
+    if ( !states.has_queries() ) {
+      states.allocate_queries();
+    }
+    if ( !states.has_kvs() ) {
+      states.allocate_kvs();
+    }
+    ops_.copy( reinterpret_cast<DType*>( states.activations().data() ), x_, states.activations().len(), CopyType::DeviceToHost );
+    ops_.copy( reinterpret_cast<DType*>( states.queries().data() ), q_, states.queries().len(), CopyType::DeviceToHost );
+    ops_.copy( reinterpret_cast<DType*>( states.kvs().data() ), kv_, states.kvs().len(), CopyType::DeviceToHost );
+    states.set_next_stage( InferenceStage::Attention );
+  }
+
+  void import_converted( DType* dst_dev, const uint8_t* src_host, const uint64_t src_bytes, const DataType wire )
+  {
+    if ( wire == DataType::Float32 ) {
+      ops_.template convert_and_copy<DType, float32_t>( dst_dev, reinterpret_cast<const float32_t*>( src_host ), src_bytes / sizeof( float32_t ), CopyType::HostToDevice );
+    } else if ( wire == DataType::Float16 ) {
+      ops_.template convert_and_copy<DType, float16_t>( dst_dev, reinterpret_cast<const float16_t*>( src_host ), src_bytes / sizeof( float16_t ), CopyType::HostToDevice );
+    } else {
+      fatal( __FILE__, __LINE__, "invalid dtype" );
+    }
+  }
+
+  void export_converted( uint8_t* dst_host, const DType* src_dev, const uint64_t dst_bytes, const DataType wire )
+  {
+    if ( wire == DataType::Float32 ) {
+      ops_.template convert_and_copy<float32_t, DType>( reinterpret_cast<float32_t*>( dst_host ), src_dev, dst_bytes / sizeof( float32_t ), CopyType::DeviceToHost );
+    } else if ( wire == DataType::Float16 ) {
+      ops_.template convert_and_copy<float16_t, DType>( reinterpret_cast<float16_t*>( dst_host ), src_dev, dst_bytes / sizeof( float16_t ), CopyType::DeviceToHost );
+    } else {
+      fatal( __FILE__, __LINE__, "invalid dtype" );
+    }
+  }
+
+  void postlude( StateType& states, const size_t most_recent_layer, const bool classification_done )
+  {
+    if ( classification_done ) {
+      std::vector<float> temps;
+      for ( size_t i = 0; i < states.batch_size(); i++ ) {
+        temps.push_back( states.temperature( i ) );
+      }
+      ops_.soft_sample( logits_, temps, Config::vocab_size );
+      ops_.template argmax<Config::vocab_size>( argmax_pos_, logits_, temp_, temps.size() );
+
+      states.deallocate_activations();
+      states.deallocate_queries();
+      states.deallocate_kvs();
+      states.set_next_layer( 0 );
+      states.set_next_stage( InferenceStage::PreAttention );
+      for ( size_t i = 0; i < states.batch_size(); i++ ) {
+        if ( states.active( i ) ) {
+          states.set_token( i, argmax_pos_[i] );
+          states.set_token_pos( i, states.token_pos( i ) + 1 );
+          if ( states.check_finished( i ) ) {
+            states.set_finished( i ); // discarding the row is the caller's business
+          }
+        }
+      }
+    } else {
+      states.allocate_activations();
+      states.deallocate_queries();
+      states.deallocate_kvs();
+      ops_.copy( reinterpret_cast<DType*>( states.activations().data() ), x_, states.batch_size() * Config::dim * sizeof( DType ), CopyType::DeviceToHost );
+      if ( most_recent_layer == Config::n_layers - 1 ) {
+        states.set_next_stage( InferenceStage::Classification );
+      } else {
+        states.set_next_stage( InferenceStage::PreAttention );
+        states.set_next_layer( static_cast<uint32_t>( most_recent_layer + 1 ) );
+      }
+    }
+  }
+
+  // ---- device-side tables of the fused path --------------------------------------------------
+  // layout of one upload: pos[cap] (u32) | for each layer of the run: layer_rows[cap], token_rows[cap] (pointers)
+  size_t table_stride() const { return settings_.concurrency_limit; }
+  const uint32_t* pos_dev() const { return reinterpret_cast<const uint32_t*>( tables_dev_.get() ); }
+  uint8_t* ptr_tables( uint8_t* base ) const { return base + ( ( table_stride() * sizeof( uint32_t ) + 15 ) / 16 * 16 ); }
+  const void* const* layer_rows_dev( size_t k ) const
+  {
+    return reinterpret_cast<const void* const*>( ptr_tables( reinterpret_cast<uint8_t*>( tables_dev_.get() ) ) ) + ( 2 * k ) * table_stride();
+  }
+  void* const* token_rows_dev( size_t k ) const
+  {
+    return reinterpret_cast<void* const*>( ptr_tables( reinterpret_cast<uint8_t*>( tables_dev_.get() ) ) ) + ( 2 * k + 1 ) * table_stride();
+  }
+
+  void upload_tables( const ContextVector& contexts, const std::vector<size_t>& run )
+  {
+    // the previous step's upload was consumed by kernels queued before this point on the same
+    // stream; wait for them before the pinned buffer is rewritten
+    ops_.synchronize();
+    auto* pos = reinterpret_cast<uint32_t*>( tables_host_ );
+    auto** ptrs = reinterpret_cast<void**>( ptr_tables( tables_host_ ) );
+    max_pos_ = 0;
+    for ( size_t i = 0; i < batch_; i++ ) {
+      pos[i] = token_positions_[i];
+      if ( !contexts[i]->empty() ) {
+        max_pos_ = std::max( max_pos_, token_positions_[i] );
+      }
+    }
+    for ( size_t k = 0; k < run.size(); k++ ) {
+      for ( size_t i = 0; i < batch_; i++ ) {
+        const auto layer = contexts[i]->layer( run[k] );
+        ptrs[( 2 * k ) * table_stride() + i] = layer.data();
+        ptrs[( 2 * k + 1 ) * table_stride() + i] = layer.token( token_positions_[i] ).key();
+      }
+    }
+    const size_t bytes = ( ptr_tables( tables_host_ ) - tables_host_ ) + run.size() * 2 * table_stride() * sizeof( void* );
+    GLINT_GH( gh_memcpy( tables_dev_.get(), tables_host_, bytes, GH_HOST_TO_DEVICE, 1, ops_.stream() ) );
+  }
+
+  // ---- allocation ----------------------------------------------------------------------------
+  static DType* carve( DType*& cursor, uint64_t n )
+  {
+    DType* p = n ? cursor : nullptr;
+    cursor += ( n + 7 ) / 8 * 8; // keep every tensor 16-byte aligned
+    return p;
+  }
+  static uint64_t padded( uint64_t n ) { return ( n + 7 ) / 8 * 8; }
+
+  void allocate_weights()
+  {
+    const auto b = WeightLayout<Config>::base_in_memory( settings_ );
+    uint64_t total = 0;
+    for ( auto n : b ) {
+      total += padded( n );
+    }
+    base_storage_ = ops_.device_allocate( std::max<uint64_t>( total, 8 ) * sizeof( DType ) );
+    DType* cur = base_storage_.get();
+    base_.token_embedding_table = carve( cur, b[0] );
+    base_.rms_final_weight = carve( cur, b[1] );
+    base_.freq_cis_real = carve( cur, b[2] );
+    base_.freq_cis_imag = carve( cur, b[3] );
+    base_.wcls = carve( cur, b[4] );
+    if ( !Config::wcls_present && settings_.hosts_in_any_layer( InferenceStage::Classification ) ) {
+      base_.wcls = base_.token_embedding_table; // shared classifier (models/llama2/model.hh weight tying)
+    }
+
+    total = 0;
+    for ( size_t l = 0; l < Config::n_layers; l++ ) {
+      for ( auto n : WeightLayout<Config>::layer_in_memory( settings_, l ) ) {
+        total += padded( n );
+      }
+    }
+    layer_storage_ = ops_.device_allocate( std::max<uint64_t>( total, 8 ) * sizeof( DType ) );
+    cur = layer_storage_.get();
+    layers_.resize( Config::n_layers );
+    for ( size_t l = 0; l < Config::n_layers; l++ ) {
+      const auto n = WeightLayout<Config>::layer_in_memory( settings_, l );
+      auto& w = layers_[l];
+      w.rms_att_weight = carve( cur, n[0] );
+      w.wq = carve( cur, n[1] );
+      w.wkv = carve( cur, n[2] );
+      w.wo = carve( cur, n[3] );
+      w.rms_ffn_weight = carve( cur, n[4] );
+      w.w1 = carve( cur, n[5] );
+      w.w2 = carve( cur, n[6] );
+      w.w3 = carve( cur, n[7] );
+    }
+  }
+
+  void allocate_scratch()
+  {
+    const uint64_t cap = settings_.concurrency_limit;
+    const bool cls = settings_.hosts_in_any_layer( InferenceStage::Classification ) && options_.allocate_logits;
+    const uint64_t att_elems = options_.fused_attention ? 0 : cap * Config::n_heads * Config::seq_len;
+    const uint64_t temp_elems = cap * std::max<uint64_t>( Config::n_heads, Config::dim ) * 4 / sizeof( DType );
+    const uint64_t total = padded( cap * Config::dim ) * 4 + padded( cap * Config::kv_dim * 2 ) + padded( cap * Config::hidden_dim ) * 2 + padded( att_elems )
+                           + padded( cls ? cap * Config::vocab_size : 0 ) + padded( temp_elems );
+    scratch_storage_ = ops_.device_allocate( total * sizeof( DType ) );
+    GLINT_GH( gh_memset_zero( scratch_storage_.get(), total * sizeof( DType ), ops_.stream() ) );
+    DType* cur = scratch_storage_.get();
+    x_ = carve( cur, cap * Config::dim );
+    xb_ = carve( cur, cap * Config::dim );
+    xb2_ = carve( cur, cap * Config::dim );
+    q_ = carve( cur, cap * Config::dim );
+    kv_ = carve( cur, cap * Config::kv_dim * 2 );
+    hb_ = carve( cur, cap * Config::hidden_dim );
+    hb2_ = carve( cur, cap * Config::hidden_dim );
+    att_ = carve( cur, att_elems );
+    logits_ = carve( cur, cls ? cap * Config::vocab_size : 0 );
+    temp_ = carve( cur, temp_elems );
+
+    if ( options_.fused_attention ) {
+      const gh_shape s = LlamaOperations::shape();
+      attn_ws_bytes_ = gh_attn_decode_workspace( cap, Config::seq_len - 1, &s );
+      attn_ws_ = ops_.device_allocate( std::max<uint64_t>( attn_ws_bytes_, 16 ) );
+      const size_t n_run = std::max<size_t>( 1, settings_.num_attention_layers_hosted() );
+      const size_t bytes = ( cap * sizeof( uint32_t ) + 15 ) / 16 * 16 + n_run * 2 * cap * sizeof( void* );
+      tables_dev_ = ops_.device_allocate( bytes );
+      void* pinned = nullptr;
+      GLINT_GH( gh_host_malloc( &pinned, bytes ) );
+      tables_host_ = static_cast<uint8_t*>( pinned );
+    }
+  }
+
+  void randomize_weights()
+  {
+    uint64_t seed = options_.seed * 1000003ull;
+    auto fill = [&]( DType* p, uint64_t n ) {
+      if ( p && n ) {
+        GLINT_GH( gh_fill_normal( p, n, 0.0f, options_.weight_std, seed++, hip::gh_type<DType>(), ops_.stream() ) );
+      } else {
+        seed++;
+      }
+    };
+    const auto b = WeightLayout<Config>::base_in_memory( settings_ );
+    fill( base_.token_embedding_table, b[0] );
+    fill( base_.rms_final_weight, b[1] );
+    if ( Config::wcls_present ) {
+      fill( base_.wcls, b[4] );
+    }
+    for ( size_t l = 0; l < Config::n_layers; l++ ) {
+      const auto n = WeightLayout<Config>::layer_in_memory( settings_, l );
+      for ( size_t k = 0; k < 8; k++ ) {
+        fill( layers_[l].tensor( k ), n[k] );
+      }
+    }
+  }
+
+  // cos / sin( pos * theta^(-2k / head_size) ), theta 10000, computed in fp32 (tools/bin2glint.py:19-25)
+  void write_rope_tables()
+  {
+    if ( base_.freq_cis_real == nullptr ) {
+      return;
+    }
+    const uint64_t half = Config::head_size / 2;
+    std::vector<DType> re( Config::seq_len * half ), im( Config::seq_len * half );
+    for ( uint64_t k = 0; k < half; k++ ) {
+      const float freq = 1.0f / std::pow( 10000.0f, static_cast<float>( 2 * k ) / static_cast<float>( Config::head_size ) );
+      for ( uint64_t p = 0; p < Config::seq_len; p++ ) {
+        const float angle = static_cast<float>( p ) * freq;
+        re[p * half + k] = static_cast<DType>( std::cos( angle ) );
+        im[p * half + k] = static_cast<DType>( std::sin( angle ) );
+      }
+    }
+    ops_.copy( base_.freq_cis_real, re.data(), re.size() * sizeof( DType ), CopyType::HostToDevice );
+    ops_.copy( base_.freq_cis_imag, im.data(), im.size() * sizeof( DType ), CopyType::HostToDevice );
+  }
+
+  SettingsType settings_;
+  ModelOptions options_;
+  LlamaOperations ops_;
+
+  DevicePtr base_storage_ {}, layer_storage_ {}, scratch_storage_ {}, attn_ws_ {}, tables_dev_ {};
+  uint64_t attn_ws_bytes_ { 0 };
+  uint8_t* tables_host_ { nullptr };
+  BaseWeights<DType> base_ {};
+  std::vector<LayerWeights<DType>> layers_ {};
+
+  // scratchpad: device buffers ...
+  DType *x_ {}, *xb_ {}, *xb2_ {}, *q_ {}, *kv_ {}, *hb_ {}, *hb2_ {}, *att_ {}, *logits_ {}, *temp_ {};
+  // ... and host arrays (models/llama2/base.hh:196-202)
+  uint64_t batch_ { 1 };
+  uint32_t max_pos_ { 0 };
+  uint32_t argmax_pos_[MAX_BATCH_SIZE] {};
+  uint32_t token_positions_[MAX_BATCH_SIZE] {};
+  typename Context::LayerContextType layer_contexts_[MAX_BATCH_SIZE] {};
+  typename Context::TokenContextType token_contexts_[MAX_BATCH_SIZE] {};
+};
+
+} // namespace glint

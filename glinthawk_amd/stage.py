@@ -1,0 +1,242 @@
+"""ctypes front-end of libglint_host.so: the C++ stage harness (model driver + context manager + one
+batched state) and the host-only bookkeeping hooks.  Used by the tests and the benchmark; all
+compute happens in the C++/HIP layers."""
+from __future__ import annotations
+
+import ctypes as C
+import os
+from typing import Optional
+
+import numpy as np
+
+from ._lib import GlintError
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+_HOST_LIB_PATH = os.path.join(_PKG, "lib", "libglint_host.so")
+
+STAGE_PRE, STAGE_ATT, STAGE_POST, STAGE_CLS = 0, 1, 2, 3
+FWD_ALL, FWD_PRE, FWD_ATT, FWD_POST, FWD_CLS = 0, 1, 2, 3, 4
+FLAG_FUSED, FLAG_CLS, FLAG_PAGED = 1, 2, 4
+
+# layer tensors in file order (rms_att_weight, wq, wkv, wo, rms_ffn_weight, w1, w2, w3)
+LAYER_TENSORS = ("rms_att_weight", "wq", "wkv", "wo", "rms_ffn_weight", "w1", "w2", "w3")
+BASE_TENSORS = ("token_embedding_table", "rms_final_weight", "freq_cis_real", "freq_cis_imag", "wcls")
+
+_host: Optional[C.CDLL] = None
+
+
+def host_lib_path() -> str:
+    return _HOST_LIB_PATH
+
+
+def host_lib() -> C.CDLL:
+    global _host
+    if _host is None:
+        if not os.path.exists(_HOST_LIB_PATH):
+            raise GlintError(f"{_HOST_LIB_PATH} is missing: build it with `python -m glinthawk_amd.build`")
+        L = C.CDLL(_HOST_LIB_PATH)
+        vp, u32, u64, i32 = C.c_void_p, C.c_uint32, C.c_uint64, C.c_int32
+        sig = {
+            "glint_stage_create": (vp, [C.c_char_p, C.c_int, u32, u32, u32, u32, u32, u64, C.c_float]),
+            "glint_stage_destroy": (None, [vp]),
+            "glint_stage_set_layer_tensor": (None, [vp, u32, u32, vp, u64]),
+            "glint_stage_set_base_tensor": (None, [vp, u32, vp, u64]),
+            "glint_stage_new_state": (None, [vp, u32, u32, C.c_int]),
+            "glint_stage_set_prompt": (None, [vp, u32, u32, u32, u32, C.c_float, u32, u32]),
+            "glint_stage_discard": (None, [vp, u32]),
+            "glint_stage_acquire_contexts": (C.c_int, [vp]),
+            "glint_stage_forward": (C.c_int, [vp, C.c_int]),
+            "glint_stage_buffer": (vp, [vp, C.c_int, C.POINTER(u64), C.c_int]),
+            "glint_stage_row_info": (None, [vp, u32, C.POINTER(u32)]),
+            "glint_stage_state_info": (None, [vp, C.POINTER(u32)]),
+            "glint_stage_context_layer_ptr": (vp, [vp, u32, u32]),
+            "glint_stage_context_slot": (i32, [vp, u32]),
+            "glint_stage_slot_counts": (None, [vp, C.POINTER(u64)]),
+            "glint_stage_release_context": (C.c_int, [vp, u32]),
+            "glint_stage_paging_info": (None, [vp, u32, u32, C.POINTER(u64)]),
+            "glint_stage_scratch": (vp, [vp, C.c_int]),
+            "glint_stage_sync": (None, [vp]),
+            "glint_book_manager_new": (vp, [u64]),
+            "glint_book_manager_delete": (None, [vp]),
+            "glint_book_manager_free": (u64, [vp]),
+            "glint_book_manager_allocated": (u64, [vp]),
+            "glint_book_manager_get_contexts": (C.c_int, [vp, vp, vp, u64, u64, u64, vp]),
+            "glint_book_manager_get_context": (i32, [vp, u32]),
+            "glint_book_manager_release": (C.c_int, [vp, u32]),
+            "glint_book_paged_new": (vp, [u32]),
+            "glint_book_paged_delete": (None, [vp]),
+            "glint_book_paged_prepare": (u64, [vp, u32, u32, C.c_int, C.POINTER(u64)]),
+            "glint_book_key_head_offset": (u64, [vp, u32, u32, u32, C.c_int]),
+        }
+        for name, (res, args) in sig.items():
+            fn = getattr(L, name)
+            fn.restype = res
+            fn.argtypes = args
+        _host = L
+    return _host
+
+
+class Stage:
+    """One pipeline stage on the GPU: `n_hosted` consecutive layers of `config` starting at
+    `first_layer`, with `max_contexts` preallocated context slots."""
+
+    def __init__(self, config: str, dtype: str, first_layer: int, n_hosted: int, concurrency: int,
+                 max_contexts: int, fused: bool = True, with_cls: bool = False, paged: bool = False,
+                 seed: int = 1, weight_std: float = 0.02):
+        self.np_dtype = np.float16 if dtype == "f16" else np.float32
+        flags = (FLAG_FUSED if fused else 0) | (FLAG_CLS if with_cls else 0) | (FLAG_PAGED if paged else 0)
+        self._h = host_lib().glint_stage_create(config.encode(), 0 if dtype == "f16" else 1, first_layer, n_hosted,
+                                                concurrency, max_contexts, flags, seed, weight_std)
+        if not self._h:
+            raise GlintError(f"unknown stage configuration {config!r}")
+
+    def close(self):
+        if getattr(self, "_h", None):
+            host_lib().glint_stage_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        self.close()
+
+    # ---- weights
+    def set_layer_tensor(self, layer: int, name: str, arr: np.ndarray) -> None:
+        a = np.ascontiguousarray(arr, dtype=self.np_dtype)
+        host_lib().glint_stage_set_layer_tensor(self._h, layer, LAYER_TENSORS.index(name), a.ctypes.data, a.size)
+
+    def set_base_tensor(self, name: str, arr: np.ndarray) -> None:
+        a = np.ascontiguousarray(arr, dtype=self.np_dtype)
+        host_lib().glint_stage_set_base_tensor(self._h, BASE_TENSORS.index(name), a.ctypes.data, a.size)
+
+    # ---- state
+    def new_state(self, batch: int, next_layer: int = 0, next_stage: int = STAGE_PRE) -> None:
+        host_lib().glint_stage_new_state(self._h, batch, next_layer, next_stage)
+
+    def set_prompt(self, row: int, context_id: int, token: int, pos: int, temperature: float = 0.0,
+                   prompt_length: int = 1, max_completion_length: int = 0) -> None:
+        host_lib().glint_stage_set_prompt(self._h, row, context_id, token, pos, temperature, prompt_length,
+                                          max_completion_length)
+
+    def discard(self, row: int) -> None:
+        host_lib().glint_stage_discard(self._h, row)
+
+    def acquire_contexts(self) -> bool:
+        return host_lib().glint_stage_acquire_contexts(self._h) == 0
+
+    def forward(self, which: int = FWD_ALL) -> bool:
+        """False when the context manager could not serve the batch (nothing ran)."""
+        rc = host_lib().glint_stage_forward(self._h, which)
+        if rc == -2:
+            raise GlintError("bad forward selector")
+        return rc == 0
+
+    def _buffer(self, which: int, allocate: bool) -> np.ndarray:
+        n = C.c_uint64(0)
+        p = host_lib().glint_stage_buffer(self._h, which, C.byref(n), int(allocate))
+        if not p or n.value == 0:
+            return np.empty(0, dtype=self.np_dtype)
+        buf = (C.c_uint8 * n.value).from_address(p)
+        return np.frombuffer(buf, dtype=self.np_dtype)
+
+    def activations(self, allocate: bool = False) -> np.ndarray:
+        return self._buffer(0, allocate)
+
+    def queries(self, allocate: bool = False) -> np.ndarray:
+        return self._buffer(1, allocate)
+
+    def kvs(self, allocate: bool = False) -> np.ndarray:
+        return self._buffer(2, allocate)
+
+    def row(self, i: int) -> dict:
+        out = (C.c_uint32 * 6)()
+        host_lib().glint_stage_row_info(self._h, i, out)
+        return dict(active=bool(out[0]), context_id=out[1], token=out[2], token_pos=out[3], finished=bool(out[4]),
+                    temperature_u8=out[5])
+
+    def state(self) -> dict:
+        out = (C.c_uint32 * 4)()
+        host_lib().glint_stage_state_info(self._h, out)
+        return dict(batch_size=out[0], next_layer=out[1], next_stage=out[2], has_activations=bool(out[3] & 1),
+                    has_queries=bool(out[3] & 2), has_kvs=bool(out[3] & 4))
+
+    # ---- contexts
+    def context_layer_ptr(self, row: int, layer: int) -> int:
+        return host_lib().glint_stage_context_layer_ptr(self._h, row, layer) or 0
+
+    def context_slot(self, row: int) -> int:
+        return host_lib().glint_stage_context_slot(self._h, row)
+
+    def slot_counts(self) -> dict:
+        out = (C.c_uint64 * 3)()
+        host_lib().glint_stage_slot_counts(self._h, out)
+        return dict(free=out[0], allocated=out[1], total=out[2])
+
+    def release_context(self, context_id: int) -> bool:
+        return bool(host_lib().glint_stage_release_context(self._h, context_id))
+
+    def paging_info(self, row: int, layer: int) -> dict:
+        out = (C.c_uint64 * 3)()
+        host_lib().glint_stage_paging_info(self._h, row, layer, out)
+        return dict(allocated_bytes=out[0], blocks_committed=out[1], clears=out[2])
+
+    def scratch_ptr(self, name: str) -> int:
+        return host_lib().glint_stage_scratch(self._h, ("x", "xb", "q", "kv", "logits").index(name)) or 0
+
+    def sync(self) -> None:
+        host_lib().glint_stage_sync(self._h)
+
+
+class BookManager:
+    """Host-only instance of the slot manager (no device memory), for bookkeeping tests."""
+
+    def __init__(self, max_context_count: int):
+        self._m = host_lib().glint_book_manager_new(max_context_count)
+
+    def __del__(self):
+        if getattr(self, "_m", None):
+            host_lib().glint_book_manager_delete(self._m)
+            self._m = None
+
+    def free(self) -> int:
+        return int(host_lib().glint_book_manager_free(self._m))
+
+    def allocated(self) -> int:
+        return int(host_lib().glint_book_manager_allocated(self._m))
+
+    def get_contexts(self, active, context_ids, start: int = 0, end: Optional[int] = None):
+        a = np.ascontiguousarray(np.asarray(active, dtype=np.uint8))
+        ids = np.ascontiguousarray(np.asarray(context_ids, dtype=np.uint32))
+        end = len(a) if end is None else end
+        out = np.empty(max(1, end - start), dtype=np.int32)
+        ok = host_lib().glint_book_manager_get_contexts(self._m, a.ctypes.data, ids.ctypes.data, len(a), start, end,
+                                                        out.ctypes.data)
+        return out[: end - start].tolist() if ok else None
+
+    def get_context(self, context_id: int) -> int:
+        return int(host_lib().glint_book_manager_get_context(self._m, context_id))
+
+    def release(self, context_id: int) -> bool:
+        return bool(host_lib().glint_book_manager_release(self._m, context_id))
+
+
+class BookPagedContext:
+    """Host-only paged context (70B-4K shape, fp16) over a region that only records commits."""
+
+    def __init__(self, n_hosted: int):
+        self._c = host_lib().glint_book_paged_new(n_hosted)
+
+    def __del__(self):
+        if getattr(self, "_c", None):
+            host_lib().glint_book_paged_delete(self._c)
+            self._c = None
+
+    def prepare(self, layer: int, token_pos: int, can_release: bool):
+        out = (C.c_uint64 * 2)()
+        allocated = host_lib().glint_book_paged_prepare(self._c, layer, token_pos, int(can_release), out)
+        return int(allocated), int(out[0]), int(out[1])
+
+
+def book_head_offset(hosted, layer: int, pos: int, head: int, value: bool) -> Optional[int]:
+    h = np.ascontiguousarray(np.asarray(hosted, dtype=np.uint8))
+    assert h.size == 80
+    v = host_lib().glint_book_key_head_offset(h.ctypes.data, layer, pos, head, int(value))
+    return None if v == 2 ** 64 - 1 else int(v)
