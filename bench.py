@@ -1,0 +1,248 @@
+#!/usr/bin/env python3
+"""Benchmark of the per-stage Llama2 KV-cache path on one MI355X.
+
+One "step" is one pass of the hot path over one batch: the C++ stage driver's forward() for a
+pipeline stage of 10 layers of the Llama2-70B GQA shape (pre-attention, KV append, RoPE, fused
+decode attention, post-attention for every layer) with decode batch 64 and every context
+pre-filled so that the current token attends 4096 keys.  Inputs are synthetic (weights N(0,0.02),
+K/V rows N(0,1), activations N(0,1), all seeded) and resident in HBM before the timed region.
+
+Prints ONE JSON line:
+  value        decode-attention algorithmic bytes / time of the attention op (split-K kernel + merge)
+  roofline     the dominant kernel (split-K attention) against the 8 TB/s HBM peak, from HIP events
+               recorded on the launch stream inside the timed steps
+  stage_*      whole stage step: tokens/s and the fraction of the bandwidth roofline
+  cpu_baseline the CPU oracle (a port of the reference's fp32 OpenMP path) timed on a bounded sample
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+# the configurations of BASELINE.json that fit one GPU as a single stage
+WORKLOADS = {
+    # name: (stage config, first layer, hosted layers, batch, keys attended, description)
+    "llama2-70b-gqa-b64-ctx4096": ("llama2-70b-4k", 10, 10, 64, 4096,
+                                   "Llama2-70B GQA shape, one stage of 10 layers, fp16, decode batch 64, 4096 keys per context"),
+    "llama2-7b-b32-ctx1024": ("llama2-7b", 8, 8, 32, 1024,
+                              "Llama2-7B MHA shape, one stage of 8 layers, fp16, decode batch 32, 1024 keys per context"),
+}
+SHAPES = {
+    "llama2-70b-4k": dict(dim=8192, n_heads=64, n_kv_heads=8, hidden_dim=28672, seq_len=4096, n_layers=80),
+    "llama2-7b": dict(dim=4096, n_heads=32, n_kv_heads=32, hidden_dim=11008, seq_len=2048, n_layers=32),
+}
+
+
+def attention_bytes(shape, batch, keys, elem=2):
+    """Algorithmic bytes of one layer's decode attention: every cached K and V element once, plus
+    q read, output write and the appended row."""
+    kv_dim = shape["dim"] // (shape["n_heads"] // shape["n_kv_heads"])
+    return batch * keys * 2 * kv_dim * elem + batch * (2 * shape["dim"] + 2 * kv_dim) * elem
+
+
+def layer_weight_bytes(shape, elem=2):
+    d, h = shape["dim"], shape["hidden_dim"]
+    kv_dim = d // (shape["n_heads"] // shape["n_kv_heads"])
+    return (2 * d + 2 * d * d + 2 * d * kv_dim + 3 * d * h) * elem
+
+
+def gpu_bench(workload, steps, warmup):
+    import numpy as np
+    import torch
+
+    from glinthawk_amd import _lib, ops, stage as S
+
+    cfg_name, first, n_hosted, batch, keys, _ = WORKLOADS[workload]
+    shape = SHAPES[cfg_name]
+    pos = keys - 1
+    ops.init(0)
+    L = _lib.lib()
+
+    st = S.Stage(cfg_name, "f16", first, n_hosted, batch, batch, fused=True, seed=4, weight_std=0.02)
+    st.new_state(batch, next_layer=first)
+    for i in range(batch):
+        st.set_prompt(i, 1000 + i, 1, pos)
+    assert st.acquire_contexts()
+    # pre-fill: every slot gets N(0,1) rows for every hosted layer
+    kv_dim = shape["dim"] // (shape["n_heads"] // shape["n_kv_heads"])
+    layer_elems = shape["seq_len"] * 2 * kv_dim
+    for i in range(batch):
+        for l in range(first, first + n_hosted):
+            _lib.check(L.gh_fill_normal(st.context_layer_ptr(i, l), layer_elems, 0.0, 1.0, 77 + i * 131 + l, _lib.GH_F16, None))
+    ops.sync()
+
+    rng = np.random.default_rng(0)
+    acts = rng.standard_normal((batch, shape["dim"])).astype(np.float16)
+
+    def one_step():
+        st.set_next(first)
+        st.activations(allocate=True)[:] = acts.reshape(-1)
+        ok = st.forward()
+        assert ok
+
+    for _ in range(warmup):
+        one_step()
+    ops.sync()
+    torch.cuda.synchronize()
+    L.gh_attn_timing_enable(1)
+    L.gh_attn_timing_reset()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        one_step()
+    ops.sync()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    k_ms, m_ms, n = C.c_double(0), C.c_double(0), C.c_uint64(0)
+    _lib.check(L.gh_attn_timing_read(C.byref(k_ms), C.byref(m_ms), C.byref(n)))
+    L.gh_attn_timing_enable(0)
+
+    out = st.activations().astype(np.float32)
+    assert np.all(np.isfinite(out)), "stage output is not finite"
+
+    ms_per_step = (t1 - t0) * 1e3 / steps
+    launches = max(1, n.value)
+    kernel_ms = k_ms.value / launches
+    merge_ms = m_ms.value / launches
+    a_bytes = attention_bytes(shape, batch, keys)
+    stage_bytes = n_hosted * (a_bytes + layer_weight_bytes(shape))
+    res = dict(
+        ms_per_step=ms_per_step,
+        attn_kernel_ms=kernel_ms,
+        attn_merge_ms=merge_ms,
+        attn_launches=int(n.value),
+        attn_bytes=a_bytes,
+        stage_bytes=stage_bytes,
+        batch=batch,
+        device=ops.device_name(),
+    )
+    st.close()
+    return res
+
+
+def cpu_baseline(workload):
+    """The oracle (port of the reference's fp32 amd64/OpenMP path) on ONE layer of the workload,
+    fp32 weights and fp32 K/V like the reference's CPU build, median of 3 after one warm-up; the
+    stage figure scales that layer time by the number of hosted layers."""
+    import numpy as np
+
+    import oracle as O
+
+    cfg_name, first, n_hosted, batch, keys, _ = WORKLOADS[workload]
+    s = SHAPES[cfg_name]
+    cfg = O.Config(dim=s["dim"], n_layers=s["n_layers"], n_heads=s["n_heads"], n_kv_heads=s["n_kv_heads"],
+                   hidden_dim=s["hidden_dim"], seq_len=s["seq_len"])
+    rng = np.random.default_rng(1)
+    block = rng.standard_normal(1 << 22).astype(np.float32)
+
+    def tiled(shape, scale):
+        n = int(np.prod(shape))
+        reps = (n + block.size - 1) // block.size
+        return (np.tile(block, reps)[:n] * np.float32(scale)).reshape(shape)
+
+    w = {
+        "rms_att_weight": tiled((cfg.dim,), 0.02), "wq": tiled((cfg.dim, cfg.dim), 0.02),
+        "wkv": tiled((2 * cfg.kv_dim, cfg.dim), 0.02), "wo": tiled((cfg.dim, cfg.dim), 0.02),
+        "rms_ffn_weight": tiled((cfg.dim,), 0.02), "w1": tiled((cfg.hidden_dim, cfg.dim), 0.02),
+        "w2": tiled((cfg.dim, cfg.hidden_dim), 0.02), "w3": tiled((cfg.hidden_dim, cfg.dim), 0.02),
+    }
+    re, im = O.rope_tables(cfg.seq_len, cfg.head_size)
+    cache = tiled((batch, cfg.seq_len, 2 * cfg.kv_dim), 1.0)
+    layers = [cache[i] for i in range(batch)]
+    pos = [keys - 1] * batch
+    scratch = {}
+    att_times, layer_times = [], []
+    for rep in range(4):
+        x = tiled((batch, cfg.dim), 1.0).copy()
+        t0 = time.perf_counter()
+        scratch = O.layer_forward(cfg, w, re, im, x, layers, pos, scratch)
+        t1 = time.perf_counter()
+        q = scratch["q"].copy()
+        O.attention_ops(cfg, pos, re, im, q, layers, att=scratch["att"])
+        t2 = time.perf_counter()
+        if rep:
+            layer_times.append(t1 - t0)
+            att_times.append(t2 - t1)
+    layer_s = float(np.median(layer_times))
+    att_s = float(np.median(att_times))
+    a_bytes32 = attention_bytes(s, batch, keys, elem=4)
+    return {
+        "value": batch / (layer_s * n_hosted),
+        "unit": "tokens/s",
+        "cores": O.num_threads(),
+        "kind": "port",
+        "sample": f"1 of {n_hosted} layers (B={batch}, {keys} keys, fp32 weights and K/V as in the reference's CPU build), "
+                  f"median of 3 after 1 warm-up; layer time {layer_s * 1e3:.0f} ms scaled x{n_hosted}",
+        "attn_GBps": a_bytes32 / att_s / 1e9,
+        "attn_ms_per_layer": att_s * 1e3,
+        "layer_ms": layer_s * 1e3,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="llama2-70b-gqa-b64-ctx4096", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+
+    if args.gpus != 1:
+        print("bench.py: this build runs one pipeline stage on ONE GPU; --gpus must be 1 "
+              "(the path shards by context with no collective, see DESIGN.md)", file=sys.stderr)
+        sys.exit(2)
+
+    g = gpu_bench(args.workload, args.steps, args.warmup)
+    cfg_name, first, n_hosted, batch, keys, desc = WORKLOADS[args.workload]
+
+    attn_op_ms = g["attn_kernel_ms"] + g["attn_merge_ms"]
+    value = g["attn_bytes"] / (attn_op_ms * 1e-3) / 1e9
+    achieved = g["attn_bytes"] / (g["attn_kernel_ms"] * 1e-3) / 1e9
+    tokens_per_s = batch / (g["ms_per_step"] * 1e-3)
+    stage_roofline_ms = g["stage_bytes"] / (HBM_PEAK_GBPS * 1e9) * 1e3
+
+    line = {
+        "metric": "decode attn HBM GB/s (% of peak) + stage tokens/s, Llama2-70B GQA, B=64, ctx 4096",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "pct_of_peak": round(100 * value / HBM_PEAK_GBPS, 2),
+        "stage_tokens_per_s": round(tokens_per_s, 1),
+        "stage_roofline_frac": round(stage_roofline_ms / g["ms_per_step"], 4),
+        "stage_bytes_per_step": g["stage_bytes"],
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(g["ms_per_step"], 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": args.workload, "description": desc, "stage_config": cfg_name, "first_layer": first,
+                   "hosted_layers": n_hosted, "batch": batch, "keys_per_context": keys, "device": g["device"]},
+        "attn_op_ms": round(attn_op_ms, 5),
+        "attn_kernel_ms": round(g["attn_kernel_ms"], 5),
+        "attn_merge_ms": round(g["attn_merge_ms"], 5),
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "kernel": "attn_decode (split-K fused decode attention)", "launches_timed": g["attn_launches"],
+                     "algorithmic_bytes_per_launch": g["attn_bytes"]},
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(args.workload)
+    else:
+        line["cpu_baseline"] = None
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -85,6 +85,7 @@ SIGNATURES = {
     "gh_rmsnorm": (_i, [_vp, _vp, _vp, _u64, _u64, _i, _vp]),
     "gh_silu": (_i, [_vp, _vp, _u64, _u64, _i, _vp]),
     "gh_argmax": (_i, [_vp, _vp, _vp, _u64, _u64, _i, _vp]),
+    "gh_gemm_set_tuning": (_i, [_i, _i, _i]),
     "gh_matmul": (_i, [_vp, _vp, _vp, _u64, _u64, _u64, _i, _vp]),
     "gh_soft_sample": (_i, [_vp, _vp, _u64, _u64, _u64, _i, _vp]),
     "gh_kv_append": (_i, [_vp, _vp, _u64, _u32, _i, _vp]),
@@ -103,7 +104,7 @@ SIGNATURES = {
     "gh_attn_decode_host": (_i, [_vp, _vp, _vp, _vp, _u64, _shp, _i, _vp, _u64, _i, _vp]),
     "gh_attn_timing_enable": (_i, [_i]),
     "gh_attn_timing_reset": (_i, []),
-    "gh_attn_timing_read": (_i, [C.POINTER(C.c_double), C.POINTER(_u64)]),
+    "gh_attn_timing_read": (_i, [C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(_u64)]),
 }
 
 

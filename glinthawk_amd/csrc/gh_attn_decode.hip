@@ -659,14 +659,12 @@ Plan make_plan( uint64_t batch, uint32_t max_pos, const gh_shape* s, gh_dtype dt
   if ( g_chunk_override ) {
     chunk = g_chunk_override;
   } else {
-    // enough independent waves to fill 256 CUs several times over, but splits no shorter than 256
-    // tokens so that the partial traffic stays a few percent of the cache traffic
+    // One wave per (context, kv head, split).  Measured on MI355X: 8 waves per CU (2048 in all), each
+    // streaming a long range, is the sweet spot; with 1024 or more (context, head) streams no split is
+    // needed at all and the merge kernel disappears.  Splits are never shorter than 256 tokens so
+    // that the partial traffic stays a few percent of the cache traffic.
     const uint64_t streams = batch * ( p.variant == GH_ATTN_GENERIC ? s->n_heads : s->n_kv_heads );
-    const uint64_t want_waves = 4096;
-    uint64_t splits = ( want_waves + streams - 1 ) / ( streams ? streams : 1 );
-    if ( splits < 1 ) {
-      splits = 1;
-    }
+    uint64_t splits = streams >= 1024 ? 1 : ( 2048 + streams - 1 ) / ( streams ? streams : 1 );
     chunk = (uint32_t)( ( n_tok + splits - 1 ) / splits );
     if ( chunk < 256 ) {
       chunk = 256;
@@ -777,7 +775,7 @@ int gh_attn_decode( const void* q, const void* const* layer_rows_dev, const uint
   hipStream_t st = as_stream( stream );
   const float scale = LOG2E / sqrtf( (float)shape->head_size );
   int timer = -1;
-  if ( int rc = timer_begin( st, &timer ) ) {
+  if ( int rc = timer_mark( st, &timer, 0 ) ) {
     return rc;
   }
 
@@ -813,6 +811,9 @@ int gh_attn_decode( const void* q, const void* const* layer_rows_dev, const uint
     }
   }
   GH_LAUNCH_CHECK();
+  if ( int rc = timer_mark( st, &timer, 1 ) ) {
+    return rc;
+  }
 
   if ( plan.max_splits > 1 ) {
     const dim3 grid( shape->n_heads, (unsigned)batch );
@@ -826,7 +827,7 @@ int gh_attn_decode( const void* q, const void* const* layer_rows_dev, const uint
     }
     GH_LAUNCH_CHECK();
   }
-  return timer_end( st, timer );
+  return timer_mark( st, &timer, 2 );
 }
 
 int gh_attn_decode_host( const void* q, const void* const* layer_rows_host, const uint32_t* pos_host, void* xb, uint64_t batch,

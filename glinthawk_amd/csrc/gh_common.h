@@ -53,9 +53,9 @@ int stage_table( const void* host_src, size_t bytes, hipStream_t stream, void** 
 // Marks the end of the work that reads the most recently staged slots on this stream.
 int stage_fence( hipStream_t stream );
 
-// Event pair around a kernel sequence when the benchmark's timer is enabled (pair == -1: off).
-int timer_begin( hipStream_t stream, int* pair_out );
-int timer_end( hipStream_t stream, int pair );
+// Three events per sampled attention call when the benchmark's timer is enabled (slot == -1: off):
+// before the split-K kernel, between it and the merge kernel, after the merge kernel.
+int timer_mark( hipStream_t stream, int* slot_inout, int which );
 
 constexpr size_t STAGE_SLOT_BYTES = 16 * 1024; // 1024 rows x (8-byte pointer + 4-byte position) fits
 constexpr uint64_t MAX_BATCH = 1024;           // models/llama2/base.hh:26

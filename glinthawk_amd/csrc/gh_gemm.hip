@@ -14,7 +14,17 @@
 #include <mutex>
 
 namespace gh {
+
+// streaming decode kernel (gh_gemm_stream.hip)
+bool gemm_stream_applicable( uint64_t s, uint64_t r, uint64_t b, const void* x, const void* w, const void* xout );
+void gemm_stream_plan( uint64_t s, uint64_t r, uint64_t b, uint32_t* splits_out, uint32_t* k_per_split_out );
+int gemm_stream_launch( __half* xout, float* partial, const __half* x, const __half* w, uint64_t s, uint64_t r, uint64_t b, uint32_t splits,
+                        uint32_t k_per_split, hipStream_t st );
+void gemm_stream_tuning( int target_wgs, int depth );
+
 namespace {
+
+int g_force_kernel = 0; // 0 auto, 1 tiled kernel of this file, 2 streaming kernel
 
 typedef _Float16 f16x8 __attribute__( ( ext_vector_type( 8 ) ) );
 typedef float f32x4 __attribute__( ( ext_vector_type( 4 ) ) );
@@ -216,6 +226,13 @@ using namespace gh;
 
 extern "C" {
 
+int gh_gemm_set_tuning( int kernel, int target_workgroups, int depth )
+{
+  g_force_kernel = kernel;
+  gemm_stream_tuning( target_workgroups, depth );
+  return GH_OK;
+}
+
 int gh_matmul( void* xout, const void* x, const void* w, uint64_t s, uint64_t r, uint64_t b, gh_dtype dt, gh_stream stream )
 {
   if ( int rc = ensure_init() ) {
@@ -235,6 +252,29 @@ int gh_matmul( void* xout, const void* x, const void* w, uint64_t s, uint64_t r,
     return GH_OK;
   }
   GH_REQUIRE( dt == GH_F16, "gh_matmul: unsupported dtype %d", (int)dt );
+
+  if ( g_force_kernel != 1 && gemm_stream_applicable( s, r, b, x, w, xout ) ) {
+    uint32_t splits = 1, k_per_split = 0;
+    gemm_stream_plan( s, r, b, &splits, &k_per_split );
+    float* ws = nullptr;
+    if ( splits > 1 ) {
+      if ( int rc = ensure_workspace( (uint64_t)splits * b * r * sizeof( float ), &ws ) ) {
+        return rc;
+      }
+    }
+    if ( int rc = gemm_stream_launch( static_cast<__half*>( xout ), ws, static_cast<const __half*>( x ), static_cast<const __half*>( w ), s, r, b, splits,
+                                      k_per_split, st ) ) {
+      return rc;
+    }
+    if ( splits > 1 ) {
+      const uint64_t n = b * r;
+      const unsigned blocks = (unsigned)std::min<uint64_t>( ( n + 255 ) / 256, 4096 );
+      gemm_reduce_kernel<<<blocks, 256, 0, st>>>( static_cast<__half*>( xout ), ws, n, splits );
+      GH_LAUNCH_CHECK();
+    }
+    return GH_OK;
+  }
+  GH_REQUIRE( g_force_kernel != 2, "gh_matmul: the streaming kernel needs s %% 128 == 0, r %% 4 == 0 and 16-byte aligned operands" );
 
   const bool k_vec_ok = ( s % 8 == 0 ) && ( ( reinterpret_cast<uintptr_t>( x ) | reinterpret_cast<uintptr_t>( w ) ) & 15u ) == 0;
   const uint32_t grid_m = (uint32_t)( ( r + BM - 1 ) / BM );

@@ -1,0 +1,283 @@
+// Weight-streaming GEMM for decode: xout(b, r) = sum_p w(r, p) * x(b, p) with a small batch
+// (64 columns per column slab), f16 storage, fp32 accumulate.  Every weight element is read from HBM
+// exactly once, so the kernel is built like a streaming read:
+//
+//   work-group = 4 waves = 128 weight rows x one K range; wave = 32 rows x all 64 batch columns
+//   weights     global -> registers with fully coalesced 16-byte loads.  A register slab is 32 rows x
+//               256 k: both 256-byte halves of a row are requested back to back, so the memory system
+//               sees 512 contiguous bytes per row per visit (256-byte visits cost a quarter of the
+//               bandwidth on this part).  Two register sets: slab i+1 is in flight while slab i is
+//               consumed.  From registers each 128-k half goes through a wave-private LDS tile
+//               (XOR-swizzled 16-byte chunks) into MFMA operand order.
+//   activations one (64 x 128) tile per half shared by the work-group through LDS (two buffers); this
+//               is the only block-level barrier and the weight loads stay in flight across it
+//   math        v_mfma_f32_32x32x16_f16: A = 32 weight rows, B = 32 batch columns, two column tiles
+//
+// K is split across work-groups when there are too few row slabs to fill the chip; the fp32 partials
+// are summed by gemm_reduce_kernel (gh_gemm.hip).
+#include "gh_common.h"
+
+namespace gh {
+
+typedef _Float16 f16x8 __attribute__( ( ext_vector_type( 8 ) ) );
+typedef float f32x16 __attribute__( ( ext_vector_type( 16 ) ) );
+
+namespace {
+
+constexpr int SLAB_K = 256;  // k per register slab: every row is read 512 contiguous bytes at a time
+constexpr int HALF_K = 128;  // k per LDS tile: 16 chunks of 8 halves
+constexpr int WG_ROWS = 128; // weight rows per work-group
+constexpr int COLS = 64;     // batch columns per work-group
+
+// one register slab of a wave: 32 rows x 256 k.  v[h][j], lane (g4, c): row 4*j + g4, 16-byte chunk c of half h
+struct WSlab
+{
+  uint4 v[2][8];
+};
+
+__device__ __forceinline__ void load_w_slab( WSlab& dst, const __half* __restrict__ w, uint64_t ld, uint32_t wave_row0, uint32_t n_rows, uint32_t k0, uint32_t k_end )
+{
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t c = lane & 15, g4 = lane >> 4;
+  const bool k_ok = k0 < k_end; // K ranges are multiples of SLAB_K
+#pragma unroll
+  for ( int j = 0; j < 8; j++ ) {
+    const uint32_t row = wave_row0 + 4 * j + g4;
+    const bool ok = k_ok && row < n_rows;
+    const __half* p = w + (uint64_t)row * ld + k0 + 8 * c;
+    // both halves of the row back to back: 512 contiguous bytes per row reach the memory system together
+    dst.v[0][j] = ok ? *reinterpret_cast<const uint4*>( p ) : make_uint4( 0, 0, 0, 0 );
+    dst.v[1][j] = ok ? *reinterpret_cast<const uint4*>( p + HALF_K ) : make_uint4( 0, 0, 0, 0 );
+  }
+}
+
+__device__ __forceinline__ void stage_w_half( uint4* tile, const WSlab& s, int h )
+{
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t c = lane & 15, g4 = lane >> 4;
+#pragma unroll
+  for ( int j = 0; j < 8; j++ ) {
+    const uint32_t row = 4 * j + g4;
+    tile[row * 16 + ( c ^ ( row & 15 ) )] = s.v[h][j];
+  }
+}
+
+// activations of one register slab: 64 columns x 256 k.  v[h][i], thread t: column t/16 + 16*i, chunk t%16 of half h
+struct XSlab
+{
+  uint4 v[2][4];
+};
+
+__device__ __forceinline__ void load_x_slab( XSlab& dst, const __half* __restrict__ x, uint64_t ld, uint32_t col0, uint32_t n_cols, uint32_t k0, uint32_t k_end )
+{
+  const uint32_t chunk = threadIdx.x & 15;
+  const bool k_ok = k0 < k_end;
+#pragma unroll
+  for ( int i = 0; i < 4; i++ ) {
+    const uint32_t col = col0 + ( threadIdx.x >> 4 ) + 16 * i;
+    const bool ok = k_ok && col < n_cols;
+    const __half* p = x + (uint64_t)col * ld + k0 + 8 * chunk;
+    dst.v[0][i] = ok ? *reinterpret_cast<const uint4*>( p ) : make_uint4( 0, 0, 0, 0 );
+    dst.v[1][i] = ok ? *reinterpret_cast<const uint4*>( p + HALF_K ) : make_uint4( 0, 0, 0, 0 );
+  }
+}
+
+__device__ __forceinline__ void load_x_half( XSlab& dst, const __half* __restrict__ x, uint64_t ld, uint32_t col0, uint32_t n_cols, uint32_t k0, uint32_t k_end, int h )
+{
+  const uint32_t chunk = threadIdx.x & 15;
+  const bool k_ok = k0 < k_end;
+#pragma unroll
+  for ( int i = 0; i < 4; i++ ) {
+    const uint32_t col = col0 + ( threadIdx.x >> 4 ) + 16 * i;
+    dst.v[h][i] = ( k_ok && col < n_cols ) ? *reinterpret_cast<const uint4*>( x + (uint64_t)col * ld + k0 + h * HALF_K + 8 * chunk ) : make_uint4( 0, 0, 0, 0 );
+  }
+}
+
+__device__ __forceinline__ void stage_x_half( uint4* tile, const XSlab& t, int h )
+{
+  const uint32_t chunk = threadIdx.x & 15;
+#pragma unroll
+  for ( int i = 0; i < 4; i++ ) {
+    const uint32_t col = ( threadIdx.x >> 4 ) + 16 * i;
+    tile[col * 16 + ( chunk ^ ( col & 15 ) )] = t.v[h][i];
+  }
+}
+
+// 128 k of math for a wave: 8 steps of k = 16
+__device__ __forceinline__ void half_mfma( f32x16 acc[2], const uint4* wtile, const uint4* xtile )
+{
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t r = lane & 31, g2 = lane >> 5;
+#pragma unroll 2
+  for ( int s = 0; s < 8; s++ ) {
+    const uint32_t ch = 2 * s + g2;
+    const f16x8 a = __builtin_bit_cast( f16x8, wtile[r * 16 + ( ch ^ ( r & 15 ) )] );
+#pragma unroll
+    for ( int t = 0; t < 2; t++ ) {
+      const uint32_t col = 32 * t + r;
+      const f16x8 b = __builtin_bit_cast( f16x8, xtile[col * 16 + ( ch ^ ( col & 15 ) )] );
+      acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16( a, b, acc[t], 0, 0, 0 );
+    }
+  }
+}
+
+// grid: (row slabs, column slabs, k splits).  s % 256 == 0, 16-byte aligned operands.
+template<bool SPLIT>
+__global__ __launch_bounds__( 256, 2 ) void gemm_stream_kernel( __half* __restrict__ xout,
+                                                             float* __restrict__ partial,
+                                                             const __half* __restrict__ x,
+                                                             const __half* __restrict__ w,
+                                                             uint32_t s,
+                                                             uint32_t r,
+                                                             uint32_t b,
+                                                             uint32_t k_per_split )
+{
+  __shared__ uint4 s_x[2][COLS * 16]; // 2 x 16 KiB
+  __shared__ uint4 s_w[4][32 * 16];   // 4 x 8 KiB, one per wave
+
+  const uint32_t wave = threadIdx.x >> 6;
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t row0 = blockIdx.x * WG_ROWS + wave * 32;
+  const uint32_t col0 = blockIdx.y * COLS;
+  const uint32_t k_begin = blockIdx.z * k_per_split;
+  const uint32_t k_end = min( s, k_begin + k_per_split );
+  uint4* wtile = s_w[wave];
+
+  f32x16 acc[2];
+#pragma unroll
+  for ( int t = 0; t < 2; t++ ) {
+#pragma unroll
+    for ( int i = 0; i < 16; i++ ) {
+      acc[t][i] = 0.0f;
+    }
+  }
+
+  // Two weight register sets: while slab i is consumed out of one, slab i+1 is in flight into the
+  // other.  Loads retire in order, so the issue order matters: the weight loads of slab i+1 go out
+  // first in iteration i, the activation halves of slab i+1 follow as their registers are staged;
+  // everything iteration i+1 waits for is then older than the weight loads it issues itself.
+  WSlab wr[2];
+  XSlab xr;
+  load_x_slab( xr, x, s, col0, b, k_begin, k_end );
+  load_w_slab( wr[0], w, s, row0, r, k_begin, k_end );
+
+  for ( uint32_t k0 = k_begin; k0 < k_end; k0 += 2 * SLAB_K ) {
+#pragma unroll
+    for ( int set = 0; set < 2; set++ ) {
+      const uint32_t ks = k0 + set * SLAB_K;
+      if ( ks < k_end ) { // uniform across the work-group
+        load_w_slab( wr[set ^ 1], w, s, row0, r, ks + SLAB_K, k_end );
+#pragma unroll
+        for ( int h = 0; h < 2; h++ ) {
+          stage_x_half( s_x[h], xr, h );
+          stage_w_half( wtile, wr[set], h );
+          load_x_half( xr, x, s, col0, b, ks + SLAB_K, k_end, h ); // same registers, next slab
+          __syncthreads();
+          half_mfma( acc, wtile, s_x[h] );
+        }
+      }
+    }
+  }
+  // acc[t][v]: row = 8*(v/4) + 4*(lane/32) + v%4 of the wave's 32, column = 32*t + lane%32
+  const uint32_t g2 = lane >> 5;
+#pragma unroll
+  for ( int t = 0; t < 2; t++ ) {
+    const uint32_t col = col0 + 32 * t + ( lane & 31 );
+    if ( col >= b ) {
+      continue;
+    }
+#pragma unroll
+    for ( int q4 = 0; q4 < 4; q4++ ) {
+      const uint32_t row = row0 + 8 * q4 + 4 * g2;
+      if ( SPLIT ) {
+        float* dst = partial + ( (uint64_t)blockIdx.z * b + col ) * r + row;
+        if ( row + 3 < r ) {
+          *reinterpret_cast<float4*>( dst ) = make_float4( acc[t][4 * q4], acc[t][4 * q4 + 1], acc[t][4 * q4 + 2], acc[t][4 * q4 + 3] );
+        } else {
+          for ( int i = 0; i < 4; i++ ) {
+            if ( row + i < r ) {
+              dst[i] = acc[t][4 * q4 + i];
+            }
+          }
+        }
+      } else {
+        __half* dst = xout + (uint64_t)col * r + row;
+        if ( row + 3 < r ) {
+          union
+          {
+            uint2 raw;
+            __half h[4];
+          } o;
+#pragma unroll
+          for ( int i = 0; i < 4; i++ ) {
+            o.h[i] = __float2half_rn( acc[t][4 * q4 + i] );
+          }
+          *reinterpret_cast<uint2*>( dst ) = o.raw;
+        } else {
+          for ( int i = 0; i < 4; i++ ) {
+            if ( row + i < r ) {
+              dst[i] = __float2half_rn( acc[t][4 * q4 + i] );
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
+int g_target_wgs = 256;
+
+void launch( dim3 grid, hipStream_t st, bool split, __half* xout, float* partial, const __half* x, const __half* w, uint32_t s, uint32_t r, uint32_t b,
+             uint32_t k_per_split )
+{
+  if ( split ) {
+    gemm_stream_kernel<true><<<grid, 256, 0, st>>>( xout, partial, x, w, s, r, b, k_per_split );
+  } else {
+    gemm_stream_kernel<false><<<grid, 256, 0, st>>>( xout, partial, x, w, s, r, b, k_per_split );
+  }
+}
+
+} // namespace
+
+bool gemm_stream_applicable( uint64_t s, uint64_t r, uint64_t b, const void* x, const void* w, const void* xout )
+{
+  (void)b;
+  return s % SLAB_K == 0 && r % 4 == 0 && ( ( reinterpret_cast<uintptr_t>( x ) | reinterpret_cast<uintptr_t>( w ) | reinterpret_cast<uintptr_t>( xout ) ) & 15u ) == 0;
+}
+
+// picks the K split; returns the number of splits and k per split
+void gemm_stream_plan( uint64_t s, uint64_t r, uint64_t b, uint32_t* splits_out, uint32_t* k_per_split_out )
+{
+  const uint64_t tiles = ( ( r + WG_ROWS - 1 ) / WG_ROWS ) * ( ( b + COLS - 1 ) / COLS );
+  uint32_t splits = 1;
+  if ( tiles < (uint64_t)g_target_wgs ) {
+    splits = (uint32_t)( ( g_target_wgs + tiles - 1 ) / tiles );
+    const uint32_t max_by_k = (uint32_t)std::max<uint64_t>( 1, s / ( 4 * SLAB_K ) ); // at least 4 slabs per work-group
+    splits = std::min( splits, max_by_k );
+  }
+  uint32_t k_per_split = (uint32_t)( ( s + splits - 1 ) / splits );
+  k_per_split = ( k_per_split + SLAB_K - 1 ) / SLAB_K * SLAB_K;
+  *splits_out = (uint32_t)( ( s + k_per_split - 1 ) / k_per_split );
+  *k_per_split_out = k_per_split;
+}
+
+int gemm_stream_launch( __half* xout, float* partial, const __half* x, const __half* w, uint64_t s, uint64_t r, uint64_t b, uint32_t splits,
+                        uint32_t k_per_split, hipStream_t st )
+{
+  const dim3 grid( (unsigned)( ( r + WG_ROWS - 1 ) / WG_ROWS ), (unsigned)( ( b + COLS - 1 ) / COLS ), splits );
+  GH_REQUIRE( grid.y <= 65535 && grid.z <= 65535, "gh_matmul: grid too large" );
+  const bool split = splits > 1;
+  launch( grid, st, split, xout, partial, x, w, (uint32_t)s, (uint32_t)r, (uint32_t)b, k_per_split );
+  GH_LAUNCH_CHECK();
+  return GH_OK;
+}
+
+void gemm_stream_tuning( int target_wgs, int depth )
+{
+  if ( target_wgs > 0 ) {
+    g_target_wgs = target_wgs;
+  }
+  (void)depth;
+}
+
+} // namespace gh

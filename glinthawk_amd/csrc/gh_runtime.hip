@@ -32,9 +32,9 @@ int g_next_slot = 0;
 std::vector<int> g_unfenced;
 
 // ---- attention kernel timer ----------------------------------------------------------------
-constexpr int TIMER_PAIRS = 8192;
+constexpr int TIMER_SLOTS = 8192;
 bool g_timing = false;
-std::vector<hipEvent_t> g_ev_begin, g_ev_end;
+std::vector<hipEvent_t> g_events; // 3 per slot
 int g_ev_used = 0;
 
 } // namespace
@@ -121,35 +121,31 @@ int stage_fence( hipStream_t stream )
   return GH_OK;
 }
 
-// timer hooks used by gh_attn_decode
-int timer_begin( hipStream_t stream, int* pair_out )
+// timer hook used by gh_attn_decode: which = 0 claims a slot and records its first event
+int timer_mark( hipStream_t stream, int* slot_inout, int which )
 {
-  *pair_out = -1;
-  if ( !g_timing ) {
+  if ( which == 0 ) {
+    *slot_inout = -1;
+    if ( !g_timing ) {
+      return GH_OK;
+    }
+    std::lock_guard<std::mutex> lock( g_mutex );
+    if ( g_ev_used >= TIMER_SLOTS ) {
+      return GH_OK; // stop sampling; the mean over the recorded calls stays valid
+    }
+    if ( (int)g_events.size() < 3 * ( g_ev_used + 1 ) ) {
+      for ( int k = 0; k < 3; k++ ) {
+        hipEvent_t e;
+        GH_HIP( hipEventCreate( &e ) );
+        g_events.push_back( e );
+      }
+    }
+    *slot_inout = g_ev_used++;
+  }
+  if ( *slot_inout < 0 ) {
     return GH_OK;
   }
-  std::lock_guard<std::mutex> lock( g_mutex );
-  if ( g_ev_used >= TIMER_PAIRS ) {
-    return GH_OK; // silently stop sampling; the mean over the recorded pairs stays valid
-  }
-  if ( (int)g_ev_begin.size() <= g_ev_used ) {
-    hipEvent_t a, b;
-    GH_HIP( hipEventCreate( &a ) );
-    GH_HIP( hipEventCreate( &b ) );
-    g_ev_begin.push_back( a );
-    g_ev_end.push_back( b );
-  }
-  *pair_out = g_ev_used++;
-  GH_HIP( hipEventRecord( g_ev_begin[*pair_out], stream ) );
-  return GH_OK;
-}
-
-int timer_end( hipStream_t stream, int pair )
-{
-  if ( pair < 0 ) {
-    return GH_OK;
-  }
-  GH_HIP( hipEventRecord( g_ev_end[pair], stream ) );
+  GH_HIP( hipEventRecord( g_events[3 * ( *slot_inout ) + which], stream ) );
   return GH_OK;
 }
 
@@ -404,18 +400,23 @@ int gh_attn_timing_reset( void )
   return GH_OK;
 }
 
-int gh_attn_timing_read( double* total_ms, uint64_t* launches )
+int gh_attn_timing_read( double* kernel_ms, double* merge_ms, uint64_t* launches )
 {
   std::lock_guard<std::mutex> lock( g_mutex );
-  double total = 0.0;
+  double k_total = 0.0, m_total = 0.0;
   for ( int i = 0; i < g_ev_used; i++ ) {
-    GH_HIP( hipEventSynchronize( g_ev_end[i] ) );
+    GH_HIP( hipEventSynchronize( g_events[3 * i + 2] ) );
     float ms = 0.0f;
-    GH_HIP( hipEventElapsedTime( &ms, g_ev_begin[i], g_ev_end[i] ) );
-    total += ms;
+    GH_HIP( hipEventElapsedTime( &ms, g_events[3 * i], g_events[3 * i + 1] ) );
+    k_total += ms;
+    GH_HIP( hipEventElapsedTime( &ms, g_events[3 * i + 1], g_events[3 * i + 2] ) );
+    m_total += ms;
   }
-  if ( total_ms ) {
-    *total_ms = total;
+  if ( kernel_ms ) {
+    *kernel_ms = k_total;
+  }
+  if ( merge_ms ) {
+    *merge_ms = m_total;
   }
   if ( launches ) {
     *launches = (uint64_t)g_ev_used;

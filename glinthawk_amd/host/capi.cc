@@ -25,6 +25,7 @@ struct StageBase
   virtual void new_state( uint32_t batch, uint32_t next_layer, int next_stage ) = 0;
   virtual void set_prompt( size_t i, uint32_t context_id, uint32_t token, uint32_t pos, float temp, uint32_t plen, uint32_t mcl ) = 0;
   virtual void discard( size_t i ) = 0;
+  virtual void set_next( uint32_t layer, int stage ) = 0;
   virtual int acquire_contexts() = 0;
   virtual int forward( int which ) = 0;
   virtual void* buffer( int which, uint64_t* bytes, bool allocate ) = 0;
@@ -74,6 +75,11 @@ struct StageImpl : StageBase
     state.set_prompt( i, context_id, token, pos, temp, plen, mcl );
   }
   void discard( size_t i ) override { state.discard( i ); }
+  void set_next( uint32_t layer, int stage ) override
+  {
+    state.set_next_layer( layer );
+    state.set_next_stage( static_cast<InferenceStage>( stage ) );
+  }
 
   int acquire_contexts() override
   {
@@ -294,6 +300,7 @@ void glint_stage_set_prompt( void* h, uint32_t row, uint32_t context_id, uint32_
   static_cast<StageBase*>( h )->set_prompt( row, context_id, token, pos, temperature, prompt_length, max_completion_length );
 }
 void glint_stage_discard( void* h, uint32_t row ) { static_cast<StageBase*>( h )->discard( row ); }
+void glint_stage_set_next( void* h, uint32_t layer, int stage ) { static_cast<StageBase*>( h )->set_next( layer, stage ); }
 int glint_stage_acquire_contexts( void* h ) { return static_cast<StageBase*>( h )->acquire_contexts(); }
 int glint_stage_forward( void* h, int which ) { return static_cast<StageBase*>( h )->forward( which ); }
 void* glint_stage_buffer( void* h, int which, uint64_t* bytes, int allocate ) { return static_cast<StageBase*>( h )->buffer( which, bytes, allocate != 0 ); }

@@ -44,6 +44,7 @@ def host_lib() -> C.CDLL:
             "glint_stage_new_state": (None, [vp, u32, u32, C.c_int]),
             "glint_stage_set_prompt": (None, [vp, u32, u32, u32, u32, C.c_float, u32, u32]),
             "glint_stage_discard": (None, [vp, u32]),
+            "glint_stage_set_next": (None, [vp, u32, C.c_int]),
             "glint_stage_acquire_contexts": (C.c_int, [vp]),
             "glint_stage_forward": (C.c_int, [vp, C.c_int]),
             "glint_stage_buffer": (vp, [vp, C.c_int, C.POINTER(u64), C.c_int]),
@@ -118,6 +119,9 @@ class Stage:
 
     def discard(self, row: int) -> None:
         host_lib().glint_stage_discard(self._h, row)
+
+    def set_next(self, layer: int, stage: int = STAGE_PRE) -> None:
+        host_lib().glint_stage_set_next(self._h, layer, stage)
 
     def acquire_contexts(self) -> bool:
         return host_lib().glint_stage_acquire_contexts(self._h) == 0

@@ -130,6 +130,9 @@ int gh_silu( void* hb, const void* hb2, uint64_t hidden_dim, uint64_t batch, gh_
 int gh_argmax( uint32_t* out_host, uint32_t* out_dev, const void* v, uint64_t n, uint64_t batch, gh_dtype dt, gh_stream stream );
 /* Operations::matmul<s,r> / untemplated_matmul  arch/amd64/common/ops.hh:74-93,212-271 :
  * xout(b, r) = sum_p w(r, p) * x(b, p); w row-major (r, s); fp32 accumulate */
+/* tuning hook: kernel 0 auto / 1 tiled / 2 streaming (decode); target number of work-groups for the K split
+ * (<= 0 keeps the current value); prefetch depth 2..4 of the streaming kernel (other values keep it) */
+int gh_gemm_set_tuning( int kernel, int target_workgroups, int depth );
 int gh_matmul( void* xout, const void* x, const void* w, uint64_t s, uint64_t r, uint64_t b, gh_dtype dt, gh_stream stream );
 /* Operations::soft_sample    arch/amd64/common/ops.hh:97-107,273-283 : rows with temperature > 0 get
  * v / T - log(-log(u)), u from a counter-based generator keyed by (seed, row, column).
@@ -189,12 +192,13 @@ int gh_attn_decode( const void* q, const void* const* layer_rows_dev, const uint
 int gh_attn_decode_host( const void* q, const void* const* layer_rows_host, const uint32_t* pos_host, void* xb, uint64_t batch,
                          const gh_shape* shape, gh_dtype dt, void* workspace, uint64_t workspace_bytes, int variant, gh_stream stream );
 
-/* Timing hooks for the benchmark: HIP events recorded on `stream` around the attention kernels of
- * gh_attn_decode (split + merge).  gh_attn_timing_read() synchronises and returns the accumulated
- * kernel milliseconds and launch count since gh_attn_timing_reset(). */
+/* Timing hooks for the benchmark: HIP events recorded on `stream` around the two kernels of
+ * gh_attn_decode.  gh_attn_timing_read() synchronises and returns, accumulated since
+ * gh_attn_timing_reset(): milliseconds in the split-K attention kernel, milliseconds in the merge
+ * kernel (0 when no split was needed) and the number of gh_attn_decode calls sampled. */
 int gh_attn_timing_enable( int on );
 int gh_attn_timing_reset( void );
-int gh_attn_timing_read( double* total_ms, uint64_t* launches );
+int gh_attn_timing_read( double* kernel_ms, double* merge_ms, uint64_t* launches );
 
 #ifdef __cplusplus
 }
