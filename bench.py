@@ -28,6 +28,11 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
 
+# HBM bytes per launch of the dominant kernel, from the FETCH_SIZE / WRITE_SIZE counter passes
+# summarised in profiles/attn_decode_mfma_llama2-70b-gqa-b64-ctx4096_hbm_counters.md (each counter
+# scaled by what it reads for a 1 GiB copy).  Only valid for the workload it was measured on.
+MEASURED_TRAFFIC = {"llama2-70b-gqa-b64-ctx4096": 1086921628}
+
 # the configurations of BASELINE.json that fit one GPU as a single stage
 WORKLOADS = {
     # name: (stage config, first layer, hosted layers, batch, keys attended, description)
@@ -53,6 +58,23 @@ def layer_weight_bytes(shape, elem=2):
     d, h = shape["dim"], shape["hidden_dim"]
     kv_dim = d // (shape["n_heads"] // shape["n_kv_heads"])
     return (2 * d + 2 * d * d + 2 * d * kv_dim + 3 * d * h) * elem
+
+
+def calibration_copy(n_bytes):
+    """A plain device-to-device copy of known size, so that hardware byte counters read under a
+    profiler can be scaled (the copy reads n_bytes and writes n_bytes)."""
+    from glinthawk_amd import _lib, ops
+
+    L = _lib.lib()
+    src, dst = C.c_void_p(), C.c_void_p()
+    _lib.check(L.gh_malloc(C.byref(src), n_bytes))
+    _lib.check(L.gh_malloc(C.byref(dst), n_bytes))
+    _lib.check(L.gh_memset_zero(src, n_bytes, None))
+    for _ in range(3):
+        _lib.check(L.gh_memcpy(dst, src, n_bytes, _lib.GH_D2D, 0, None))
+    ops.sync()
+    _lib.check(L.gh_free(src))
+    _lib.check(L.gh_free(dst))
 
 
 def gpu_bench(workload, steps, warmup):
@@ -194,6 +216,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="llama2-70b-gqa-b64-ctx4096", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibration-copy-mib", type=int, default=0,
+                    help="also run a plain D2D copy of this many MiB (reference point for profiler byte counters)")
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -201,6 +225,10 @@ def main():
               "(the path shards by context with no collective, see DESIGN.md)", file=sys.stderr)
         sys.exit(2)
 
+    if args.calibration_copy_mib > 0:
+        from glinthawk_amd import ops
+        ops.init(0)
+        calibration_copy(args.calibration_copy_mib << 20)
     g = gpu_bench(args.workload, args.steps, args.warmup)
     cfg_name, first, n_hosted, batch, keys, desc = WORKLOADS[args.workload]
 
@@ -233,7 +261,7 @@ def main():
         "attn_kernel_ms": round(g["attn_kernel_ms"], 5),
         "attn_merge_ms": round(g["attn_merge_ms"], 5),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC.get(args.workload),
                      "kernel": "attn_decode (split-K fused decode attention)", "launches_timed": g["attn_launches"],
                      "algorithmic_bytes_per_launch": g["attn_bytes"]},
     }
