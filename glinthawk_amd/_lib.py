@@ -87,6 +87,9 @@ SIGNATURES = {
     "gh_argmax": (_i, [_vp, _vp, _vp, _u64, _u64, _i, _vp]),
     "gh_gemm_set_tuning": (_i, [_i, _i, _i]),
     "gh_matmul": (_i, [_vp, _vp, _vp, _u64, _u64, _u64, _i, _vp]),
+    "gh_matmul_accum": (_i, [_vp, _vp, _vp, _u64, _u64, _u64, _vp, _vp, _i, _vp]),
+    "gh_matmul_silu_gate": (_i, [_vp, _vp, _vp, _u64, _u64, _u64, _i, _vp]),
+    "gh_matmul_qkv_rope_append": (_i, [_vp, _vp, _vp, _vp, _u64, _u64, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _i, _vp]),
     "gh_soft_sample": (_i, [_vp, _vp, _u64, _u64, _u64, _i, _vp]),
     "gh_kv_append": (_i, [_vp, _vp, _u64, _u32, _i, _vp]),
     "gh_kv_append_host": (_i, [_vp, _vp, _u64, _u32, _i, _vp]),

@@ -19,7 +19,7 @@ namespace gh {
 bool gemm_stream_applicable( uint64_t s, uint64_t r, uint64_t b, const void* x, const void* w, const void* xout );
 void gemm_stream_plan( uint64_t s, uint64_t r, uint64_t b, uint32_t* splits_out, uint32_t* k_per_split_out );
 int gemm_stream_launch( __half* xout, float* partial, const __half* x, const __half* w, uint64_t s, uint64_t r, uint64_t b, uint32_t splits,
-                        uint32_t k_per_split, hipStream_t st );
+                        uint32_t k_per_split, bool write_partials, hipStream_t st );
 void gemm_stream_tuning( int target_wgs, int depth );
 
 namespace {
@@ -222,6 +222,87 @@ __global__ __launch_bounds__( 256 ) void gemm_f32_kernel( float* __restrict__ xo
 } // namespace
 } // namespace gh
 
+namespace gh {
+
+// Runs the GEMM proper.  With `want_partials` the result is always left as fp32 partial sums
+// `[splits][b][r]` in the library's workspace (*partial_out, *splits_out) for a fused epilogue;
+// otherwise the kernel may store DType results straight into `xout` (*splits_out == 0 then).
+int gemm_partials( void* xout, const void* x, const void* w, uint64_t s, uint64_t r, uint64_t b, gh_dtype dt, hipStream_t st, bool want_partials,
+                   float** partial_out, uint32_t* splits_out )
+{
+  *partial_out = nullptr;
+  *splits_out = 0;
+  if ( dt == GH_F32 ) {
+    float* dst = static_cast<float*>( xout );
+    if ( want_partials ) {
+      if ( int rc = ensure_workspace( b * r * sizeof( float ), &dst ) ) {
+        return rc;
+      }
+      *partial_out = dst;
+      *splits_out = 1;
+    }
+    gemm_f32_kernel<<<(unsigned)( ( r + 3 ) / 4 ), 256, 0, st>>>( dst, static_cast<const float*>( x ), static_cast<const float*>( w ), (uint32_t)s, (uint32_t)r,
+                                                                 (uint32_t)b );
+    GH_LAUNCH_CHECK();
+    return GH_OK;
+  }
+  GH_REQUIRE( dt == GH_F16, "gh_matmul: unsupported dtype %d", (int)dt );
+
+  if ( g_force_kernel != 1 && gemm_stream_applicable( s, r, b, x, w, xout ? xout : x ) ) {
+    uint32_t splits = 1, k_per_split = 0;
+    gemm_stream_plan( s, r, b, &splits, &k_per_split );
+    float* ws = nullptr;
+    const bool partial = want_partials || splits > 1;
+    if ( partial ) {
+      if ( int rc = ensure_workspace( (uint64_t)splits * b * r * sizeof( float ), &ws ) ) {
+        return rc;
+      }
+      *partial_out = ws;
+      *splits_out = splits;
+    }
+    return gemm_stream_launch( static_cast<__half*>( xout ), ws, static_cast<const __half*>( x ), static_cast<const __half*>( w ), s, r, b, splits, k_per_split,
+                               partial, st );
+  }
+  GH_REQUIRE( g_force_kernel != 2, "gh_matmul: the streaming kernel needs s %% 256 == 0, r %% 4 == 0 and 16-byte aligned operands" );
+
+  const bool k_vec_ok = ( s % 8 == 0 ) && ( ( reinterpret_cast<uintptr_t>( x ) | reinterpret_cast<uintptr_t>( w ) ) & 15u ) == 0;
+  const uint32_t grid_m = (uint32_t)( ( r + BM - 1 ) / BM );
+  const uint32_t grid_n = (uint32_t)( ( b + BN - 1 ) / BN );
+  GH_REQUIRE( grid_n <= 65535, "gh_matmul: batch too large" );
+  // split K until there are about 1024 work-groups (4 per CU), keeping at least 1024 k per split
+  uint32_t splits = 1;
+  const uint64_t tiles = (uint64_t)grid_m * grid_n;
+  if ( tiles < 1024 ) {
+    splits = (uint32_t)( ( 1024 + tiles - 1 ) / tiles );
+    const uint32_t max_by_k = (uint32_t)std::max<uint64_t>( 1, s / 1024 );
+    splits = std::min( splits, max_by_k );
+    splits = std::min<uint32_t>( splits, 16 );
+  }
+  uint32_t k_per_split = (uint32_t)( ( s + splits - 1 ) / splits );
+  k_per_split = ( k_per_split + BK - 1 ) / BK * BK;
+  splits = (uint32_t)( ( s + k_per_split - 1 ) / k_per_split );
+
+  const dim3 grid( grid_m, grid_n, splits );
+  if ( splits == 1 && !want_partials ) {
+    gemm_f16_kernel<false><<<grid, 256, 0, st>>>( static_cast<__half*>( xout ), nullptr, static_cast<const __half*>( x ), static_cast<const __half*>( w ),
+                                                 (uint32_t)s, (uint32_t)r, (uint32_t)b, k_per_split, k_vec_ok );
+    GH_LAUNCH_CHECK();
+    return GH_OK;
+  }
+  float* ws = nullptr;
+  if ( int rc = ensure_workspace( (uint64_t)splits * b * r * sizeof( float ), &ws ) ) {
+    return rc;
+  }
+  gemm_f16_kernel<true><<<grid, 256, 0, st>>>( nullptr, ws, static_cast<const __half*>( x ), static_cast<const __half*>( w ), (uint32_t)s, (uint32_t)r,
+                                              (uint32_t)b, k_per_split, k_vec_ok );
+  GH_LAUNCH_CHECK();
+  *partial_out = ws;
+  *splits_out = splits;
+  return GH_OK;
+}
+
+} // namespace gh
+
 using namespace gh;
 
 extern "C" {
@@ -244,73 +325,17 @@ int gh_matmul( void* xout, const void* x, const void* w, uint64_t s, uint64_t r,
   GH_REQUIRE( xout && x && w, "gh_matmul: NULL pointer" );
   GH_REQUIRE( s > 0 && s <= 0x7fffffffull && r <= 0x7fffffffull && b <= 0x7fffffffull, "gh_matmul: bad shape" );
   hipStream_t st = as_stream( stream );
-
-  if ( dt == GH_F32 ) {
-    gemm_f32_kernel<<<(unsigned)( ( r + 3 ) / 4 ), 256, 0, st>>>( static_cast<float*>( xout ), static_cast<const float*>( x ), static_cast<const float*>( w ),
-                                                                 (uint32_t)s, (uint32_t)r, (uint32_t)b );
-    GH_LAUNCH_CHECK();
-    return GH_OK;
-  }
-  GH_REQUIRE( dt == GH_F16, "gh_matmul: unsupported dtype %d", (int)dt );
-
-  if ( g_force_kernel != 1 && gemm_stream_applicable( s, r, b, x, w, xout ) ) {
-    uint32_t splits = 1, k_per_split = 0;
-    gemm_stream_plan( s, r, b, &splits, &k_per_split );
-    float* ws = nullptr;
-    if ( splits > 1 ) {
-      if ( int rc = ensure_workspace( (uint64_t)splits * b * r * sizeof( float ), &ws ) ) {
-        return rc;
-      }
-    }
-    if ( int rc = gemm_stream_launch( static_cast<__half*>( xout ), ws, static_cast<const __half*>( x ), static_cast<const __half*>( w ), s, r, b, splits,
-                                      k_per_split, st ) ) {
-      return rc;
-    }
-    if ( splits > 1 ) {
-      const uint64_t n = b * r;
-      const unsigned blocks = (unsigned)std::min<uint64_t>( ( n + 255 ) / 256, 4096 );
-      gemm_reduce_kernel<<<blocks, 256, 0, st>>>( static_cast<__half*>( xout ), ws, n, splits );
-      GH_LAUNCH_CHECK();
-    }
-    return GH_OK;
-  }
-  GH_REQUIRE( g_force_kernel != 2, "gh_matmul: the streaming kernel needs s %% 128 == 0, r %% 4 == 0 and 16-byte aligned operands" );
-
-  const bool k_vec_ok = ( s % 8 == 0 ) && ( ( reinterpret_cast<uintptr_t>( x ) | reinterpret_cast<uintptr_t>( w ) ) & 15u ) == 0;
-  const uint32_t grid_m = (uint32_t)( ( r + BM - 1 ) / BM );
-  const uint32_t grid_n = (uint32_t)( ( b + BN - 1 ) / BN );
-  GH_REQUIRE( grid_n <= 65535, "gh_matmul: batch too large" );
-  // split K until there are about 1024 work-groups (4 per CU), keeping at least 1024 k per split
-  uint32_t splits = 1;
-  const uint64_t tiles = (uint64_t)grid_m * grid_n;
-  if ( tiles < 1024 ) {
-    splits = (uint32_t)( ( 1024 + tiles - 1 ) / tiles );
-    const uint32_t max_by_k = (uint32_t)std::max<uint64_t>( 1, s / 1024 );
-    splits = std::min( splits, max_by_k );
-    splits = std::min<uint32_t>( splits, 16 );
-  }
-  uint32_t k_per_split = (uint32_t)( ( s + splits - 1 ) / splits );
-  k_per_split = ( k_per_split + BK - 1 ) / BK * BK;
-  splits = (uint32_t)( ( s + k_per_split - 1 ) / k_per_split );
-
-  const dim3 grid( grid_m, grid_n, splits );
-  if ( splits == 1 ) {
-    gemm_f16_kernel<false><<<grid, 256, 0, st>>>( static_cast<__half*>( xout ), nullptr, static_cast<const __half*>( x ), static_cast<const __half*>( w ),
-                                                 (uint32_t)s, (uint32_t)r, (uint32_t)b, k_per_split, k_vec_ok );
-    GH_LAUNCH_CHECK();
-    return GH_OK;
-  }
-  float* ws = nullptr;
-  if ( int rc = ensure_workspace( (uint64_t)splits * b * r * sizeof( float ), &ws ) ) {
+  float* partial = nullptr;
+  uint32_t splits = 0;
+  if ( int rc = gemm_partials( xout, x, w, s, r, b, dt, st, false, &partial, &splits ) ) {
     return rc;
   }
-  gemm_f16_kernel<true><<<grid, 256, 0, st>>>( nullptr, ws, static_cast<const __half*>( x ), static_cast<const __half*>( w ), (uint32_t)s, (uint32_t)r,
-                                              (uint32_t)b, k_per_split, k_vec_ok );
-  GH_LAUNCH_CHECK();
-  const uint64_t n = b * r;
-  const unsigned blocks = (unsigned)std::min<uint64_t>( ( n + 255 ) / 256, 4096 );
-  gemm_reduce_kernel<<<blocks, 256, 0, st>>>( static_cast<__half*>( xout ), ws, n, splits );
-  GH_LAUNCH_CHECK();
+  if ( splits > 0 ) { // only the f16 kernels leave partials when not asked to
+    const uint64_t n = b * r;
+    const unsigned blocks = (unsigned)std::min<uint64_t>( ( n + 255 ) / 256, 4096 );
+    gemm_reduce_kernel<<<blocks, 256, 0, st>>>( static_cast<__half*>( xout ), partial, n, splits );
+    GH_LAUNCH_CHECK();
+  }
   return GH_OK;
 }
 

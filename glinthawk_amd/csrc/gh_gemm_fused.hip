@@ -1,0 +1,291 @@
+// Projection GEMMs fused with the ops that follow them in the reference's layer
+// (models/llama2/model.hh:326-427).  The GEMM kernel leaves fp32 partial sums [splits][b][r]; one
+// epilogue kernel per call sums the splits and applies the follow-up ops, so a layer needs 10
+// launches instead of 21.  Rounding points are those of the unfused sequence: every matmul result
+// is rounded to DType first (the reference stores it), later math is fp32 with one rounding per store.
+#include "gh_common.h"
+
+namespace gh {
+
+int gemm_partials( void* xout, const void* x, const void* w, uint64_t s, uint64_t r, uint64_t b, gh_dtype dt, hipStream_t st, bool want_partials,
+                   float** partial_out, uint32_t* splits_out );
+
+namespace {
+
+__device__ __forceinline__ float sum_splits( const float* __restrict__ partial, uint64_t idx, uint64_t n, uint32_t splits )
+{
+  float acc = 0.0f;
+  for ( uint32_t k = 0; k < splits; k++ ) {
+    acc += partial[(uint64_t)k * n + idx];
+  }
+  return acc;
+}
+
+// residual(b, r) += DType(matmul); optionally norm_out = rmsnorm(residual) * norm_weight.
+// block <-> batch row, 1024 threads, four columns per thread and pass so that a row's partials are
+// fetched with independent 16-byte loads (the kernel is latency-bound: only `b` blocks exist)
+constexpr int EPI_THREADS = 1024;
+
+template<typename T>
+__global__ __launch_bounds__( EPI_THREADS ) void epi_accum_norm_kernel( T* __restrict__ residual,
+                                                                       const float* __restrict__ partial,
+                                                                       uint32_t r,
+                                                                       uint32_t b,
+                                                                       uint32_t splits,
+                                                                       T* __restrict__ norm_out,
+                                                                       const T* __restrict__ norm_weight )
+{
+  __shared__ float smem[EPI_THREADS / WAVE];
+  const uint32_t row = blockIdx.x;
+  const uint64_t n = (uint64_t)b * r;
+  T* res = residual + (uint64_t)row * r;
+  const float* prow = partial + (uint64_t)row * r;
+  const bool vec = ( r % 4 == 0 ) && ( ( reinterpret_cast<uintptr_t>( res ) & 7u ) == 0 );
+  float ss = 0.0f;
+  if ( vec ) {
+    for ( uint32_t j = threadIdx.x * 4; j < r; j += blockDim.x * 4 ) {
+      float4 acc = make_float4( 0.0f, 0.0f, 0.0f, 0.0f );
+      for ( uint32_t k = 0; k < splits; k++ ) {
+        const float4 p = *reinterpret_cast<const float4*>( prow + (uint64_t)k * n + j );
+        acc.x += p.x;
+        acc.y += p.y;
+        acc.z += p.z;
+        acc.w += p.w;
+      }
+      const float y[4] = { acc.x, acc.y, acc.z, acc.w };
+#pragma unroll
+      for ( int e = 0; e < 4; e++ ) {
+        const T v = from_f32<T>( to_f32( res[j + e] ) + to_f32( from_f32<T>( y[e] ) ) ); // xb2 = DType(matmul), then accum
+        res[j + e] = v;
+        const float f = to_f32( v );
+        ss += f * f;
+      }
+    }
+  } else {
+    for ( uint32_t j = threadIdx.x; j < r; j += blockDim.x ) {
+      const T y = from_f32<T>( sum_splits( partial, (uint64_t)row * r + j, n, splits ) );
+      const T v = from_f32<T>( to_f32( res[j] ) + to_f32( y ) );
+      res[j] = v;
+      const float f = to_f32( v );
+      ss += f * f;
+    }
+  }
+  if ( norm_out == nullptr ) {
+    return;
+  }
+  ss = wave_sum( ss );
+  if ( threadIdx.x % WAVE == 0 ) {
+    smem[threadIdx.x / WAVE] = ss;
+  }
+  __syncthreads();
+  ss = 0.0f;
+  for ( int w = 0; w < EPI_THREADS / WAVE; w++ ) {
+    ss += smem[w];
+  }
+  ss = ss / (float)r + 1e-5f;
+  const float inv = 1.0f / sqrtf( ss );
+  T* o = norm_out + (uint64_t)row * r;
+  // each thread re-reads only what it wrote itself
+  if ( vec ) {
+    for ( uint32_t j = threadIdx.x * 4; j < r; j += blockDim.x * 4 ) {
+#pragma unroll
+      for ( int e = 0; e < 4; e++ ) {
+        o[j + e] = from_f32<T>( to_f32( norm_weight[j + e] ) * ( inv * to_f32( res[j + e] ) ) );
+      }
+    }
+  } else {
+    for ( uint32_t j = threadIdx.x; j < r; j += blockDim.x ) {
+      o[j] = from_f32<T>( to_f32( norm_weight[j] ) * ( inv * to_f32( res[j] ) ) );
+    }
+  }
+}
+
+// hb(b, hidden) = DType( silu(DType(y1)) * DType(y3) ), partial rows [0, hidden) = w1, [hidden, 2 hidden) = w3
+template<typename T>
+__global__ __launch_bounds__( 256 ) void epi_silu_gate_kernel( T* __restrict__ hb, const float* __restrict__ partial, uint32_t hidden, uint32_t b, uint32_t splits )
+{
+  const uint64_t n = (uint64_t)b * 2 * hidden;
+  const uint64_t total = (uint64_t)b * hidden;
+  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  for ( uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride ) {
+    const uint64_t row = i / hidden, j = i % hidden;
+    const float x = to_f32( from_f32<T>( sum_splits( partial, row * 2 * hidden + j, n, splits ) ) );
+    const float y = to_f32( from_f32<T>( sum_splits( partial, row * 2 * hidden + hidden + j, n, splits ) ) );
+    hb[i] = from_f32<T>( x / ( 1.0f + __expf( -x ) ) * y );
+  }
+}
+
+// partial rows: [0, dim) q, [dim, dim + kv_dim) k, [dim + kv_dim, dim + 2 kv_dim) v.  thread <-> pair of columns.
+// q(b, dim) = rope(DType(q)); cache row = [rope(DType(k)) | DType(v)]; kv_out (optional) = [DType(k) | DType(v)] unrotated
+template<typename T>
+__global__ __launch_bounds__( 256 ) void epi_qkv_kernel( T* __restrict__ q,
+                                                        T* __restrict__ kv_out,
+                                                        const float* __restrict__ partial,
+                                                        uint32_t b,
+                                                        uint32_t splits,
+                                                        const uint32_t* __restrict__ pos,
+                                                        const T* __restrict__ freq_real,
+                                                        const T* __restrict__ freq_imag,
+                                                        void* const* __restrict__ token_rows,
+                                                        uint32_t dim,
+                                                        uint32_t kv_dim,
+                                                        uint32_t head_size )
+{
+  const uint32_t ctx = blockIdx.y;
+  const uint32_t r = dim + 2 * kv_dim;
+  const uint64_t n = (uint64_t)b * r;
+  const uint32_t pair = blockIdx.x * blockDim.x + threadIdx.x;
+  if ( pair >= r / 2 ) {
+    return;
+  }
+  const uint32_t col = 2 * pair;
+  const T y0 = from_f32<T>( sum_splits( partial, (uint64_t)ctx * r + col, n, splits ) );
+  const T y1 = from_f32<T>( sum_splits( partial, (uint64_t)ctx * r + col + 1, n, splits ) );
+  T* row = static_cast<T*>( token_rows[ctx] );
+
+  if ( kv_out != nullptr && col >= dim ) {
+    kv_out[(uint64_t)ctx * 2 * kv_dim + ( col - dim )] = y0;
+    kv_out[(uint64_t)ctx * 2 * kv_dim + ( col - dim ) + 1] = y1;
+  }
+  if ( col >= dim + kv_dim ) { // V: stored as is
+    if ( row != nullptr ) {
+      row[col - dim] = y0;
+      row[col - dim + 1] = y1;
+    }
+    return;
+  }
+  // q and k rotate by the angle of (position, pair index inside the head); an empty context keeps its
+  // query unrotated and has no row, as in the unfused ops
+  T o0 = y0, o1 = y1;
+  if ( row != nullptr ) {
+    const uint32_t k = ( col % head_size ) / 2;
+    const uint64_t p = pos[ctx];
+    const float fcr = to_f32( freq_real[p * ( head_size / 2 ) + k] );
+    const float fci = to_f32( freq_imag[p * ( head_size / 2 ) + k] );
+    const float a = to_f32( y0 ), c = to_f32( y1 );
+    o0 = from_f32<T>( a * fcr - c * fci );
+    o1 = from_f32<T>( a * fci + c * fcr );
+  }
+  if ( col < dim ) {
+    q[(uint64_t)ctx * dim + col] = o0;
+    q[(uint64_t)ctx * dim + col + 1] = o1;
+  } else if ( row != nullptr ) {
+    row[col - dim] = o0;
+    row[col - dim + 1] = o1;
+  }
+}
+
+int check_common( const void* x, const void* w, uint64_t s, uint64_t r, uint64_t b, gh_dtype dt, const char* who )
+{
+  GH_REQUIRE( x && w, "%s: NULL pointer", who );
+  GH_REQUIRE( dt == GH_F16 || dt == GH_F32, "%s: unsupported dtype %d", who, (int)dt );
+  GH_REQUIRE( s > 0 && s <= 0x7fffffffull && r > 0 && r <= 0x7fffffffull && b <= 65535, "%s: bad shape", who );
+  return GH_OK;
+}
+
+} // namespace
+} // namespace gh
+
+using namespace gh;
+
+extern "C" {
+
+int gh_matmul_accum( void* residual, const void* x, const void* w, uint64_t s, uint64_t r, uint64_t b, void* norm_out, const void* norm_weight,
+                     gh_dtype dt, gh_stream stream )
+{
+  if ( int rc = ensure_init() ) {
+    return rc;
+  }
+  if ( b == 0 ) {
+    return GH_OK;
+  }
+  if ( int rc = check_common( x, w, s, r, b, dt, "gh_matmul_accum" ) ) {
+    return rc;
+  }
+  GH_REQUIRE( residual != nullptr, "gh_matmul_accum: NULL residual" );
+  GH_REQUIRE( ( norm_out == nullptr ) == ( norm_weight == nullptr ), "gh_matmul_accum: norm_out and norm_weight go together" );
+  hipStream_t st = as_stream( stream );
+  float* partial = nullptr;
+  uint32_t splits = 0;
+  if ( int rc = gemm_partials( nullptr, x, w, s, r, b, dt, st, true, &partial, &splits ) ) {
+    return rc;
+  }
+  if ( dt == GH_F16 ) {
+    epi_accum_norm_kernel<__half><<<(unsigned)b, EPI_THREADS, 0, st>>>( static_cast<__half*>( residual ), partial, (uint32_t)r, (uint32_t)b, splits,
+                                                               static_cast<__half*>( norm_out ), static_cast<const __half*>( norm_weight ) );
+  } else {
+    epi_accum_norm_kernel<float><<<(unsigned)b, EPI_THREADS, 0, st>>>( static_cast<float*>( residual ), partial, (uint32_t)r, (uint32_t)b, splits,
+                                                              static_cast<float*>( norm_out ), static_cast<const float*>( norm_weight ) );
+  }
+  GH_LAUNCH_CHECK();
+  return GH_OK;
+}
+
+int gh_matmul_silu_gate( void* hb, const void* x, const void* w13, uint64_t s, uint64_t hidden_dim, uint64_t b, gh_dtype dt, gh_stream stream )
+{
+  if ( int rc = ensure_init() ) {
+    return rc;
+  }
+  if ( b == 0 ) {
+    return GH_OK;
+  }
+  if ( int rc = check_common( x, w13, s, 2 * hidden_dim, b, dt, "gh_matmul_silu_gate" ) ) {
+    return rc;
+  }
+  GH_REQUIRE( hb != nullptr, "gh_matmul_silu_gate: NULL output" );
+  hipStream_t st = as_stream( stream );
+  float* partial = nullptr;
+  uint32_t splits = 0;
+  if ( int rc = gemm_partials( nullptr, x, w13, s, 2 * hidden_dim, b, dt, st, true, &partial, &splits ) ) {
+    return rc;
+  }
+  const uint64_t total = b * hidden_dim;
+  const unsigned blocks = (unsigned)std::min<uint64_t>( ( total + 255 ) / 256, 8192 );
+  if ( dt == GH_F16 ) {
+    epi_silu_gate_kernel<__half><<<blocks, 256, 0, st>>>( static_cast<__half*>( hb ), partial, (uint32_t)hidden_dim, (uint32_t)b, splits );
+  } else {
+    epi_silu_gate_kernel<float><<<blocks, 256, 0, st>>>( static_cast<float*>( hb ), partial, (uint32_t)hidden_dim, (uint32_t)b, splits );
+  }
+  GH_LAUNCH_CHECK();
+  return GH_OK;
+}
+
+int gh_matmul_qkv_rope_append( void* q, void* kv_out, const void* x, const void* wqkv, uint64_t s, uint64_t b, const uint32_t* pos_dev, const void* freq_real,
+                               const void* freq_imag, void* const* token_rows_dev, uint32_t n_kv_heads, uint32_t gqa_size, uint32_t head_size, gh_dtype dt,
+                               gh_stream stream )
+{
+  if ( int rc = ensure_init() ) {
+    return rc;
+  }
+  if ( b == 0 ) {
+    return GH_OK;
+  }
+  GH_REQUIRE( n_kv_heads > 0 && gqa_size > 0 && head_size > 0 && head_size % 2 == 0, "gh_matmul_qkv_rope_append: bad head shape" );
+  const uint64_t kv_dim = (uint64_t)n_kv_heads * head_size;
+  const uint64_t dim = kv_dim * gqa_size;
+  const uint64_t r = dim + 2 * kv_dim;
+  if ( int rc = check_common( x, wqkv, s, r, b, dt, "gh_matmul_qkv_rope_append" ) ) {
+    return rc;
+  }
+  GH_REQUIRE( q && pos_dev && freq_real && freq_imag && token_rows_dev, "gh_matmul_qkv_rope_append: NULL pointer" );
+  hipStream_t st = as_stream( stream );
+  float* partial = nullptr;
+  uint32_t splits = 0;
+  if ( int rc = gemm_partials( nullptr, x, wqkv, s, r, b, dt, st, true, &partial, &splits ) ) {
+    return rc;
+  }
+  const dim3 grid( (unsigned)( ( r / 2 + 255 ) / 256 ), (unsigned)b );
+  if ( dt == GH_F16 ) {
+    epi_qkv_kernel<__half><<<grid, 256, 0, st>>>( static_cast<__half*>( q ), static_cast<__half*>( kv_out ), partial, (uint32_t)b, splits, pos_dev,
+                                                 static_cast<const __half*>( freq_real ), static_cast<const __half*>( freq_imag ), token_rows_dev, (uint32_t)dim,
+                                                 (uint32_t)kv_dim, head_size );
+  } else {
+    epi_qkv_kernel<float><<<grid, 256, 0, st>>>( static_cast<float*>( q ), static_cast<float*>( kv_out ), partial, (uint32_t)b, splits, pos_dev,
+                                                static_cast<const float*>( freq_real ), static_cast<const float*>( freq_imag ), token_rows_dev, (uint32_t)dim,
+                                                (uint32_t)kv_dim, head_size );
+  }
+  GH_LAUNCH_CHECK();
+  return GH_OK;
+}
+
+} // extern "C"

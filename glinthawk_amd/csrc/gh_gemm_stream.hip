@@ -262,11 +262,11 @@ void gemm_stream_plan( uint64_t s, uint64_t r, uint64_t b, uint32_t* splits_out,
 }
 
 int gemm_stream_launch( __half* xout, float* partial, const __half* x, const __half* w, uint64_t s, uint64_t r, uint64_t b, uint32_t splits,
-                        uint32_t k_per_split, hipStream_t st )
+                        uint32_t k_per_split, bool write_partials, hipStream_t st )
 {
   const dim3 grid( (unsigned)( ( r + WG_ROWS - 1 ) / WG_ROWS ), (unsigned)( ( b + COLS - 1 ) / COLS ), splits );
   GH_REQUIRE( grid.y <= 65535 && grid.z <= 65535, "gh_matmul: grid too large" );
-  const bool split = splits > 1;
+  const bool split = write_partials;
   launch( grid, st, split, xout, partial, x, w, (uint32_t)s, (uint32_t)r, (uint32_t)b, k_per_split );
   GH_LAUNCH_CHECK();
   return GH_OK;

@@ -202,6 +202,7 @@ StageBase* make_stage( int dtype, uint32_t first_layer, uint32_t n_hosted, uint3
   auto s = StageSettings<Config>::slice( first_layer, n_hosted, concurrency, max_contexts, with_cls );
   ModelOptions o;
   o.fused_attention = flags & 1u;
+  o.fused_projections = !( flags & 8u );
   o.seed = seed;
   o.weight_std = std;
   return make_for_config<Config>( dtype, flags & 4u, s, o );
@@ -269,7 +270,7 @@ using PagedBookContext = glint::DynamicContext<BookConfig, float16_t, CountingRe
 extern "C" {
 
 // ---- stage harness --------------------------------------------------------------------------
-// flags: 1 fused attention, 2 host the classifier, 4 paged (virtual-memory) contexts
+// flags: 1 fused attention, 2 host the classifier, 4 paged (virtual-memory) contexts, 8 keep the projections unfused
 void* glint_stage_create( const char* config, int dtype, uint32_t first_layer, uint32_t n_hosted, uint32_t concurrency, uint32_t max_contexts,
                           uint32_t flags, uint64_t seed, float weight_std )
 {

@@ -298,6 +298,33 @@ public:
                               GH_ATTN_AUTO, this->stream_ ) );
   }
 
+  // Extensions used by the stage driver: a projection together with the ops that follow it in the
+  // layer (same arithmetic and rounding points as the separate calls, fewer launches).
+  // wo / w2 + accum (+ the rmsnorm that follows): x += xb . w^T; norm_out = rmsnorm(x) * norm_weight
+  template<uint64_t s, uint64_t r>
+  void matmul_accum( DType* x, const DType* xb, const DType* w, const uint64_t batch_size, DType* norm_out = nullptr, const DType* norm_weight = nullptr ) const
+  {
+    GLINT_GH( gh_matmul_accum( x, xb, w, s, r, batch_size, norm_out, norm_weight, gh_type<DType>(), this->stream_ ) );
+  }
+  // w1, w3, silu: hb = silu(xb . w1^T) * (xb . w3^T); w13 holds the rows of w1 followed by those of w3
+  void matmul_silu_gate( DType* hb, const DType* xb, const DType* w13, const uint64_t batch_size ) const
+  {
+    GLINT_GH( gh_matmul_silu_gate( hb, xb, w13, Config::dim, Config::hidden_dim, batch_size, gh_type<DType>(), this->stream_ ) );
+  }
+  // wq, wkv, copy_kv_cache, apply_rope: wqkv holds the rows of wq followed by those of wkv
+  void matmul_qkv_rope_append( DType* q,
+                               const DType* xb,
+                               const DType* wqkv,
+                               const uint64_t batch_size,
+                               const uint32_t* token_positions_dev,
+                               const DType* freq_cis_real,
+                               const DType* freq_cis_imag,
+                               void* const* token_rows_dev ) const
+  {
+    GLINT_GH( gh_matmul_qkv_rope_append( q, nullptr, xb, wqkv, Config::dim, batch_size, token_positions_dev, freq_cis_real, freq_cis_imag, token_rows_dev,
+                                         Config::n_kv_heads, Config::gqa_size, Config::head_size, gh_type<DType>(), this->stream_ ) );
+  }
+
 private:
   // TokenContext / LayerContext are a single pointer each, so an array of them is a pointer table
   static_assert( sizeof( typename ContextType::TokenContextType ) == sizeof( void* ) );

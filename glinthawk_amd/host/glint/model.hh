@@ -93,6 +93,7 @@ struct LayerWeights
 struct ModelOptions
 {
   bool fused_attention { true };  // false: the reference's three unfused ops + score buffer
+  bool fused_projections { true }; // with fused_attention: projections fused with the ops that follow them
   bool allocate_logits { true };  // only needed when the classifier is hosted
   uint64_t seed { 1 };            // random initialisation of weights
   float weight_std { 0.02f };     // N(0, std) for every tensor, as the benchmark configurations say
@@ -182,17 +183,26 @@ public:
       upload_tables( contexts, run );
     }
 
+    const bool fused_layers = options_.fused_attention && options_.fused_projections;
+    if ( fused_layers && !run.empty() ) {
+      // the first attention norm stands alone; every later one rides on the epilogue of the previous w2
+      ops_.template rmsnorm<Config::dim>( xb_, x_, reinterpret_cast<float32_t*>( temp_ ), layers_[run[0]].rms_att_weight, batch_ );
+    }
     for ( size_t k = 0; k < run.size(); k++ ) {
       const size_t l = run[k];
-      for ( size_t i = 0; i < contexts.size(); i++ ) {
-        layer_contexts_[i] = contexts[i]->layer( l );
-        token_contexts_[i] = contexts[i]->layer( l ).token( states.token_pos( i ) );
+      GLINT_CHECK( settings_.hosts( l, InferenceStage::Attention ) && settings_.hosts( l, InferenceStage::PostAttention ) );
+      if ( fused_layers ) {
+        const DType* next_norm = k + 1 < run.size() ? layers_[run[k + 1]].rms_att_weight : nullptr;
+        fused_layer_ops( l, k, next_norm );
+      } else {
+        for ( size_t i = 0; i < contexts.size(); i++ ) {
+          layer_contexts_[i] = contexts[i]->layer( l );
+          token_contexts_[i] = contexts[i]->layer( l ).token( states.token_pos( i ) );
+        }
+        pre_attention_ops( l, true, k );
+        attention_ops( k );
+        post_attention_ops( l );
       }
-      pre_attention_ops( l, true, k );
-      GLINT_CHECK( settings_.hosts( l, InferenceStage::Attention ) );
-      attention_ops( k );
-      GLINT_CHECK( settings_.hosts( l, InferenceStage::PostAttention ) );
-      post_attention_ops( l );
       last = l;
     }
     GLINT_CHECK( last < Config::n_layers );
@@ -334,6 +344,19 @@ private:
     ops_.template silu<Config::hidden_dim>( hb_, hb2_, batch_ );
     ops_.template matmul<Config::hidden_dim, Config::dim>( xb_, hb_, w.w2, batch_ );
     ops_.template accum<Config::dim>( x_, xb_, batch_ );
+  }
+
+  // One whole layer with the projections fused with their follow-up ops: 10 launches instead of 21.
+  // Expects xb_ = rmsnorm(x_) * rms_att_weight on entry; leaves the same for the next layer when
+  // `next_att_norm` is given.
+  void fused_layer_ops( const size_t layer, const size_t table_index, const DType* next_att_norm )
+  {
+    const auto& w = layers_[layer];
+    ops_.matmul_qkv_rope_append( q_, xb_, w.wq, batch_, pos_dev(), base_.freq_cis_real, base_.freq_cis_imag, token_rows_dev( table_index ) );
+    ops_.attention_fused( q_, layer_rows_dev( table_index ), pos_dev(), xb_, batch_, max_pos_, attn_ws_.get(), attn_ws_bytes_ );
+    ops_.template matmul_accum<Config::dim, Config::dim>( x_, xb_, w.wo, batch_, xb_, w.rms_ffn_weight );
+    ops_.matmul_silu_gate( hb_, xb_, w.w1, batch_ );
+    ops_.template matmul_accum<Config::hidden_dim, Config::dim>( x_, hb_, w.w2, batch_, next_att_norm ? xb_ : nullptr, next_att_norm );
   }
 
   void classify_ops()
@@ -527,9 +550,17 @@ private:
       w.wkv = carve( cur, n[2] );
       w.wo = carve( cur, n[3] );
       w.rms_ffn_weight = carve( cur, n[4] );
+      // w3 is placed right after w1 (and wkv right after wq) so that each pair is one row-major
+      // matrix for the fused projections; the file order (w1, w2, w3) only matters when loading
       w.w1 = carve( cur, n[5] );
-      w.w2 = carve( cur, n[6] );
       w.w3 = carve( cur, n[7] );
+      w.w2 = carve( cur, n[6] );
+      if ( n[1] && n[2] ) {
+        GLINT_CHECK( w.wkv == w.wq + n[1] );
+      }
+      if ( n[5] && n[7] ) {
+        GLINT_CHECK( w.w3 == w.w1 + n[5] );
+      }
     }
   }
 

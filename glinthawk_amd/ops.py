@@ -99,6 +99,35 @@ def matmul(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None)
     return out
 
 
+def matmul_accum(residual: torch.Tensor, x: torch.Tensor, w: torch.Tensor, norm_weight: Optional[torch.Tensor] = None):
+    """residual += x @ w.T; returns rmsnorm(residual) * norm_weight when a weight is given."""
+    b, s = x.shape
+    r = w.shape[0]
+    norm_out = torch.empty_like(residual) if norm_weight is not None else None
+    check(lib().gh_matmul_accum(_p(residual), _p(x), _p(w), s, r, b, _p(norm_out), _p(norm_weight), _dt(x), _stream()),
+          "gh_matmul_accum")
+    return norm_out
+
+
+def matmul_silu_gate(x: torch.Tensor, w13: torch.Tensor) -> torch.Tensor:
+    b, s = x.shape
+    hidden = w13.shape[0] // 2
+    hb = torch.empty((b, hidden), dtype=x.dtype, device=x.device)
+    check(lib().gh_matmul_silu_gate(_p(hb), _p(x), _p(w13), s, hidden, b, _dt(x), _stream()), "gh_matmul_silu_gate")
+    return hb
+
+
+def matmul_qkv_rope_append(x: torch.Tensor, wqkv: torch.Tensor, pos: torch.Tensor, freq_real, freq_imag,
+                           token_rows: torch.Tensor, shape: Shape, want_kv: bool = False):
+    b, s = x.shape
+    q = torch.empty((b, shape.dim), dtype=x.dtype, device=x.device)
+    kv = torch.empty((b, 2 * shape.kv_dim), dtype=x.dtype, device=x.device) if want_kv else None
+    check(lib().gh_matmul_qkv_rope_append(_p(q), _p(kv), _p(x), _p(wqkv), s, b, _p(pos), _p(freq_real), _p(freq_imag),
+                                          _p(token_rows), shape.n_kv_heads, shape.gqa_size, shape.head_size, _dt(x),
+                                          _stream()), "gh_matmul_qkv_rope_append")
+    return q, kv
+
+
 def soft_sample(v: torch.Tensor, temperatures: Sequence[float], seed: int = 0) -> None:
     batch, vocab = v.shape
     temps = (C.c_float * batch)(*[float(t) for t in temperatures])

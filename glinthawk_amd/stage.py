@@ -16,7 +16,7 @@ _HOST_LIB_PATH = os.path.join(_PKG, "lib", "libglint_host.so")
 
 STAGE_PRE, STAGE_ATT, STAGE_POST, STAGE_CLS = 0, 1, 2, 3
 FWD_ALL, FWD_PRE, FWD_ATT, FWD_POST, FWD_CLS = 0, 1, 2, 3, 4
-FLAG_FUSED, FLAG_CLS, FLAG_PAGED = 1, 2, 4
+FLAG_FUSED, FLAG_CLS, FLAG_PAGED, FLAG_UNFUSED_PROJ = 1, 2, 4, 8
 
 # layer tensors in file order (rms_att_weight, wq, wkv, wo, rms_ffn_weight, w1, w2, w3)
 LAYER_TENSORS = ("rms_att_weight", "wq", "wkv", "wo", "rms_ffn_weight", "w1", "w2", "w3")
@@ -83,9 +83,10 @@ class Stage:
 
     def __init__(self, config: str, dtype: str, first_layer: int, n_hosted: int, concurrency: int,
                  max_contexts: int, fused: bool = True, with_cls: bool = False, paged: bool = False,
-                 seed: int = 1, weight_std: float = 0.02):
+                 seed: int = 1, weight_std: float = 0.02, fused_projections: bool = True):
         self.np_dtype = np.float16 if dtype == "f16" else np.float32
-        flags = (FLAG_FUSED if fused else 0) | (FLAG_CLS if with_cls else 0) | (FLAG_PAGED if paged else 0)
+        flags = ((FLAG_FUSED if fused else 0) | (FLAG_CLS if with_cls else 0) | (FLAG_PAGED if paged else 0)
+                 | (0 if fused_projections else FLAG_UNFUSED_PROJ))
         self._h = host_lib().glint_stage_create(config.encode(), 0 if dtype == "f16" else 1, first_layer, n_hosted,
                                                 concurrency, max_contexts, flags, seed, weight_std)
         if not self._h:

@@ -134,7 +134,25 @@ int gh_argmax( uint32_t* out_host, uint32_t* out_dev, const void* v, uint64_t n,
  * (<= 0 keeps the current value); prefetch depth 2..4 of the streaming kernel (other values keep it) */
 int gh_gemm_set_tuning( int kernel, int target_workgroups, int depth );
 int gh_matmul( void* xout, const void* x, const void* w, uint64_t s, uint64_t r, uint64_t b, gh_dtype dt, gh_stream stream );
-/* Operations::soft_sample    arch/amd64/common/ops.hh:97-107,273-283 : rows with temperature > 0 get
+/* A projection fused with the ops that follow it in the reference's layer; same arithmetic and the
+ * same rounding points as the separate calls (every matmul result is rounded to DType first).
+ *
+ * matmul + accum [+ rmsnorm]  (post_attention_ops, models/llama2/model.hh:390-427: wo/accum/rmsnorm and w2/accum):
+ *   residual(b, r) = DType(float(residual) + float(DType(x . w^T)));
+ *   if norm_out: norm_out(b, r) = rmsnorm(residual) * norm_weight                                   */
+int gh_matmul_accum( void* residual, const void* x, const void* w, uint64_t s, uint64_t r, uint64_t b, void* norm_out, const void* norm_weight,
+                     gh_dtype dt, gh_stream stream );
+/* matmul w1, matmul w3, silu  (model.hh:411-418): w13 = w1 rows followed by w3 rows, (2 * hidden, s);
+ *   hb(b, hidden) = DType(silu(DType(x . w1^T)) * DType(x . w3^T))                                  */
+int gh_matmul_silu_gate( void* hb, const void* x, const void* w13, uint64_t s, uint64_t hidden_dim, uint64_t b, gh_dtype dt, gh_stream stream );
+/* matmul wq, matmul wkv, copy_kv_cache, apply_rope  (model.hh:326-364): wqkv = wq rows followed by wkv rows;
+ *   q(b, dim) = rope(DType(x . wq^T)); cache row i = [rope(DType(x . wk^T)) | DType(x . wv^T)];
+ *   kv_out (optional, (b, 2 kv_dim)) receives the unrotated [K | V] the reference keeps in its scratchpad.
+ *   Rows of empty contexts (NULL) are skipped and their queries stay unrotated, as in the separate ops. */
+int gh_matmul_qkv_rope_append( void* q, void* kv_out, const void* x, const void* wqkv, uint64_t s, uint64_t b, const uint32_t* pos_dev, const void* freq_real,
+                               const void* freq_imag, void* const* token_rows_dev, uint32_t n_kv_heads, uint32_t gqa_size, uint32_t head_size, gh_dtype dt,
+                               gh_stream stream );
+/* Operations::soft_sample   arch/amd64/common/ops.hh:97-107,273-283 : rows with temperature > 0 get
  * v / T - log(-log(u)), u from a counter-based generator keyed by (seed, row, column).
  * `temperatures` is a HOST array (batch floats), as in the reference. */
 int gh_soft_sample( void* v, const float* temperatures, uint64_t vocab, uint64_t batch, uint64_t seed, gh_dtype dt, gh_stream stream );
