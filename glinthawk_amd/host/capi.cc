@@ -38,6 +38,8 @@ struct StageBase
   virtual int release_context( uint32_t id ) = 0;
   virtual void paging_info( size_t row, size_t layer, uint64_t out[3] ) = 0;
   virtual void sync() = 0;
+  virtual int prefill( uint32_t batch, const uint32_t* context_ids, const uint32_t* start_pos, uint32_t n_tokens, uint32_t first_layer,
+                       const uint32_t* token_ids, const void* acts_in, void* acts_out, uint32_t* next_tokens ) = 0;
 };
 
 template<typename Config, typename DType, typename Ctx>
@@ -178,6 +180,22 @@ struct StageImpl : StageBase
     }
   }
   void sync() override { model.ops().synchronize(); }
+
+  int prefill( uint32_t batch, const uint32_t* context_ids, const uint32_t* start_pos, uint32_t n_tokens, uint32_t first_layer, const uint32_t* token_ids,
+               const void* acts_in, void* acts_out, uint32_t* next_tokens ) override
+  {
+    State tmp( batch, dtype_of<DType>() );
+    for ( uint32_t i = 0; i < batch; i++ ) {
+      tmp.set_prompt( i, context_ids[i], 0, start_pos[i], 0.0f, n_tokens, 0 );
+    }
+    auto got = contexts.get_contexts( tmp );
+    if ( !got.has_value() ) {
+      return -1;
+    }
+    held = std::move( *got );
+    model.prefill( held, start_pos, n_tokens, first_layer, token_ids, static_cast<const DType*>( acts_in ), static_cast<DType*>( acts_out ), next_tokens );
+    return 0;
+  }
 };
 
 template<typename Config>
@@ -314,6 +332,12 @@ int glint_stage_release_context( void* h, uint32_t id ) { return static_cast<Sta
 void glint_stage_paging_info( void* h, uint32_t row, uint32_t layer, uint64_t out[3] ) { static_cast<StageBase*>( h )->paging_info( row, layer, out ); }
 void* glint_stage_scratch( void* h, int which ) { return static_cast<StageBase*>( h )->scratch( which ); }
 void glint_stage_sync( void* h ) { static_cast<StageBase*>( h )->sync(); }
+// batched prefill of n_tokens tokens per context; -1 when the contexts cannot be served
+int glint_stage_prefill( void* h, uint32_t batch, const uint32_t* context_ids, const uint32_t* start_pos, uint32_t n_tokens, uint32_t first_layer,
+                         const uint32_t* token_ids, const void* acts_in, void* acts_out, uint32_t* next_tokens )
+{
+  return static_cast<StageBase*>( h )->prefill( batch, context_ids, start_pos, n_tokens, first_layer, token_ids, acts_in, acts_out, next_tokens );
+}
 
 // ---- host-only bookkeeping hooks ---------------------------------------------------------------
 void* glint_book_manager_new( uint64_t max_context_count ) { return new BookManager( max_context_count ); }

@@ -294,6 +294,100 @@ public:
     postlude( states, states.next_layer(), true );
   }
 
+  // ------------------------------------------------------------------------------------------
+  // Batched prefill (new functionality: the reference feeds prompts one token per forward).
+  // `n_tokens` consecutive tokens per context, context i starting at position start_pos[i]; runs
+  // every hosted layer from `first_layer` on all batch * n_tokens tokens at once.  The cache rows
+  // and the outputs equal those of n_tokens sequential forward() calls.
+  //   token_ids     (batch * n_tokens) when the embedding is hosted and first_layer == 0, else nullptr
+  //   acts_in_host  (batch * n_tokens, dim) activations otherwise
+  //   acts_out_host (batch * n_tokens, dim) residual stream after the last hosted layer (may be nullptr)
+  //   next_tokens   (batch) greedy token after the last prompt token, when the classifier is hosted (may be nullptr)
+  // ------------------------------------------------------------------------------------------
+  void prefill( const ContextVector& contexts,
+                const uint32_t* start_pos,
+                const uint32_t n_tokens,
+                const uint32_t first_layer,
+                const uint32_t* token_ids,
+                const DType* acts_in_host,
+                DType* acts_out_host,
+                uint32_t* next_tokens )
+  {
+    GLINT_CHECK( options_.fused_attention && options_.fused_projections );
+    const size_t batch = contexts.size();
+    GLINT_CHECK( batch > 0 && batch <= settings_.concurrency_limit && n_tokens > 0 );
+    const uint64_t n = (uint64_t)batch * n_tokens;
+    ensure_prefill_scratch( n );
+    batch_ = batch;
+
+    std::vector<size_t> run;
+    for ( size_t l = first_layer; l < Config::n_layers && settings_.hosts( l, InferenceStage::PreAttention ); l++ ) {
+      run.push_back( l );
+    }
+    GLINT_CHECK( !run.empty() );
+    uint32_t max_start = 0;
+    for ( size_t i = 0; i < batch; i++ ) {
+      GLINT_CHECK( (uint64_t)start_pos[i] + n_tokens <= Config::seq_len );
+      token_positions_[i] = start_pos[i];
+      max_start = std::max( max_start, start_pos[i] );
+      for ( size_t k = 0; k < run.size(); k++ ) {
+        GLINT_CHECK( contexts[i]->prepare( run[k], start_pos[i] + n_tokens - 1,
+                                           k == 0 && start_pos[i] == 0 && settings_.first_layer_served == first_layer ) );
+      }
+    }
+    upload_tables( contexts, run ); // per-context tables: pos = start positions, layer bases per layer
+
+    DType* px = pf_x_.get();
+    DType* pxb = pf_xb_.get();
+    DType* pq = pf_q_.get();
+    DType* phb = pf_hb_.get();
+    if ( first_layer == 0 && token_ids != nullptr ) {
+      for ( uint64_t r = 0; r < n; r++ ) {
+        GLINT_CHECK( token_ids[r] < Config::vocab_size );
+        ops_.copy( px + r * Config::dim, base_.token_embedding_table + (uint64_t)token_ids[r] * Config::dim, Config::dim * sizeof( DType ),
+                   CopyType::DeviceToDevice, true );
+      }
+    } else {
+      GLINT_CHECK( acts_in_host != nullptr );
+      ops_.copy( px, acts_in_host, n * Config::dim * sizeof( DType ), CopyType::HostToDevice, true );
+    }
+
+    const gh_shape shape = LlamaOperations::shape();
+    const uint64_t row_bytes = 2ull * Config::kv_dim * sizeof( DType );
+    ops_.template rmsnorm<Config::dim>( pxb, px, reinterpret_cast<float32_t*>( temp_ ), layers_[run[0]].rms_att_weight, n );
+    for ( size_t k = 0; k < run.size(); k++ ) {
+      const auto& w = layers_[run[k]];
+      // one table entry per (context, token) for this layer's rows
+      GLINT_GH( gh_prefill_tables( layer_rows_dev( k ), pos_dev(), batch, n_tokens, row_bytes, nullptr, pf_token_rows(), pf_pos(), ops_.stream() ) );
+      ops_.matmul_qkv_rope_append( pq, pxb, w.wq, n, pf_pos(), base_.freq_cis_real, base_.freq_cis_imag, pf_token_rows() );
+      GLINT_GH( gh_attn_prefill( pq, layer_rows_dev( k ), pos_dev(), pxb, batch, n_tokens, max_start, &shape, hip::gh_type<DType>(), pf_attn_ws_.get(),
+                                 pf_attn_ws_bytes_, GH_ATTN_AUTO, ops_.stream() ) );
+      ops_.template matmul_accum<Config::dim, Config::dim>( px, pxb, w.wo, n, pxb, w.rms_ffn_weight );
+      ops_.matmul_silu_gate( phb, pxb, w.w1, n );
+      const DType* next_norm = k + 1 < run.size() ? layers_[run[k + 1]].rms_att_weight : nullptr;
+      ops_.template matmul_accum<Config::hidden_dim, Config::dim>( px, phb, w.w2, n, next_norm ? pxb : nullptr, next_norm );
+    }
+
+    if ( acts_out_host != nullptr ) {
+      ops_.copy( acts_out_host, px, n * Config::dim * sizeof( DType ), CopyType::DeviceToHost );
+    }
+    const size_t last = run.back();
+    if ( next_tokens != nullptr && last == Config::n_layers - 1 && settings_.hosts( last, InferenceStage::Classification ) ) {
+      // only the last prompt token of each context is classified
+      for ( size_t i = 0; i < batch; i++ ) {
+        ops_.copy( x_ + i * Config::dim, px + ( (uint64_t)i * n_tokens + n_tokens - 1 ) * Config::dim, Config::dim * sizeof( DType ), CopyType::DeviceToDevice,
+                   true );
+      }
+      classify_ops();
+      ops_.template argmax<Config::vocab_size>( argmax_pos_, logits_, temp_, batch );
+      for ( size_t i = 0; i < batch; i++ ) {
+        next_tokens[i] = argmax_pos_[i];
+      }
+    } else {
+      ops_.synchronize();
+    }
+  }
+
   // scratch views for tests (device pointers)
   DType* scratch_x() const { return x_; }
   DType* scratch_xb() const { return xb_; }
@@ -647,7 +741,30 @@ private:
   ModelOptions options_;
   LlamaOperations ops_;
 
+  // prefill scratch: activations for `pf_capacity_` tokens, grown on demand
+  void ensure_prefill_scratch( const uint64_t n )
+  {
+    if ( n <= pf_capacity_ ) {
+      return;
+    }
+    ops_.synchronize();
+    pf_x_ = ops_.device_allocate( n * Config::dim * sizeof( DType ) );
+    pf_xb_ = ops_.device_allocate( n * Config::dim * sizeof( DType ) );
+    pf_q_ = ops_.device_allocate( n * Config::dim * sizeof( DType ) );
+    pf_hb_ = ops_.device_allocate( n * Config::hidden_dim * sizeof( DType ) );
+    pf_tables_ = ops_.device_allocate( n * ( sizeof( void* ) + sizeof( uint32_t ) ) + 64 );
+    const gh_shape shape = LlamaOperations::shape();
+    // sized for the widest call: every context contributes all n tokens
+    pf_attn_ws_bytes_ = gh_attn_prefill_workspace( 1, static_cast<uint32_t>( n ), &shape );
+    pf_attn_ws_ = ops_.device_allocate( std::max<uint64_t>( pf_attn_ws_bytes_, 16 ) );
+    pf_capacity_ = n;
+  }
+  void** pf_token_rows() const { return reinterpret_cast<void**>( pf_tables_.get() ); }
+  uint32_t* pf_pos() const { return reinterpret_cast<uint32_t*>( pf_token_rows() + pf_capacity_ ); }
+
   DevicePtr base_storage_ {}, layer_storage_ {}, scratch_storage_ {}, attn_ws_ {}, tables_dev_ {};
+  DevicePtr pf_x_ {}, pf_xb_ {}, pf_q_ {}, pf_hb_ {}, pf_tables_ {}, pf_attn_ws_ {};
+  uint64_t pf_capacity_ { 0 }, pf_attn_ws_bytes_ { 0 };
   uint64_t attn_ws_bytes_ { 0 };
   uint8_t* tables_host_ { nullptr };
   BaseWeights<DType> base_ {};

@@ -232,6 +232,27 @@ def attn_decode_host(q, layer_rows: Sequence[int], pos: Sequence[int], xb, shape
           "gh_attn_decode_host")
 
 
+def prefill_tables(layer_rows: torch.Tensor, start_pos: torch.Tensor, n_tokens: int, row_bytes: int):
+    """Expanded (context, token) tables: (layer_rows, token_rows, pos), each of batch * n_tokens entries."""
+    batch = layer_rows.numel()
+    n = batch * n_tokens
+    rows = torch.empty(n, dtype=torch.int64, device=layer_rows.device)
+    trows = torch.empty(n, dtype=torch.int64, device=layer_rows.device)
+    pos = torch.empty(n, dtype=torch.int32, device=layer_rows.device)
+    check(lib().gh_prefill_tables(_p(layer_rows), _p(start_pos), batch, n_tokens, row_bytes, _p(rows), _p(trows), _p(pos),
+                                  _stream()), "gh_prefill_tables")
+    return rows, trows, pos
+
+
+def attn_prefill(q, layer_rows: torch.Tensor, start_pos: torch.Tensor, xb, n_tokens: int, max_start_pos: int, shape: Shape,
+                 variant: int = GH_ATTN_AUTO) -> None:
+    s = shape.c()
+    batch = layer_rows.numel()
+    ws = torch.empty(int(lib().gh_attn_prefill_workspace(batch, n_tokens, C.byref(s))), dtype=torch.uint8, device=q.device)
+    check(lib().gh_attn_prefill(_p(q), _p(layer_rows), _p(start_pos), _p(xb), batch, n_tokens, max_start_pos, C.byref(s),
+                                _dt(q), _p(ws), ws.numel(), variant, _stream()), "gh_attn_prefill")
+
+
 def attn_set_chunk(tokens: int) -> None:
     check(lib().gh_attn_set_chunk(tokens), "gh_attn_set_chunk")
 

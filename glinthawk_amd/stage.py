@@ -57,6 +57,7 @@ def host_lib() -> C.CDLL:
             "glint_stage_paging_info": (None, [vp, u32, u32, C.POINTER(u64)]),
             "glint_stage_scratch": (vp, [vp, C.c_int]),
             "glint_stage_sync": (None, [vp]),
+            "glint_stage_prefill": (C.c_int, [vp, u32, vp, vp, u32, u32, vp, vp, vp, vp]),
             "glint_book_manager_new": (vp, [u64]),
             "glint_book_manager_delete": (None, [vp]),
             "glint_book_manager_free": (u64, [vp]),
@@ -188,6 +189,33 @@ class Stage:
 
     def sync(self) -> None:
         host_lib().glint_stage_sync(self._h)
+
+    def prefill(self, context_ids, start_pos, n_tokens: int, first_layer: int = 0, token_ids=None, activations=None,
+                want_activations: bool = True, want_next_tokens: bool = False):
+        """Batched prefill of `n_tokens` tokens per context.  Returns (activations_out or None,
+        next_tokens or None); None overall when the contexts could not be served."""
+        batch = len(context_ids)
+        ids = np.ascontiguousarray(np.asarray(context_ids, dtype=np.uint32))
+        start = np.ascontiguousarray(np.asarray(start_pos, dtype=np.uint32))
+        toks = None if token_ids is None else np.ascontiguousarray(np.asarray(token_ids, dtype=np.uint32).reshape(-1))
+        acts = None if activations is None else np.ascontiguousarray(activations, dtype=self.np_dtype)
+        if toks is not None:
+            assert toks.size == batch * n_tokens
+        dim = None if acts is None else acts.reshape(batch * n_tokens, -1).shape[1]
+        out = None
+        if want_activations:
+            if dim is None:
+                raise ValueError("pass dim via activations or call with want_activations=False")
+            out = np.empty((batch * n_tokens, dim), dtype=self.np_dtype)
+        nxt = np.zeros(batch, dtype=np.uint32) if want_next_tokens else None
+        rc = host_lib().glint_stage_prefill(self._h, batch, ids.ctypes.data, start.ctypes.data, n_tokens, first_layer,
+                                            None if toks is None else toks.ctypes.data,
+                                            None if acts is None else acts.ctypes.data,
+                                            None if out is None else out.ctypes.data,
+                                            None if nxt is None else nxt.ctypes.data)
+        if rc != 0:
+            return None
+        return out, nxt
 
 
 class BookManager:

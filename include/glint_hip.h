@@ -210,6 +210,25 @@ int gh_attn_decode( const void* q, const void* const* layer_rows_dev, const uint
 int gh_attn_decode_host( const void* q, const void* const* layer_rows_host, const uint32_t* pos_host, void* xb, uint64_t batch,
                          const gh_shape* shape, gh_dtype dt, void* workspace, uint64_t workspace_bytes, int variant, gh_stream stream );
 
+/* Batched prefill (no counterpart in the reference, which feeds prompts one token per forward:
+ * frontend/infer.cc:124-125, models/llama2/model.hh:356-357).  `n_tokens` new tokens per context at
+ * positions [start_pos_i, start_pos_i + n_tokens); activations are (batch * n_tokens, dim) with row
+ * index context * n_tokens + token.  The result equals n_tokens sequential decode steps.
+ *
+ * gh_prefill_tables expands per-context tables to one entry per (context, token) -- the tables the
+ * decode-style entry points (gh_matmul_qkv_rope_append, gh_kv_append, gh_rope, gh_attn_decode) take:
+ *   layer_rows_out[i*T+t] = layer_rows[i], token_rows_out[i*T+t] = layer_rows[i] + (start_i + t) * row_bytes,
+ *   pos_out[i*T+t] = start_i + t.  Any output may be NULL. */
+int gh_prefill_tables( const void* const* layer_rows_dev, const uint32_t* start_pos_dev, uint64_t batch, uint32_t n_tokens, uint64_t row_bytes,
+                       const void** layer_rows_out, void** token_rows_out, uint32_t* pos_out, gh_stream stream );
+/* Causal attention of the new tokens over the cache (their rows already appended and rotated):
+ * query token t of context i attends keys [0, start_i + t].  f16 / head size 128 runs a tiled MFMA
+ * kernel; other shapes run the decode kernels on expanded tables (workspace needed, see
+ * gh_attn_prefill_workspace).  max_start_pos: host-side upper bound of start_pos. */
+uint64_t gh_attn_prefill_workspace( uint64_t batch, uint32_t n_tokens, const gh_shape* shape );
+int gh_attn_prefill( const void* q, const void* const* layer_rows_dev, const uint32_t* start_pos_dev, void* xb, uint64_t batch, uint32_t n_tokens,
+                     uint32_t max_start_pos, const gh_shape* shape, gh_dtype dt, void* workspace, uint64_t workspace_bytes, int variant, gh_stream stream );
+
 /* Timing hooks for the benchmark: HIP events recorded on `stream` around the two kernels of
  * gh_attn_decode.  gh_attn_timing_read() synchronises and returns, accumulated since
  * gh_attn_timing_reset(): milliseconds in the split-K attention kernel, milliseconds in the merge

@@ -1,0 +1,195 @@
+"""Batched prefill attention against the sequential definition: query token t of a context attends
+keys [0, start + t], i.e. exactly what T decode calls compute.  Checked against the oracle's fp32
+attention ops on the same inputs and against the decode kernels on expanded tables."""
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from glinthawk_amd import Shape, ops
+from glinthawk_amd._lib import GH_ATTN_AUTO, GH_ATTN_GENERIC, GH_ATTN_MFMA
+from helpers import Arena, assert_close, errors, oracle_cfg
+
+pytestmark = pytest.mark.gpu
+
+TINY = Shape(dim=32, n_layers=1, n_heads=4, n_kv_heads=2, hidden_dim=48, seq_len=64)
+STORIES = Shape(dim=288, n_layers=1, n_heads=6, n_kv_heads=6, hidden_dim=768, seq_len=256)
+MHA = Shape(dim=768, n_layers=1, n_heads=6, n_kv_heads=6, hidden_dim=64, seq_len=400)
+GQA2 = Shape(dim=1024, n_layers=1, n_heads=8, n_kv_heads=4, hidden_dim=64, seq_len=300)
+GQA4 = Shape(dim=1536, n_layers=1, n_heads=12, n_kv_heads=3, hidden_dim=64, seq_len=330)
+GQA8 = Shape(dim=2048, n_layers=1, n_heads=16, n_kv_heads=2, hidden_dim=64, seq_len=700)
+GQA16 = Shape(dim=2048, n_layers=1, n_heads=16, n_kv_heads=1, hidden_dim=64, seq_len=300)
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _init():
+    ops.init(0)
+
+
+def run_case(shape, dt, variant, n_tokens, starts, present, seed=1):
+    batch = len(starts)
+    tdt = torch.float16 if dt == "f16" else torch.float32
+    ndt = np.float16 if dt == "f16" else np.float32
+    arena = Arena(shape, batch, tdt, seed=seed)
+    rng = np.random.default_rng(seed + 1)
+    q = rng.standard_normal((batch * n_tokens, shape.dim)).astype(ndt)
+    dq = torch.from_numpy(q).cuda()
+    layers = ops.row_table([arena.layer_ptr(i) if present[i] else 0 for i in range(batch)])
+    dstart = torch.tensor(starts, dtype=torch.int32, device="cuda")
+    xb = torch.full((batch * n_tokens, shape.dim), 5.0, dtype=tdt, device="cuda")
+    ops.attn_prefill(dq, layers, dstart, xb, n_tokens, max(starts), shape, variant=variant)
+    got = xb.float().cpu().numpy()
+
+    # sequential definition on the CPU: one decode row per (context, token)
+    cfg = oracle_cfg(shape)
+    l32 = arena.host_layers_f32(present)
+    rows = [l32[i] for i in range(batch) for _ in range(n_tokens)]
+    pos = [starts[i] + t for i in range(batch) for t in range(n_tokens)]
+    q32 = q.astype(np.float32)
+    att = np.zeros((batch * n_tokens, shape.n_heads, shape.seq_len), np.float32)
+    want = np.full((batch * n_tokens, shape.dim), 5.0, np.float32)
+    O.attention_0_gemm(cfg, q32, rows, att, pos)
+    O.attention_softmax(cfg, att, pos)
+    O.attention_2_gemm(cfg, att, rows, want, pos)
+    live = [i * n_tokens + t for i in range(batch) if present[i] for t in range(n_tokens)]
+    assert_close(got[live], want[live], what=f"prefill attention {dt} T={n_tokens} variant {variant}")
+    for i in range(batch):
+        if not present[i]:
+            assert np.all(got[i * n_tokens:(i + 1) * n_tokens] == 5.0)
+    return got
+
+
+@pytest.mark.parametrize("shape", [MHA, GQA2, GQA4, GQA8, GQA16], ids=["mha", "gqa2", "gqa4", "gqa8", "gqa16"])
+@pytest.mark.parametrize("n_tokens", [1, 5, 16, 37, 130])
+def test_prefill_mfma(shape, n_tokens):
+    starts = [0, 7, min(100, shape.seq_len - n_tokens), 3]
+    got = run_case(shape, "f16", GH_ATTN_MFMA, n_tokens, starts, [True, True, True, False])
+    # the decode kernels on expanded tables give the same numbers up to rounding
+    other = run_case(shape, "f16", GH_ATTN_GENERIC, n_tokens, starts, [True, True, True, False])
+    a, r = errors(got[: 3 * n_tokens], other[: 3 * n_tokens])
+    assert a < 4e-3 and r < 1e-3
+
+
+@pytest.mark.parametrize("shape,dt", [(TINY, "f32"), (TINY, "f16"), (STORIES, "f32")], ids=["tiny32", "tiny16", "stories15m"])
+@pytest.mark.parametrize("n_tokens", [1, 8, 33])
+def test_prefill_generic_shapes(shape, dt, n_tokens):
+    starts = [0, 5, shape.seq_len - n_tokens]
+    run_case(shape, dt, GH_ATTN_AUTO, n_tokens, starts, [True, True, True])
+
+
+def test_prefill_tables():
+    layer_rows = ops.row_table([1 << 20, 0, 3 << 20])
+    start = torch.tensor([0, 4, 10], dtype=torch.int32, device="cuda")
+    rows, trows, pos = ops.prefill_tables(layer_rows, start, 3, 4096)
+    assert rows.tolist() == [1 << 20] * 3 + [0] * 3 + [3 << 20] * 3
+    assert pos.tolist() == [0, 1, 2, 4, 5, 6, 10, 11, 12]
+    assert trows.tolist() == [(1 << 20) + 4096 * p for p in (0, 1, 2)] + [0, 0, 0] + [(3 << 20) + 4096 * p for p in (10, 11, 12)]
+
+
+def test_prefill_first_token_sees_one_key():
+    shape = GQA8
+    arena = Arena(shape, 1, torch.float16, seed=9)
+    q = torch.randn((16, shape.dim), dtype=torch.float16, device="cuda")
+    xb = torch.zeros_like(q)
+    ops.attn_prefill(q, ops.row_table([arena.layer_ptr(0)]), torch.zeros(1, dtype=torch.int32, device="cuda"), xb, 16, 0, shape)
+    v0 = arena.dev[0, 0, shape.kv_dim:].reshape(shape.n_kv_heads, 1, shape.head_size).expand(-1, shape.gqa_size, -1).reshape(-1)
+    assert torch.equal(xb[0], v0)          # token 0 attends key 0 only: weight exactly 1
+
+
+# ------------------------------------------------------------------ whole stage: batched prefill vs token by token
+from glinthawk_amd import stage as S  # noqa: E402
+from test_gpu_stage import SHAPES, OracleModel, d2h, load_weights, make_weights  # noqa: E402
+
+
+@pytest.mark.parametrize("name,dtype,n_prompt", [("test-gqa4", "f16", 37), ("test-mha", "f16", 20), ("stories15m", "f32", 9),
+                                                 ("test-tiny", "f32", 5)])
+def test_stage_prefill_equals_token_by_token(name, dtype, n_prompt):
+    cfg = SHAPES[name]
+    np_dt = np.float16 if dtype == "f16" else np.float32
+    wcls = name in ("test-gqa4", "test-tiny")
+    layers, base = make_weights(cfg, np_dt, seed=41, wcls=wcls)
+    batch = 3
+    rng = np.random.default_rng(42)
+    prompts = rng.integers(0, cfg.vocab_size, (batch, n_prompt))
+    a = S.Stage(name, dtype, 0, cfg.n_layers, batch, batch, with_cls=True)      # batched prefill
+    b = S.Stage(name, dtype, 0, cfg.n_layers, batch, batch, with_cls=True)      # the reference's way: one token per forward
+    ref = OracleModel(cfg, layers, base)
+    for st in (a, b):
+        load_weights(st, cfg, layers, base, wcls)
+
+    # sequential path (and the oracle beside it)
+    b.new_state(batch)
+    for i in range(batch):
+        b.set_prompt(i, 10 + i, int(prompts[i, 0]), 0, 0.0, n_prompt, 0)
+    for pos in range(n_prompt):
+        want = ref.step(prompts[:, pos].tolist(), [10 + i for i in range(batch)], [pos] * batch)
+        assert b.forward()
+        if pos + 1 < n_prompt:
+            for i in range(batch):
+                b.set_prompt(i, 10 + i, int(prompts[i, pos + 1]), pos + 1, 0.0, n_prompt, 0)
+    seq_logits = d2h(b.scratch_ptr("logits"), (batch, cfg.vocab_size), np_dt).astype(np.float32)
+    seq_next = [b.row(i)["token"] for i in range(batch)]
+
+    # batched path
+    res = a.prefill([10 + i for i in range(batch)], [0] * batch, n_prompt, 0, token_ids=prompts, want_activations=False,
+                    want_next_tokens=True)
+    assert res is not None
+    _, nxt = res
+    pre_logits = d2h(a.scratch_ptr("logits"), (batch, cfg.vocab_size), np_dt).astype(np.float32)
+    tol = 6e-3 if dtype == "f16" else 5e-5
+    np.testing.assert_allclose(pre_logits, seq_logits, rtol=tol, atol=tol)
+    assert_close(pre_logits, want, mean_rel=2e-3 if dtype == "f16" else 1e-3, what=f"{name} prefill logits vs oracle")
+    for i in range(batch):
+        if nxt[i] != seq_next[i]:
+            assert abs(seq_logits[i, nxt[i]] - seq_logits[i, seq_next[i]]) < 1e-2      # near tie only
+
+    # the caches agree row by row (K rotated, V raw), so decoding can continue from either
+    a.new_state(batch)
+    for i in range(batch):
+        a.set_prompt(i, 10 + i, seq_next[i], n_prompt)
+        b.set_prompt(i, 10 + i, seq_next[i], n_prompt)
+    assert a.acquire_contexts() and b.acquire_contexts()
+    row_elems = 2 * cfg.kv_dim
+    for i in range(batch):
+        for l in range(cfg.n_layers):
+            ka = d2h(a.context_layer_ptr(i, l), (n_prompt, row_elems), np_dt).astype(np.float32)
+            kb = d2h(b.context_layer_ptr(i, l), (n_prompt, row_elems), np_dt).astype(np.float32)
+            np.testing.assert_allclose(ka, kb, rtol=tol, atol=tol)
+    for step in range(3):
+        assert a.forward() and b.forward()
+        la = d2h(a.scratch_ptr("logits"), (batch, cfg.vocab_size), np_dt).astype(np.float32)
+        lb = d2h(b.scratch_ptr("logits"), (batch, cfg.vocab_size), np_dt).astype(np.float32)
+        np.testing.assert_allclose(la, lb, rtol=tol, atol=tol)
+        for i in range(batch):
+            a.set_prompt(i, 10 + i, b.row(i)["token"], n_prompt + step + 1)
+    a.close()
+    b.close()
+
+
+def test_stage_prefill_middle_stage_and_chunks():
+    # layers 1..2 of the 3-layer test model, activations in/out; the prompt is prefetched in two chunks
+    name, dtype = "test-gqa4", "f16"
+    cfg = SHAPES[name]
+    layers, base = make_weights(cfg, np.float16, seed=43, wcls=True)
+    batch, T = 2, 24
+    rng = np.random.default_rng(44)
+    x = rng.standard_normal((batch, T, cfg.dim)).astype(np.float16)
+    a = S.Stage(name, dtype, 1, 2, batch, batch)
+    b = S.Stage(name, dtype, 1, 2, batch, batch)
+    for st in (a, b):
+        load_weights(st, cfg, layers, base, True, layer_range=[1, 2], with_embedding=False, with_cls=False)
+    outs = np.zeros((batch, T, cfg.dim), np.float32)
+    for pos in range(T):
+        b.new_state(batch, next_layer=1)
+        for i in range(batch):
+            b.set_prompt(i, 70 + i, 1, pos)
+        b.activations(allocate=True)[:] = x[:, pos].reshape(-1)
+        assert b.forward()
+        outs[:, pos] = b.activations().reshape(batch, cfg.dim).astype(np.float32)
+    first, second = 16, T - 16
+    o1, _ = a.prefill([70, 71], [0, 0], first, 1, activations=x[:, :first].reshape(batch * first, cfg.dim))
+    o2, _ = a.prefill([70, 71], [first, first], second, 1, activations=x[:, first:].reshape(batch * second, cfg.dim))
+    got = np.concatenate([o1.reshape(batch, first, cfg.dim), o2.reshape(batch, second, cfg.dim)], axis=1).astype(np.float32)
+    np.testing.assert_allclose(got, outs, rtol=6e-3, atol=6e-3)
+    a.close()
+    b.close()
