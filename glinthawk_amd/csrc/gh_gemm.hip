@@ -21,10 +21,13 @@ void gemm_stream_plan( uint64_t s, uint64_t r, uint64_t b, uint32_t* splits_out,
 int gemm_stream_launch( __half* xout, float* partial, const __half* x, const __half* w, uint64_t s, uint64_t r, uint64_t b, uint32_t splits,
                         uint32_t k_per_split, bool write_partials, hipStream_t st );
 void gemm_stream_tuning( int target_wgs, int depth );
+// large-batch (prefill) kernel (gh_gemm_tile.hip)
+bool gemm_tile_applicable( uint64_t s, uint64_t r, uint64_t b, const void* x, const void* w, const void* xout );
+int gemm_tile_launch( __half* xout, const __half* x, const __half* w, uint64_t s, uint64_t r, uint64_t b, hipStream_t st );
 
 namespace {
 
-int g_force_kernel = 0; // 0 auto, 1 tiled kernel of this file, 2 streaming kernel
+int g_force_kernel = 0; // 0 auto, 1 small tiled kernel of this file, 2 streaming kernel, 3 large tile kernel
 
 typedef _Float16 f16x8 __attribute__( ( ext_vector_type( 8 ) ) );
 typedef float f32x4 __attribute__( ( ext_vector_type( 4 ) ) );
@@ -247,6 +250,12 @@ int gemm_partials( void* xout, const void* x, const void* w, uint64_t s, uint64_
     return GH_OK;
   }
   GH_REQUIRE( dt == GH_F16, "gh_matmul: unsupported dtype %d", (int)dt );
+
+  // many tokens at once (prefill): the MFMA-bound tile kernel; few (decode): the weight-streaming one
+  if ( !want_partials && ( g_force_kernel == 0 || g_force_kernel == 3 ) && gemm_tile_applicable( s, r, b, x, w, xout ) ) {
+    return gemm_tile_launch( static_cast<__half*>( xout ), static_cast<const __half*>( x ), static_cast<const __half*>( w ), s, r, b, st );
+  }
+  GH_REQUIRE( g_force_kernel != 3, "gh_matmul: the tile kernel needs b >= 128, s %% 8 == 0 and 16-byte aligned operands" );
 
   if ( g_force_kernel != 1 && gemm_stream_applicable( s, r, b, x, w, xout ? xout : x ) ) {
     uint32_t splits = 1, k_per_split = 0;

@@ -1,0 +1,170 @@
+// Large-batch GEMM for prefill: xout(b, r) = sum_p w(r, p) * x(b, p) with b in the hundreds or
+// thousands (all prompt tokens of a batch at once), f16 storage, fp32 accumulate.  This regime is
+// MFMA-bound, not HBM-bound: both operands are re-used across a 128 x 128 output tile.
+//
+//   work-group = 4 waves (2 x 2), tile 128 weight rows x 128 tokens, K in steps of 64
+//   wave        = 64 x 64 = 2 x 2 accumulators of v_mfma_f32_32x32x16_f16
+//   operands    global -> registers (next step in flight while the current one is multiplied)
+//               -> LDS, 16-byte chunks XOR-swizzled so that the MFMA-order reads are conflict free,
+//               two LDS buffers, one barrier per step
+#include "gh_common.h"
+
+namespace gh {
+
+typedef _Float16 f16x8 __attribute__( ( ext_vector_type( 8 ) ) );
+typedef float f32x16 __attribute__( ( ext_vector_type( 16 ) ) );
+
+namespace {
+
+constexpr int TM = 128; // weight rows per work-group
+constexpr int TN = 128; // tokens per work-group
+constexpr int TK = 64;  // k per step: 8 chunks of 8 halves
+
+struct Frag
+{
+  uint4 v[4]; // thread t: row t/8 + 32*i, chunk t%8
+};
+
+__device__ __forceinline__ void load_frag( Frag& f, const __half* __restrict__ mat, uint64_t ld, uint32_t row0, uint32_t n_rows, uint32_t k0, uint32_t k_end )
+{
+  const uint32_t chunk = threadIdx.x & 7;
+  const uint32_t k = k0 + 8 * chunk;
+#pragma unroll
+  for ( int i = 0; i < 4; i++ ) {
+    const uint32_t row = row0 + ( threadIdx.x >> 3 ) + 32 * i;
+    f.v[i] = ( row < n_rows && k < k_end ) ? *reinterpret_cast<const uint4*>( mat + (uint64_t)row * ld + k ) : make_uint4( 0, 0, 0, 0 );
+  }
+}
+
+// rows are 128 bytes (8 chunks); chunk position is XORed with bits 1..3 of the row so that 16 rows
+// of one chunk column fall into 16 different 16-byte bank groups
+__device__ __forceinline__ uint32_t swz( uint32_t row, uint32_t chunk ) { return row * 8 + ( chunk ^ ( ( row >> 1 ) & 7 ) ); }
+
+__device__ __forceinline__ void store_frag( uint4* tile, const Frag& f )
+{
+  const uint32_t chunk = threadIdx.x & 7;
+#pragma unroll
+  for ( int i = 0; i < 4; i++ ) {
+    const uint32_t row = ( threadIdx.x >> 3 ) + 32 * i;
+    tile[swz( row, chunk )] = f.v[i];
+  }
+}
+
+// grid: (row tiles, token tiles).  s % 8 == 0, 16-byte aligned operands.
+__global__ __launch_bounds__( 256 ) void gemm_tile_kernel( __half* __restrict__ xout,
+                                                           const __half* __restrict__ x,
+                                                           const __half* __restrict__ w,
+                                                           uint32_t s,
+                                                           uint32_t r,
+                                                           uint32_t b )
+{
+  __shared__ uint4 s_w[2][TM * 8]; // 2 x 16 KiB
+  __shared__ uint4 s_x[2][TN * 8]; // 2 x 16 KiB
+
+  const uint32_t wave = threadIdx.x >> 6;
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t wm = wave & 1, wn = wave >> 1; // wave position inside the tile
+  const uint32_t row0 = blockIdx.x * TM;
+  const uint32_t col0 = blockIdx.y * TN;
+  const uint32_t lr = lane & 31, g2 = lane >> 5;
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for ( int i = 0; i < 2; i++ ) {
+#pragma unroll
+    for ( int j = 0; j < 2; j++ ) {
+#pragma unroll
+      for ( int e = 0; e < 16; e++ ) {
+        acc[i][j][e] = 0.0f;
+      }
+    }
+  }
+
+  Frag fw, fx;
+  load_frag( fw, w, s, row0, r, 0, s );
+  load_frag( fx, x, s, col0, b, 0, s );
+  int buf = 0;
+  for ( uint32_t k0 = 0; k0 < s; k0 += TK ) {
+    store_frag( s_w[buf], fw );
+    store_frag( s_x[buf], fx );
+    __syncthreads();
+    if ( k0 + TK < s ) {
+      load_frag( fw, w, s, row0, r, k0 + TK, s );
+      load_frag( fx, x, s, col0, b, k0 + TK, s );
+    }
+    const uint4* lw = s_w[buf];
+    const uint4* lx = s_x[buf];
+#pragma unroll
+    for ( int st = 0; st < 4; st++ ) {
+      const uint32_t ch = 2 * st + g2;
+      f16x8 a[2], bb[2];
+#pragma unroll
+      for ( int i = 0; i < 2; i++ ) {
+        a[i] = __builtin_bit_cast( f16x8, lw[swz( wm * 64 + 32 * i + lr, ch )] );
+        bb[i] = __builtin_bit_cast( f16x8, lx[swz( wn * 64 + 32 * i + lr, ch )] );
+      }
+#pragma unroll
+      for ( int i = 0; i < 2; i++ ) {
+#pragma unroll
+        for ( int j = 0; j < 2; j++ ) {
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16( a[i], bb[j], acc[i][j], 0, 0, 0 );
+        }
+      }
+    }
+    buf ^= 1;
+  }
+
+  // acc[i][j][v]: weight row = row0 + wm*64 + 32*i + 8*(v/4) + 4*g2 + v%4, token = col0 + wn*64 + 32*j + lr
+#pragma unroll
+  for ( int j = 0; j < 2; j++ ) {
+    const uint32_t col = col0 + wn * 64 + 32 * j + lr;
+    if ( col >= b ) {
+      continue;
+    }
+#pragma unroll
+    for ( int i = 0; i < 2; i++ ) {
+#pragma unroll
+      for ( int q4 = 0; q4 < 4; q4++ ) {
+        const uint32_t row = row0 + wm * 64 + 32 * i + 8 * q4 + 4 * g2;
+        __half* dst = xout + (uint64_t)col * r + row;
+        if ( row + 3 < r && ( r & 3 ) == 0 ) {
+          union
+          {
+            uint2 raw;
+            __half h[4];
+          } o;
+#pragma unroll
+          for ( int e = 0; e < 4; e++ ) {
+            o.h[e] = __float2half_rn( acc[i][j][4 * q4 + e] );
+          }
+          *reinterpret_cast<uint2*>( dst ) = o.raw;
+        } else {
+          for ( int e = 0; e < 4; e++ ) {
+            if ( row + e < r ) {
+              dst[e] = __float2half_rn( acc[i][j][4 * q4 + e] );
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
+} // namespace
+
+bool gemm_tile_applicable( uint64_t s, uint64_t r, uint64_t b, const void* x, const void* w, const void* xout )
+{
+  (void)r;
+  return b >= 128 && s % 8 == 0 && ( ( reinterpret_cast<uintptr_t>( x ) | reinterpret_cast<uintptr_t>( w ) | reinterpret_cast<uintptr_t>( xout ) ) & 15u ) == 0;
+}
+
+int gemm_tile_launch( __half* xout, const __half* x, const __half* w, uint64_t s, uint64_t r, uint64_t b, hipStream_t st )
+{
+  const dim3 grid( (unsigned)( ( r + TM - 1 ) / TM ), (unsigned)( ( b + TN - 1 ) / TN ) );
+  GH_REQUIRE( grid.y <= 65535, "gh_matmul: batch too large" );
+  gemm_tile_kernel<<<grid, 256, 0, st>>>( xout, x, w, (uint32_t)s, (uint32_t)r, (uint32_t)b );
+  GH_LAUNCH_CHECK();
+  return GH_OK;
+}
+
+} // namespace gh

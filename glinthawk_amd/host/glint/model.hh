@@ -359,13 +359,40 @@ public:
       const auto& w = layers_[run[k]];
       // one table entry per (context, token) for this layer's rows
       GLINT_GH( gh_prefill_tables( layer_rows_dev( k ), pos_dev(), batch, n_tokens, row_bytes, nullptr, pf_token_rows(), pf_pos(), ops_.stream() ) );
-      ops_.matmul_qkv_rope_append( pq, pxb, w.wq, n, pf_pos(), base_.freq_cis_real, base_.freq_cis_imag, pf_token_rows() );
-      GLINT_GH( gh_attn_prefill( pq, layer_rows_dev( k ), pos_dev(), pxb, batch, n_tokens, max_start, &shape, hip::gh_type<DType>(), pf_attn_ws_.get(),
-                                 pf_attn_ws_bytes_, GH_ATTN_AUTO, ops_.stream() ) );
-      ops_.template matmul_accum<Config::dim, Config::dim>( px, pxb, w.wo, n, pxb, w.rms_ffn_weight );
-      ops_.matmul_silu_gate( phb, pxb, w.w1, n );
-      const DType* next_norm = k + 1 < run.size() ? layers_[run[k + 1]].rms_att_weight : nullptr;
-      ops_.template matmul_accum<Config::hidden_dim, Config::dim>( px, phb, w.w2, n, next_norm ? pxb : nullptr, next_norm );
+      if ( n < 128 ) {
+        // few tokens: the weight-streaming GEMM with fused follow-up ops, as in decode
+        ops_.matmul_qkv_rope_append( pq, pxb, w.wq, n, pf_pos(), base_.freq_cis_real, base_.freq_cis_imag, pf_token_rows() );
+        GLINT_GH( gh_attn_prefill( pq, layer_rows_dev( k ), pos_dev(), pxb, batch, n_tokens, max_start, &shape, hip::gh_type<DType>(), pf_attn_ws_.get(),
+                                   pf_attn_ws_bytes_, GH_ATTN_AUTO, ops_.stream() ) );
+        ops_.template matmul_accum<Config::dim, Config::dim>( px, pxb, w.wo, n, pxb, w.rms_ffn_weight );
+        ops_.matmul_silu_gate( phb, pxb, w.w1, n );
+        const DType* next_norm = k + 1 < run.size() ? layers_[run[k + 1]].rms_att_weight : nullptr;
+        ops_.template matmul_accum<Config::hidden_dim, Config::dim>( px, phb, w.w2, n, next_norm ? pxb : nullptr, next_norm );
+      } else {
+        // many tokens: MFMA-bound tile GEMMs storing DType directly, element-wise ops as separate
+        // (bandwidth-trivial) kernels -- the reference's op sequence on batch * n_tokens rows
+        DType* pkv = pf_kv_.get();
+        DType* pxb2 = pf_xb2_.get();
+        DType* phb2 = pf_hb2_.get();
+        ops_.template matmul<Config::dim, Config::dim>( pq, pxb, w.wq, n );
+        ops_.template matmul<Config::dim, Config::kv_dim * 2>( pkv, pxb, w.wkv, n );
+        GLINT_GH( gh_kv_append( pf_token_rows(), pkv, n, Config::kv_dim, hip::gh_type<DType>(), ops_.stream() ) );
+        GLINT_GH( gh_rope( n, pf_pos(), base_.freq_cis_real, base_.freq_cis_imag, pq, pf_token_rows(), Config::n_kv_heads, Config::gqa_size, Config::head_size,
+                           hip::gh_type<DType>(), ops_.stream() ) );
+        GLINT_GH( gh_attn_prefill( pq, layer_rows_dev( k ), pos_dev(), pxb, batch, n_tokens, max_start, &shape, hip::gh_type<DType>(), pf_attn_ws_.get(),
+                                   pf_attn_ws_bytes_, GH_ATTN_AUTO, ops_.stream() ) );
+        ops_.template matmul<Config::dim, Config::dim>( pxb2, pxb, w.wo, n );
+        ops_.template accum<Config::dim>( px, pxb2, n );
+        ops_.template rmsnorm<Config::dim>( pxb, px, reinterpret_cast<float32_t*>( temp_ ), w.rms_ffn_weight, n );
+        ops_.template matmul<Config::dim, Config::hidden_dim>( phb, pxb, w.w1, n );
+        ops_.template matmul<Config::dim, Config::hidden_dim>( phb2, pxb, w.w3, n );
+        ops_.template silu<Config::hidden_dim>( phb, phb2, n );
+        ops_.template matmul<Config::hidden_dim, Config::dim>( pxb, phb, w.w2, n );
+        ops_.template accum<Config::dim>( px, pxb, n );
+        if ( k + 1 < run.size() ) {
+          ops_.template rmsnorm<Config::dim>( pxb, px, reinterpret_cast<float32_t*>( temp_ ), layers_[run[k + 1]].rms_att_weight, n );
+        }
+      }
     }
 
     if ( acts_out_host != nullptr ) {
@@ -752,6 +779,11 @@ private:
     pf_xb_ = ops_.device_allocate( n * Config::dim * sizeof( DType ) );
     pf_q_ = ops_.device_allocate( n * Config::dim * sizeof( DType ) );
     pf_hb_ = ops_.device_allocate( n * Config::hidden_dim * sizeof( DType ) );
+    if ( n >= 128 ) {
+      pf_hb2_ = ops_.device_allocate( n * Config::hidden_dim * sizeof( DType ) );
+      pf_xb2_ = ops_.device_allocate( n * Config::dim * sizeof( DType ) );
+      pf_kv_ = ops_.device_allocate( n * Config::kv_dim * 2 * sizeof( DType ) );
+    }
     pf_tables_ = ops_.device_allocate( n * ( sizeof( void* ) + sizeof( uint32_t ) ) + 64 );
     const gh_shape shape = LlamaOperations::shape();
     // sized for the widest call: every context contributes all n tokens
@@ -763,7 +795,7 @@ private:
   uint32_t* pf_pos() const { return reinterpret_cast<uint32_t*>( pf_token_rows() + pf_capacity_ ); }
 
   DevicePtr base_storage_ {}, layer_storage_ {}, scratch_storage_ {}, attn_ws_ {}, tables_dev_ {};
-  DevicePtr pf_x_ {}, pf_xb_ {}, pf_q_ {}, pf_hb_ {}, pf_tables_ {}, pf_attn_ws_ {};
+  DevicePtr pf_x_ {}, pf_xb_ {}, pf_q_ {}, pf_hb_ {}, pf_hb2_ {}, pf_xb2_ {}, pf_kv_ {}, pf_tables_ {}, pf_attn_ws_ {};
   uint64_t pf_capacity_ { 0 }, pf_attn_ws_bytes_ { 0 };
   uint64_t attn_ws_bytes_ { 0 };
   uint8_t* tables_host_ { nullptr };

@@ -146,6 +146,31 @@ def test_matmul(dt, b, s, r):
         np.testing.assert_allclose(got, want, rtol=2e-5, atol=2e-5)
 
 
+# many rows of x at once (prompt tokens): the MFMA tile kernel, ragged edges in both dimensions
+@pytest.mark.parametrize("dt", ["f16", "f32"])
+@pytest.mark.parametrize("b,s,r", [(128, 64, 128), (130, 512, 200), (257, 288, 288), (300, 72, 37), (512, 1024, 130),
+                                   (1000, 776, 514), (129, 100, 64)])
+def test_matmul_many_rows(dt, b, s, r):
+    rng = np.random.default_rng(16)
+    x = rng.standard_normal((b, s)).astype(ndt(dt))
+    w = (rng.standard_normal((r, s)) / np.sqrt(s)).astype(ndt(dt))
+    got = ops.matmul(torch.from_numpy(x).cuda(), torch.from_numpy(w).cuda()).cpu().numpy()
+    want = O.matmul(x.astype(np.float32), w.astype(np.float32))
+    assert got.shape == (b, r)
+    assert_close(got, want, what=f"matmul {dt} {b}x{s}x{r}")
+
+
+def test_matmul_many_rows_layout_one_hot():
+    # x rows that select single columns of w: the tile kernel must return them bit for bit
+    s, r, b = 320, 200, 260
+    w = torch.arange(r * s, dtype=torch.float32).reshape(r, s).remainder(1000).half().cuda()
+    x = torch.zeros((b, s), dtype=torch.float16, device="cuda")
+    cols = [(7 * i + 3) % s for i in range(b)]
+    x[torch.arange(b), torch.tensor(cols)] = 1
+    got = ops.matmul(x, w)
+    assert torch.equal(got, w[:, cols].t().contiguous())
+
+
 def test_matmul_layout_one_hot():
     s, r = 256, 192
     w = torch.arange(r * s, dtype=torch.float32).reshape(r, s).remainder(1000).half().cuda()

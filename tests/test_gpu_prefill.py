@@ -102,7 +102,9 @@ from test_gpu_stage import SHAPES, OracleModel, d2h, load_weights, make_weights 
 
 
 @pytest.mark.parametrize("name,dtype,n_prompt", [("test-gqa4", "f16", 37), ("test-mha", "f16", 20), ("stories15m", "f32", 9),
-                                                 ("test-tiny", "f32", 5)])
+                                                 ("test-tiny", "f32", 5),
+                                                 # 3 prompts x n >= 128 tokens: the tile-GEMM sequence
+                                                 ("test-gqa4", "f16", 50), ("stories15m", "f32", 44), ("stories15m", "f16", 64)])
 def test_stage_prefill_equals_token_by_token(name, dtype, n_prompt):
     cfg = SHAPES[name]
     np_dt = np.float16 if dtype == "f16" else np.float32
