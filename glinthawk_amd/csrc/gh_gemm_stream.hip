@@ -3,12 +3,15 @@
 // exactly once, so the kernel is built like a streaming read:
 //
 //   work-group = 4 waves = 128 weight rows x one K range; wave = 32 rows x all 64 batch columns
-//   weights     global -> registers with fully coalesced 16-byte loads.  A register slab is 32 rows x
-//               256 k: both 256-byte halves of a row are requested back to back, so the memory system
-//               sees 512 contiguous bytes per row per visit (256-byte visits cost a quarter of the
-//               bandwidth on this part).  Two register sets: slab i+1 is in flight while slab i is
-//               consumed.  From registers each 128-k half goes through a wave-private LDS tile
-//               (XOR-swizzled 16-byte chunks) into MFMA operand order.
+//   weights     global -> registers with fully coalesced 16-byte buffer loads (scalar row/k offsets,
+//               rows past the end read as zero by the descriptor's bound).  A register slab is 32 rows
+//               x 256 k, 512 contiguous bytes per row per visit.  Two register sets: slab i+1 is in
+//               flight while slab i is consumed.  From registers each 128-k half goes through a
+//               wave-private LDS tile (XOR-swizzled 16-byte chunks) into MFMA operand order.
+//   k order     every work-group walks its K range from a different starting slab and wraps around.
+//               Work-groups that start together would otherwise all read the same column range of
+//               their rows, and rows are a power-of-two stride apart: those addresses fall on few
+//               HBM channels (measured: 4.4 TB/s for 256-byte visits in lock step, 6.3 TB/s rotated).
 //   activations one (64 x 128) tile per half shared by the work-group through LDS (two buffers); this
 //               is the only block-level barrier and the weight loads stay in flight across it
 //   math        v_mfma_f32_32x32x16_f16: A = 32 weight rows, B = 32 batch columns, two column tiles
@@ -35,19 +38,20 @@ struct WSlab
   uint4 v[2][8];
 };
 
-__device__ __forceinline__ void load_w_slab( WSlab& dst, const __half* __restrict__ w, uint64_t ld, uint32_t wave_row0, uint32_t n_rows, uint32_t k0, uint32_t k_end )
+__device__ __forceinline__ uint4 buffer_load16( __amdgpu_buffer_rsrc_t rsrc, uint32_t lane_offset, uint32_t uniform_offset )
 {
-  const uint32_t lane = threadIdx.x & 63;
-  const uint32_t c = lane & 15, g4 = lane >> 4;
-  const bool k_ok = k0 < k_end; // K ranges are multiples of SLAB_K
+  return __builtin_bit_cast( uint4, __builtin_amdgcn_raw_buffer_load_b128( rsrc, lane_offset, uniform_offset, 0 ) );
+}
+
+// `rsrc` starts at the wave's first row; lane_offset = g4 * row bytes + 16 c; kb = byte offset of the slab in the row
+__device__ __forceinline__ void load_w_slab( WSlab& dst, __amdgpu_buffer_rsrc_t rsrc, uint32_t lane_offset, uint32_t ld_bytes, uint32_t kb )
+{
 #pragma unroll
   for ( int j = 0; j < 8; j++ ) {
-    const uint32_t row = wave_row0 + 4 * j + g4;
-    const bool ok = k_ok && row < n_rows;
-    const __half* p = w + (uint64_t)row * ld + k0 + 8 * c;
+    const uint32_t row_offset = 4 * j * ld_bytes + kb;
     // both halves of the row back to back: 512 contiguous bytes per row reach the memory system together
-    dst.v[0][j] = ok ? *reinterpret_cast<const uint4*>( p ) : make_uint4( 0, 0, 0, 0 );
-    dst.v[1][j] = ok ? *reinterpret_cast<const uint4*>( p + HALF_K ) : make_uint4( 0, 0, 0, 0 );
+    dst.v[0][j] = buffer_load16( rsrc, lane_offset, row_offset );
+    dst.v[1][j] = buffer_load16( rsrc, lane_offset + 2 * HALF_K, row_offset );
   }
 }
 
@@ -68,28 +72,12 @@ struct XSlab
   uint4 v[2][4];
 };
 
-__device__ __forceinline__ void load_x_slab( XSlab& dst, const __half* __restrict__ x, uint64_t ld, uint32_t col0, uint32_t n_cols, uint32_t k0, uint32_t k_end )
+// `rsrc` starts at the work-group's first column; lane_offset = (t / 16) * row bytes + 16 * (t % 16)
+__device__ __forceinline__ void load_x_half( XSlab& dst, __amdgpu_buffer_rsrc_t rsrc, uint32_t lane_offset, uint32_t ld_bytes, uint32_t kb, int h )
 {
-  const uint32_t chunk = threadIdx.x & 15;
-  const bool k_ok = k0 < k_end;
 #pragma unroll
   for ( int i = 0; i < 4; i++ ) {
-    const uint32_t col = col0 + ( threadIdx.x >> 4 ) + 16 * i;
-    const bool ok = k_ok && col < n_cols;
-    const __half* p = x + (uint64_t)col * ld + k0 + 8 * chunk;
-    dst.v[0][i] = ok ? *reinterpret_cast<const uint4*>( p ) : make_uint4( 0, 0, 0, 0 );
-    dst.v[1][i] = ok ? *reinterpret_cast<const uint4*>( p + HALF_K ) : make_uint4( 0, 0, 0, 0 );
-  }
-}
-
-__device__ __forceinline__ void load_x_half( XSlab& dst, const __half* __restrict__ x, uint64_t ld, uint32_t col0, uint32_t n_cols, uint32_t k0, uint32_t k_end, int h )
-{
-  const uint32_t chunk = threadIdx.x & 15;
-  const bool k_ok = k0 < k_end;
-#pragma unroll
-  for ( int i = 0; i < 4; i++ ) {
-    const uint32_t col = col0 + ( threadIdx.x >> 4 ) + 16 * i;
-    dst.v[h][i] = ( k_ok && col < n_cols ) ? *reinterpret_cast<const uint4*>( x + (uint64_t)col * ld + k0 + h * HALF_K + 8 * chunk ) : make_uint4( 0, 0, 0, 0 );
+    dst.v[h][i] = buffer_load16( rsrc, lane_offset + h * 2 * HALF_K, 16 * i * ld_bytes + kb );
   }
 }
 
@@ -135,13 +123,22 @@ __global__ __launch_bounds__( 256, 2 ) void gemm_stream_kernel( __half* __restri
   __shared__ uint4 s_x[2][COLS * 16]; // 2 x 16 KiB
   __shared__ uint4 s_w[4][32 * 16];   // 4 x 8 KiB, one per wave
 
-  const uint32_t wave = threadIdx.x >> 6;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane( threadIdx.x >> 6 ); // provably uniform: keeps descriptors in SGPRs
   const uint32_t lane = threadIdx.x & 63;
   const uint32_t row0 = blockIdx.x * WG_ROWS + wave * 32;
   const uint32_t col0 = blockIdx.y * COLS;
   const uint32_t k_begin = blockIdx.z * k_per_split;
   const uint32_t k_end = min( s, k_begin + k_per_split );
+  const uint32_t ld_bytes = s * 2;
   uint4* wtile = s_w[wave];
+
+  // descriptors bounded to the wave's rows / the work-group's columns: anything past the matrix reads as zero
+  const uint32_t w_rows = row0 < r ? min( 32u, r - row0 ) : 0u;
+  const uint32_t x_cols = col0 < b ? min( (uint32_t)COLS, b - col0 ) : 0u;
+  const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc( const_cast<__half*>( w + (uint64_t)row0 * s ), 0, (int)( w_rows * ld_bytes ), 0x00020000 );
+  const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc( const_cast<__half*>( x + (uint64_t)col0 * s ), 0, (int)( x_cols * ld_bytes ), 0x00020000 );
+  const uint32_t w_lane = ( lane >> 4 ) * ld_bytes + ( lane & 15 ) * 16;
+  const uint32_t x_lane = ( threadIdx.x >> 4 ) * ld_bytes + ( threadIdx.x & 15 ) * 16;
 
   f32x16 acc[2];
 #pragma unroll
@@ -156,22 +153,34 @@ __global__ __launch_bounds__( 256, 2 ) void gemm_stream_kernel( __half* __restri
   // other.  Loads retire in order, so the issue order matters: the weight loads of slab i+1 go out
   // first in iteration i, the activation halves of slab i+1 follow as their registers are staged;
   // everything iteration i+1 waits for is then older than the weight loads it issues itself.
+  const uint32_t n_slabs = ( k_end - k_begin ) / SLAB_K; // K ranges are multiples of SLAB_K
+  uint32_t cur = ( ( blockIdx.x + blockIdx.z ) * 3u ) % n_slabs; // rotated start, see the header
   WSlab wr[2];
   XSlab xr;
-  load_x_slab( xr, x, s, col0, b, k_begin, k_end );
-  load_w_slab( wr[0], w, s, row0, r, k_begin, k_end );
-
-  for ( uint32_t k0 = k_begin; k0 < k_end; k0 += 2 * SLAB_K ) {
+  {
+    const uint32_t kb = ( k_begin + cur * SLAB_K ) * 2;
+    load_x_half( xr, x_rsrc, x_lane, ld_bytes, kb, 0 );
+    load_x_half( xr, x_rsrc, x_lane, ld_bytes, kb, 1 );
+    load_w_slab( wr[0], w_rsrc, w_lane, ld_bytes, kb );
+  }
+  for ( uint32_t j0 = 0; j0 < n_slabs; j0 += 2 ) {
 #pragma unroll
     for ( int set = 0; set < 2; set++ ) {
-      const uint32_t ks = k0 + set * SLAB_K;
-      if ( ks < k_end ) { // uniform across the work-group
-        load_w_slab( wr[set ^ 1], w, s, row0, r, ks + SLAB_K, k_end );
+      const uint32_t j = j0 + set;
+      if ( j < n_slabs ) { // uniform across the work-group
+        cur = cur + 1 == n_slabs ? 0 : cur + 1;
+        const bool more = j + 1 < n_slabs;
+        const uint32_t kb = ( k_begin + cur * SLAB_K ) * 2;
+        if ( more ) {
+          load_w_slab( wr[set ^ 1], w_rsrc, w_lane, ld_bytes, kb );
+        }
 #pragma unroll
         for ( int h = 0; h < 2; h++ ) {
           stage_x_half( s_x[h], xr, h );
           stage_w_half( wtile, wr[set], h );
-          load_x_half( xr, x, s, col0, b, ks + SLAB_K, k_end, h ); // same registers, next slab
+          if ( more ) {
+            load_x_half( xr, x_rsrc, x_lane, ld_bytes, kb, h ); // same registers, next slab
+          }
           __syncthreads();
           half_mfma( acc, wtile, s_x[h] );
         }
@@ -242,7 +251,7 @@ void launch( dim3 grid, hipStream_t st, bool split, __half* xout, float* partial
 bool gemm_stream_applicable( uint64_t s, uint64_t r, uint64_t b, const void* x, const void* w, const void* xout )
 {
   (void)b;
-  return s % SLAB_K == 0 && r % 4 == 0 && ( ( reinterpret_cast<uintptr_t>( x ) | reinterpret_cast<uintptr_t>( w ) | reinterpret_cast<uintptr_t>( xout ) ) & 15u ) == 0;
+  return s % SLAB_K == 0 && s < ( 1u << 24 ) && r % 4 == 0 && ( ( reinterpret_cast<uintptr_t>( x ) | reinterpret_cast<uintptr_t>( w ) | reinterpret_cast<uintptr_t>( xout ) ) & 15u ) == 0;
 }
 
 // picks the K split; returns the number of splits and k per split
@@ -251,9 +260,16 @@ void gemm_stream_plan( uint64_t s, uint64_t r, uint64_t b, uint32_t* splits_out,
   const uint64_t tiles = ( ( r + WG_ROWS - 1 ) / WG_ROWS ) * ( ( b + COLS - 1 ) / COLS );
   uint32_t splits = 1;
   if ( tiles < (uint64_t)g_target_wgs ) {
-    splits = (uint32_t)( ( g_target_wgs + tiles - 1 ) / tiles );
-    const uint32_t max_by_k = (uint32_t)std::max<uint64_t>( 1, s / ( 4 * SLAB_K ) ); // at least 4 slabs per work-group
-    splits = std::min( splits, max_by_k );
+    // two work-groups per CU hide each other's staging and MFMA phases, but only pay off while every
+    // work-group still streams at least 8 slabs; otherwise one per CU with at least 4 slabs each
+    const uint32_t two_per_cu = (uint32_t)( ( 2 * g_target_wgs + tiles - 1 ) / tiles );
+    if ( s / two_per_cu >= 8 * SLAB_K ) {
+      splits = two_per_cu;
+    } else {
+      splits = (uint32_t)( ( g_target_wgs + tiles - 1 ) / tiles );
+      const uint32_t max_by_k = (uint32_t)std::max<uint64_t>( 1, s / ( 4 * SLAB_K ) );
+      splits = std::min( splits, max_by_k );
+    }
   }
   uint32_t k_per_split = (uint32_t)( ( s + splits - 1 ) / splits );
   k_per_split = ( k_per_split + SLAB_K - 1 ) / SLAB_K * SLAB_K;
