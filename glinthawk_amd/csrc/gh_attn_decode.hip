@@ -313,17 +313,25 @@ __global__ __launch_bounds__( 256 ) void attn_decode_valu_kernel( const __half* 
   const __half* kp = job.base + (uint64_t)job.h * HS + 8 * c;
   const uint4 zero4 = make_uint4( 0, 0, 0, 0 );
 
+  // 16-token tiles in rotated order, a different starting tile per block (see the mfma kernel)
+  const uint32_t n_tiles = ( job.t_end - job.t_begin + 15 ) / 16;
+  uint32_t tile_i = ( ( job.ctx * 5u + job.split * 3u ) * 7u ) % n_tiles;
+  uint32_t t0 = job.t_begin + 16 * tile_i;
+
   uint4 kn[4], vn[4]; // prefetched block
 #pragma unroll
   for ( int j = 0; j < 4; j++ ) {
-    const uint32_t tok = job.t_begin + 4 * j + r;
+    const uint32_t tok = t0 + 4 * j + r;
     const bool ok = tok < job.t_end;
     const __half* row = kp + (uint64_t)tok * row_elems;
     kn[j] = ok ? load16( row ) : zero4;
     vn[j] = ok ? load16( row + v_off ) : zero4;
   }
 
-  for ( uint32_t t0 = job.t_begin; t0 < job.t_end; t0 += 16 ) {
+  for ( uint32_t it = 0; it < n_tiles; it++ ) {
+    tile_i = tile_i + 1 == n_tiles ? 0 : tile_i + 1;
+    const uint32_t t_next = job.t_begin + 16 * tile_i;
+    const bool more = it + 1 < n_tiles;
     uint4 kc[4], vc[4];
 #pragma unroll
     for ( int j = 0; j < 4; j++ ) {
@@ -333,8 +341,8 @@ __global__ __launch_bounds__( 256 ) void attn_decode_valu_kernel( const __half* 
     // prefetch the next 16 tokens while this block is processed
 #pragma unroll
     for ( int j = 0; j < 4; j++ ) {
-      const uint32_t tok = t0 + 16 + 4 * j + r;
-      const bool ok = tok < job.t_end;
+      const uint32_t tok = t_next + 4 * j + r;
+      const bool ok = more && tok < job.t_end;
       const __half* row = kp + (uint64_t)tok * row_elems;
       kn[j] = ok ? load16( row ) : zero4;
       vn[j] = ok ? load16( row + v_off ) : zero4;
@@ -378,6 +386,7 @@ __global__ __launch_bounds__( 256 ) void attn_decode_valu_kernel( const __half* 
         }
       }
     }
+    t0 = t_next;
   }
 
   // merge the four token streams (lane rows) of the wave
@@ -492,17 +501,28 @@ __global__ __launch_bounds__( 256 ) void attn_decode_mfma_kernel( const __half* 
   const __half* kp = job.base + (uint64_t)job.h * HS + 8 * c;
   const uint4 zero4 = make_uint4( 0, 0, 0, 0 );
 
+  // The 16-token tiles of the range are visited from a starting tile that differs between blocks,
+  // wrapping around (the online softmax does not care about the order).  Blocks launched together
+  // otherwise walk their ranges in lock step, and ranges of different contexts and splits lie
+  // large power-of-two distances apart: such addresses share few HBM channels.
+  const uint32_t n_tiles = ( job.t_end - job.t_begin + 15 ) / 16;
+  uint32_t tile_i = ( ( job.ctx * 5u + job.split * 3u ) * 7u ) % n_tiles;
+  uint32_t t0 = job.t_begin + 16 * tile_i;
+
   uint4 kn[4], vn[4];
 #pragma unroll
   for ( int i = 0; i < 4; i++ ) {
-    const uint32_t tok = job.t_begin + 4 * g4 + i;
+    const uint32_t tok = t0 + 4 * g4 + i;
     const bool ok = tok < job.t_end;
     const __half* row = kp + (uint64_t)tok * row_elems;
     kn[i] = ok ? load16( row ) : zero4;
     vn[i] = ok ? load16( row + v_off ) : zero4;
   }
 
-  for ( uint32_t t0 = job.t_begin; t0 < job.t_end; t0 += 16 ) {
+  for ( uint32_t it = 0; it < n_tiles; it++ ) {
+    tile_i = tile_i + 1 == n_tiles ? 0 : tile_i + 1;
+    const uint32_t t_next = job.t_begin + 16 * tile_i;
+    const bool more = it + 1 < n_tiles;
     uint4 vc[4];
     // K tile into LDS: token 4*g4+i, chunk c, stored at chunk position c ^ token
 #pragma unroll
@@ -514,8 +534,8 @@ __global__ __launch_bounds__( 256 ) void attn_decode_mfma_kernel( const __half* 
     // prefetch the next tile
 #pragma unroll
     for ( int i = 0; i < 4; i++ ) {
-      const uint32_t tok = t0 + 16 + 4 * g4 + i;
-      const bool ok = tok < job.t_end;
+      const uint32_t tok = t_next + 4 * g4 + i;
+      const bool ok = more && tok < job.t_end;
       const __half* row = kp + (uint64_t)tok * row_elems;
       kn[i] = ok ? load16( row ) : zero4;
       vn[i] = ok ? load16( row + v_off ) : zero4;
@@ -585,6 +605,7 @@ __global__ __launch_bounds__( 256 ) void attn_decode_mfma_kernel( const __half* 
       acc[2 * w] = __builtin_amdgcn_mfma_f32_16x16x16f16( pa, __builtin_bit_cast( f16x4, lo ), acc[2 * w], 0, 0, 0 );
       acc[2 * w + 1] = __builtin_amdgcn_mfma_f32_16x16x16f16( pa, __builtin_bit_cast( f16x4, hi ), acc[2 * w + 1], 0, 0, 0 );
     }
+    t0 = t_next;
   }
 
   // total sum of head c over the four lane groups
