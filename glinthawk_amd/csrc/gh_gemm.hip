@@ -23,7 +23,9 @@ int gemm_stream_launch( __half* xout, float* partial, const __half* x, const __h
 void gemm_stream_tuning( int target_wgs, int depth );
 // large-batch (prefill) kernel (gh_gemm_tile.hip)
 bool gemm_tile_applicable( uint64_t s, uint64_t r, uint64_t b, const void* x, const void* w, const void* xout );
-int gemm_tile_launch( __half* xout, const __half* x, const __half* w, uint64_t s, uint64_t r, uint64_t b, hipStream_t st );
+void gemm_tile_plan( uint64_t s, uint64_t r, uint64_t b, uint32_t* splits_out, uint32_t* k_per_split_out );
+int gemm_tile_launch( __half* xout, float* partial, const __half* x, const __half* w, uint64_t s, uint64_t r, uint64_t b, uint32_t splits, uint32_t k_per_split,
+                      hipStream_t st );
 
 namespace {
 
@@ -252,10 +254,20 @@ int gemm_partials( void* xout, const void* x, const void* w, uint64_t s, uint64_
   GH_REQUIRE( dt == GH_F16, "gh_matmul: unsupported dtype %d", (int)dt );
 
   // many tokens at once (prefill): the MFMA-bound tile kernel; few (decode): the weight-streaming one
-  if ( !want_partials && ( g_force_kernel == 0 || g_force_kernel == 3 ) && gemm_tile_applicable( s, r, b, x, w, xout ) ) {
-    return gemm_tile_launch( static_cast<__half*>( xout ), static_cast<const __half*>( x ), static_cast<const __half*>( w ), s, r, b, st );
+  if ( ( g_force_kernel == 0 || g_force_kernel == 3 ) && gemm_tile_applicable( s, r, b, x, w, xout ? xout : x ) ) {
+    uint32_t splits = 1, k_per_split = 0;
+    gemm_tile_plan( s, r, b, &splits, &k_per_split );
+    float* ws = nullptr;
+    if ( want_partials || splits > 1 ) {
+      if ( int rc = ensure_workspace( (uint64_t)splits * b * r * sizeof( float ), &ws ) ) {
+        return rc;
+      }
+      *partial_out = ws;
+      *splits_out = splits;
+    }
+    return gemm_tile_launch( static_cast<__half*>( xout ), ws, static_cast<const __half*>( x ), static_cast<const __half*>( w ), s, r, b, splits, k_per_split, st );
   }
-  GH_REQUIRE( g_force_kernel != 3, "gh_matmul: the tile kernel needs b >= 128, s %% 8 == 0 and 16-byte aligned operands" );
+  GH_REQUIRE( g_force_kernel != 3, "gh_matmul: the tile kernel needs b > 64, s %% 8 == 0 and 16-byte aligned operands" );
 
   if ( g_force_kernel != 1 && gemm_stream_applicable( s, r, b, x, w, xout ? xout : x ) ) {
     uint32_t splits = 1, k_per_split = 0;

@@ -109,7 +109,7 @@ __device__ __forceinline__ void half_mfma( f32x16 acc[2], const uint4* wtile, co
   }
 }
 
-// grid: (row slabs, column slabs, k splits).  s % 256 == 0, 16-byte aligned operands.
+// grid: (row blocks x column slabs, 1, k splits).  s % 256 == 0, 16-byte aligned operands.
 template<bool SPLIT>
 __global__ __launch_bounds__( 256, 2 ) void gemm_stream_kernel( __half* __restrict__ xout,
                                                              float* __restrict__ partial,
@@ -118,15 +118,28 @@ __global__ __launch_bounds__( 256, 2 ) void gemm_stream_kernel( __half* __restri
                                                              uint32_t s,
                                                              uint32_t r,
                                                              uint32_t b,
-                                                             uint32_t k_per_split )
+                                                             uint32_t k_per_split,
+                                                             uint32_t n_col_slabs )
 {
   __shared__ uint4 s_x[2][COLS * 16]; // 2 x 16 KiB
   __shared__ uint4 s_w[4][32 * 16];   // 4 x 8 KiB, one per wave
 
   const uint32_t wave = __builtin_amdgcn_readfirstlane( threadIdx.x >> 6 ); // provably uniform: keeps descriptors in SGPRs
   const uint32_t lane = threadIdx.x & 63;
-  const uint32_t row0 = blockIdx.x * WG_ROWS + wave * 32;
-  const uint32_t col0 = blockIdx.y * COLS;
+  // Work-groups are handed to the 8 XCDs round robin by their linear index, and every XCD has its own
+  // L2.  With more than one column slab, the slabs of one row block get indices 8 apart and adjacent
+  // in time: they run on the same XCD together and the weights leave HBM once, not once per slab.
+  uint32_t row_block = blockIdx.x, col_slab = 0;
+  if ( n_col_slabs > 1 ) {
+    const uint32_t idx = blockIdx.x >> 3;
+    col_slab = idx % n_col_slabs;
+    row_block = ( idx / n_col_slabs ) * 8 + ( blockIdx.x & 7 );
+    if ( row_block * WG_ROWS >= r ) {
+      return; // padding of the grid to a multiple of 8 row blocks (whole work-group)
+    }
+  }
+  const uint32_t row0 = row_block * WG_ROWS + wave * 32;
+  const uint32_t col0 = col_slab * COLS;
   const uint32_t k_begin = blockIdx.z * k_per_split;
   const uint32_t k_end = min( s, k_begin + k_per_split );
   const uint32_t ld_bytes = s * 2;
@@ -154,7 +167,7 @@ __global__ __launch_bounds__( 256, 2 ) void gemm_stream_kernel( __half* __restri
   // first in iteration i, the activation halves of slab i+1 follow as their registers are staged;
   // everything iteration i+1 waits for is then older than the weight loads it issues itself.
   const uint32_t n_slabs = ( k_end - k_begin ) / SLAB_K; // K ranges are multiples of SLAB_K
-  uint32_t cur = ( ( blockIdx.x + blockIdx.z ) * 3u ) % n_slabs; // rotated start, see the header
+  uint32_t cur = ( ( row_block + blockIdx.z ) * 3u ) % n_slabs; // rotated start, see the header
   WSlab wr[2];
   XSlab xr;
   {
@@ -237,12 +250,12 @@ __global__ __launch_bounds__( 256, 2 ) void gemm_stream_kernel( __half* __restri
 int g_target_wgs = 256;
 
 void launch( dim3 grid, hipStream_t st, bool split, __half* xout, float* partial, const __half* x, const __half* w, uint32_t s, uint32_t r, uint32_t b,
-             uint32_t k_per_split )
+             uint32_t k_per_split, uint32_t n_col_slabs )
 {
   if ( split ) {
-    gemm_stream_kernel<true><<<grid, 256, 0, st>>>( xout, partial, x, w, s, r, b, k_per_split );
+    gemm_stream_kernel<true><<<grid, 256, 0, st>>>( xout, partial, x, w, s, r, b, k_per_split, n_col_slabs );
   } else {
-    gemm_stream_kernel<false><<<grid, 256, 0, st>>>( xout, partial, x, w, s, r, b, k_per_split );
+    gemm_stream_kernel<false><<<grid, 256, 0, st>>>( xout, partial, x, w, s, r, b, k_per_split, n_col_slabs );
   }
 }
 
@@ -280,10 +293,12 @@ void gemm_stream_plan( uint64_t s, uint64_t r, uint64_t b, uint32_t* splits_out,
 int gemm_stream_launch( __half* xout, float* partial, const __half* x, const __half* w, uint64_t s, uint64_t r, uint64_t b, uint32_t splits,
                         uint32_t k_per_split, bool write_partials, hipStream_t st )
 {
-  const dim3 grid( (unsigned)( ( r + WG_ROWS - 1 ) / WG_ROWS ), (unsigned)( ( b + COLS - 1 ) / COLS ), splits );
-  GH_REQUIRE( grid.y <= 65535 && grid.z <= 65535, "gh_matmul: grid too large" );
-  const bool split = write_partials;
-  launch( grid, st, split, xout, partial, x, w, (uint32_t)s, (uint32_t)r, (uint32_t)b, k_per_split );
+  const uint64_t row_blocks = ( r + WG_ROWS - 1 ) / WG_ROWS;
+  const uint64_t col_slabs = ( b + COLS - 1 ) / COLS;
+  const uint64_t gx = col_slabs == 1 ? row_blocks : ( row_blocks + 7 ) / 8 * 8 * col_slabs;
+  GH_REQUIRE( gx < ( 1ull << 31 ) && splits <= 65535, "gh_matmul: grid too large" );
+  const dim3 grid( (unsigned)gx, 1, splits );
+  launch( grid, st, write_partials, xout, partial, x, w, (uint32_t)s, (uint32_t)r, (uint32_t)b, k_per_split, (uint32_t)col_slabs );
   GH_LAUNCH_CHECK();
   return GH_OK;
 }

@@ -7,7 +7,17 @@
 //   operands    global -> registers (next step in flight while the current one is multiplied)
 //               -> LDS, 16-byte chunks XOR-swizzled so that the MFMA-order reads are conflict free,
 //               two LDS buffers, one barrier per step
+//   tile order  work-groups reach the 8 XCDs round robin by linear index and each XCD has its own L2.
+//               An XCD owns every 8th row tile and walks its (row tile, token tile) grid in patches
+//               of GM x GN tiles that are resident together (64 = 2 work-groups on each of its 32
+//               CUs): a patch re-reads GM weight tiles and GN activation tiles out of L2 instead of
+//               64 + 64 from memory.  Row-major order re-streamed the whole weight matrix once per
+//               token tile and was bound by that (4.5 TB/s), not by MFMA.
+//   split K     when the tiles are too few to fill the chip, K is split across work-groups and the
+//               fp32 partials (splits, b, r) are summed by the caller's reduce / fused epilogue
 #include "gh_common.h"
+
+#include <algorithm>
 
 namespace gh {
 
@@ -50,23 +60,48 @@ __device__ __forceinline__ void store_frag( uint4* tile, const Frag& f )
   }
 }
 
-// grid: (row tiles, token tiles).  s % 8 == 0, 16-byte aligned operands.
+struct TileOrder
+{
+  uint32_t row_tiles, token_tiles; // of the whole product
+  uint32_t gm, gn;                 // patch: row tiles x token tiles
+  uint32_t patches_n;              // patches along the token direction
+};
+
+// grid: (8 * padded tiles per XCD, 1, k splits).  s % 8 == 0, 16-byte aligned operands.
+template<bool SPLIT>
 __global__ __launch_bounds__( 256 ) void gemm_tile_kernel( __half* __restrict__ xout,
+                                                           float* __restrict__ partial,
                                                            const __half* __restrict__ x,
                                                            const __half* __restrict__ w,
                                                            uint32_t s,
                                                            uint32_t r,
-                                                           uint32_t b )
+                                                           uint32_t b,
+                                                           uint32_t k_per_split,
+                                                           TileOrder ord )
 {
   __shared__ uint4 s_w[2][TM * 8]; // 2 x 16 KiB
   __shared__ uint4 s_x[2][TN * 8]; // 2 x 16 KiB
 
+  // linear index -> XCD, then patch by patch inside the XCD, token tiles fastest inside a patch
+  const uint32_t xcd = blockIdx.x & 7;
+  const uint32_t idx = blockIdx.x >> 3;
+  const uint32_t per_patch = ord.gm * ord.gn;
+  const uint32_t patch = idx / per_patch, in_patch = idx % per_patch;
+  const uint32_t patch_m = patch / ord.patches_n, patch_n = patch % ord.patches_n;
+  const uint32_t row_tile = ( patch_m * ord.gm + in_patch / ord.gn ) * 8 + xcd;
+  const uint32_t token_tile = patch_n * ord.gn + in_patch % ord.gn;
+  if ( row_tile >= ord.row_tiles || token_tile >= ord.token_tiles ) {
+    return; // padding of the last patches (whole work-group)
+  }
+
   const uint32_t wave = threadIdx.x >> 6;
   const uint32_t lane = threadIdx.x & 63;
   const uint32_t wm = wave & 1, wn = wave >> 1; // wave position inside the tile
-  const uint32_t row0 = blockIdx.x * TM;
-  const uint32_t col0 = blockIdx.y * TN;
+  const uint32_t row0 = row_tile * TM;
+  const uint32_t col0 = token_tile * TN;
   const uint32_t lr = lane & 31, g2 = lane >> 5;
+  const uint32_t k_begin = blockIdx.z * k_per_split;
+  const uint32_t k_end = min( s, k_begin + k_per_split );
 
   f32x16 acc[2][2];
 #pragma unroll
@@ -81,16 +116,16 @@ __global__ __launch_bounds__( 256 ) void gemm_tile_kernel( __half* __restrict__ 
   }
 
   Frag fw, fx;
-  load_frag( fw, w, s, row0, r, 0, s );
-  load_frag( fx, x, s, col0, b, 0, s );
+  load_frag( fw, w, s, row0, r, k_begin, k_end );
+  load_frag( fx, x, s, col0, b, k_begin, k_end );
   int buf = 0;
-  for ( uint32_t k0 = 0; k0 < s; k0 += TK ) {
+  for ( uint32_t k0 = k_begin; k0 < k_end; k0 += TK ) {
     store_frag( s_w[buf], fw );
     store_frag( s_x[buf], fx );
     __syncthreads();
-    if ( k0 + TK < s ) {
-      load_frag( fw, w, s, row0, r, k0 + TK, s );
-      load_frag( fx, x, s, col0, b, k0 + TK, s );
+    if ( k0 + TK < k_end ) {
+      load_frag( fw, w, s, row0, r, k0 + TK, k_end );
+      load_frag( fx, x, s, col0, b, k0 + TK, k_end );
     }
     const uint4* lw = s_w[buf];
     const uint4* lx = s_x[buf];
@@ -126,6 +161,19 @@ __global__ __launch_bounds__( 256 ) void gemm_tile_kernel( __half* __restrict__ 
 #pragma unroll
       for ( int q4 = 0; q4 < 4; q4++ ) {
         const uint32_t row = row0 + wm * 64 + 32 * i + 8 * q4 + 4 * g2;
+        if ( SPLIT ) {
+          float* dst = partial + ( (uint64_t)blockIdx.z * b + col ) * r + row;
+          if ( row + 3 < r && ( r & 3 ) == 0 ) {
+            *reinterpret_cast<float4*>( dst ) = make_float4( acc[i][j][4 * q4], acc[i][j][4 * q4 + 1], acc[i][j][4 * q4 + 2], acc[i][j][4 * q4 + 3] );
+          } else {
+            for ( int e = 0; e < 4; e++ ) {
+              if ( row + e < r ) {
+                dst[e] = acc[i][j][4 * q4 + e];
+              }
+            }
+          }
+          continue;
+        }
         __half* dst = xout + (uint64_t)col * r + row;
         if ( row + 3 < r && ( r & 3 ) == 0 ) {
           union
@@ -155,14 +203,47 @@ __global__ __launch_bounds__( 256 ) void gemm_tile_kernel( __half* __restrict__ 
 bool gemm_tile_applicable( uint64_t s, uint64_t r, uint64_t b, const void* x, const void* w, const void* xout )
 {
   (void)r;
-  return b >= 128 && s % 8 == 0 && ( ( reinterpret_cast<uintptr_t>( x ) | reinterpret_cast<uintptr_t>( w ) | reinterpret_cast<uintptr_t>( xout ) ) & 15u ) == 0;
+  return b > 64 && s % 8 == 0 && ( ( reinterpret_cast<uintptr_t>( x ) | reinterpret_cast<uintptr_t>( w ) | reinterpret_cast<uintptr_t>( xout ) ) & 15u ) == 0;
 }
 
-int gemm_tile_launch( __half* xout, const __half* x, const __half* w, uint64_t s, uint64_t r, uint64_t b, hipStream_t st )
+// K split so that about two work-groups per CU exist, each with at least 8 steps of K
+void gemm_tile_plan( uint64_t s, uint64_t r, uint64_t b, uint32_t* splits_out, uint32_t* k_per_split_out )
 {
-  const dim3 grid( (unsigned)( ( r + TM - 1 ) / TM ), (unsigned)( ( b + TN - 1 ) / TN ) );
-  GH_REQUIRE( grid.y <= 65535, "gh_matmul: batch too large" );
-  gemm_tile_kernel<<<grid, 256, 0, st>>>( xout, x, w, (uint32_t)s, (uint32_t)r, (uint32_t)b );
+  const uint64_t tiles = ( ( r + TM - 1 ) / TM ) * ( ( b + TN - 1 ) / TN );
+  uint32_t splits = 1;
+  if ( tiles < 384 ) {
+    splits = (uint32_t)( ( 512 + tiles - 1 ) / tiles );
+    splits = std::min<uint32_t>( splits, (uint32_t)std::max<uint64_t>( 1, s / ( 8 * TK ) ) );
+    splits = std::min<uint32_t>( splits, 16 );
+  }
+  uint32_t k_per_split = (uint32_t)( ( s + splits - 1 ) / splits );
+  k_per_split = ( k_per_split + TK - 1 ) / TK * TK;
+  *splits_out = (uint32_t)( ( s + k_per_split - 1 ) / k_per_split );
+  *k_per_split_out = k_per_split;
+}
+
+// `partial` != nullptr: fp32 partial sums (splits, b, r) instead of xout
+int gemm_tile_launch( __half* xout, float* partial, const __half* x, const __half* w, uint64_t s, uint64_t r, uint64_t b, uint32_t splits, uint32_t k_per_split,
+                      hipStream_t st )
+{
+  TileOrder ord;
+  ord.row_tiles = (uint32_t)( ( r + TM - 1 ) / TM );
+  ord.token_tiles = (uint32_t)( ( b + TN - 1 ) / TN );
+  ord.gn = std::min<uint32_t>( ord.token_tiles, 8 );
+  ord.gm = std::max<uint32_t>( 1, 64 / ord.gn );
+  const uint32_t rows_per_xcd = ( ord.row_tiles + 7 ) / 8;
+  ord.gm = std::min( ord.gm, rows_per_xcd );
+  const uint32_t patches_m = ( rows_per_xcd + ord.gm - 1 ) / ord.gm;
+  ord.patches_n = ( ord.token_tiles + ord.gn - 1 ) / ord.gn;
+  const uint64_t gx = 8ull * patches_m * ord.patches_n * ord.gm * ord.gn;
+  GH_REQUIRE( gx < ( 1ull << 31 ) && splits <= 65535, "gh_matmul: grid too large" );
+  GH_REQUIRE( partial != nullptr || splits == 1, "gh_matmul: split K needs a partials buffer" );
+  const dim3 grid( (unsigned)gx, 1, splits );
+  if ( partial != nullptr ) {
+    gemm_tile_kernel<true><<<grid, 256, 0, st>>>( xout, partial, x, w, (uint32_t)s, (uint32_t)r, (uint32_t)b, k_per_split, ord );
+  } else {
+    gemm_tile_kernel<false><<<grid, 256, 0, st>>>( xout, partial, x, w, (uint32_t)s, (uint32_t)r, (uint32_t)b, k_per_split, ord );
+  }
   GH_LAUNCH_CHECK();
   return GH_OK;
 }

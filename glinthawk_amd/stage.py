@@ -99,7 +99,10 @@ class Stage:
             self._h = None
 
     def __del__(self):
-        self.close()
+        try:
+            self.close()
+        except Exception:       # interpreter shutdown: module globals may already be gone
+            pass
 
     # ---- weights
     def set_layer_tensor(self, layer: int, name: str, arr: np.ndarray) -> None:
