@@ -8,6 +8,7 @@
 #include <vector>
 
 #include "glint/contextman.hh"
+#include "glint/loader.hh"
 #include "glint/model.hh"
 
 using namespace glint;
@@ -22,6 +23,7 @@ struct StageBase
   virtual ~StageBase() = default;
   virtual void set_layer_tensor( size_t layer, size_t k, const void* host, uint64_t n ) = 0;
   virtual void set_base_tensor( size_t k, const void* host, uint64_t n ) = 0;
+  virtual std::string load_dir( const char* model_dir ) = 0;
   virtual void new_state( uint32_t batch, uint32_t next_layer, int next_stage ) = 0;
   virtual void set_prompt( size_t i, uint32_t context_id, uint32_t token, uint32_t pos, float temp, uint32_t plen, uint32_t mcl ) = 0;
   virtual void discard( size_t i ) = 0;
@@ -58,6 +60,7 @@ struct StageImpl : StageBase
     , contexts( s )
   {
   }
+  std::string load_dir( const char* model_dir ) override { return load_model_dir( model, model_dir ); }
 
   void set_layer_tensor( size_t layer, size_t k, const void* host, uint64_t n ) override
   {
@@ -283,6 +286,8 @@ struct BookManager
 
 using PagedBookContext = glint::DynamicContext<BookConfig, float16_t, CountingRegion>;
 
+thread_local std::string g_last_error;
+
 } // namespace
 
 extern "C" {
@@ -310,6 +315,54 @@ void* glint_stage_create( const char* config, int dtype, uint32_t first_layer, u
 }
 
 void glint_stage_destroy( void* h ) { delete static_cast<StageBase*>( h ); }
+
+// the reference's model directory (CONFIG, BASEWEIGHTS_<DT>, LAYER<i>_<DT>) -> the tensors this stage hosts.
+// 0 on success; otherwise nothing is guaranteed about the weights and glint_last_error() says what was wrong.
+int glint_stage_load( void* h, const char* model_dir )
+{
+  g_last_error = static_cast<StageBase*>( h )->load_dir( model_dir );
+  return g_last_error.empty() ? 0 : -1;
+}
+const char* glint_last_error() { return g_last_error.c_str(); }
+
+// Host-only walk over a model directory for a stage hosting layers [first_layer, first_layer + n_hosted)
+// (flags & 2: the classifier too): checks CONFIG and the size of every file the stage would open, and
+// records each resident tensor as 4 numbers (is_base, layer, k in file order, byte offset in the file)
+// followed by its element count, up to `max_records`.  Returns the number of tensors, or -1 (see glint_last_error()).
+int64_t glint_model_dir_walk( const char* config, int dtype, uint32_t first_layer, uint32_t n_hosted, uint32_t flags, const char* model_dir, uint64_t* records,
+                              uint64_t max_records )
+{
+  const std::string name( config );
+  uint64_t count = 0;
+  auto sink = [&]( bool is_base, size_t layer, size_t k, const auto*, uint64_t n, uint64_t offset ) {
+    if ( count < max_records && records != nullptr ) {
+      uint64_t* r = records + 5 * count;
+      r[0] = is_base ? 1 : 0;
+      r[1] = layer;
+      r[2] = k;
+      r[3] = offset;
+      r[4] = n;
+    }
+    count++;
+  };
+  bool known = false;
+#define GLINT_CASE( NAME, CFG )                                                                                         \
+  if ( name == NAME ) {                                                                                                 \
+    known = true;                                                                                                       \
+    const auto s = StageSettings<configs::CFG>::slice( first_layer, n_hosted, 1, 1, flags & 2u );                        \
+    g_last_error = dtype == 0 ? walk_model_dir<configs::CFG, float16_t>( s, model_dir, sink ) : walk_model_dir<configs::CFG, float32_t>( s, model_dir, sink ); \
+  }
+  GLINT_CASE( "llama2-7b", Llama2_7B_Chat )
+  GLINT_CASE( "stories15m", Stories_15M )
+  GLINT_CASE( "test-gqa4", Test_GQA4 )
+  GLINT_CASE( "test-mha", Test_MHA )
+  GLINT_CASE( "test-tiny", Test_Tiny )
+#undef GLINT_CASE
+  if ( !known ) {
+    g_last_error = "unknown configuration " + name;
+  }
+  return g_last_error.empty() ? (int64_t)count : -1;
+}
 void glint_stage_set_layer_tensor( void* h, uint32_t layer, uint32_t k, const void* host, uint64_t n ) { static_cast<StageBase*>( h )->set_layer_tensor( layer, k, host, n ); }
 void glint_stage_set_base_tensor( void* h, uint32_t k, const void* host, uint64_t n ) { static_cast<StageBase*>( h )->set_base_tensor( k, host, n ); }
 void glint_stage_new_state( void* h, uint32_t batch, uint32_t next_layer, int next_stage ) { static_cast<StageBase*>( h )->new_state( batch, next_layer, next_stage ); }

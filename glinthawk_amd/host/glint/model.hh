@@ -13,6 +13,8 @@
 
 #include <algorithm>
 #include <cmath>
+#include <cstdio>
+#include <filesystem>
 #include <memory>
 #include <vector>
 
@@ -62,6 +64,10 @@ struct WeightLayout
   }
 };
 
+// glint/loader.hh: copies the hosted tensors out of the reference's model directory
+template<typename Model>
+std::string load_model_dir( Model& model, const std::filesystem::path& model_dir );
+
 template<typename DType>
 struct BaseWeights
 {
@@ -97,6 +103,7 @@ struct ModelOptions
   bool allocate_logits { true };  // only needed when the classifier is hosted
   uint64_t seed { 1 };            // random initialisation of weights
   float weight_std { 0.02f };     // N(0, std) for every tensor, as the benchmark configurations say
+  bool randomize { true };        // false: leave the weights for load() / set_*_tensor()
 };
 
 template<typename Config, typename DType, typename LlamaOperations = hip::LlamaOperations<Config, DType>, typename Context = hip::Context<Config, DType>>
@@ -124,8 +131,30 @@ public:
     GLINT_CHECK( settings_.concurrency_limit <= MAX_BATCH_SIZE );
     allocate_weights();
     allocate_scratch();
-    randomize_weights();
+    if ( options_.randomize ) {
+      randomize_weights();
+    }
     write_rope_tables();
+  }
+
+  // The reference's constructor (models/llama2/model.hh:150-270): settings + model directory.  The
+  // CONFIG file must describe Config, every weight file opened must have the size the shape implies;
+  // anything else aborts, as the reference's CHECKs do.  Needs glint/loader.hh at the point of use.
+  Llama2( const std::filesystem::path& model_dir, const SettingsType& settings, ModelOptions options = {} )
+    : Llama2( settings, without_random_weights( options, settings ) )
+  {
+    if ( !settings.randomize_parameters ) {
+      load( model_dir );
+    }
+  }
+
+  void load( const std::filesystem::path& model_dir )
+  {
+    const std::string err = load_model_dir( *this, model_dir );
+    if ( !err.empty() ) {
+      std::fprintf( stderr, "glint: %s\n", err.c_str() );
+      std::abort();
+    }
   }
 
   const SettingsType& settings() const { return settings_; }
@@ -635,6 +664,12 @@ private:
     return p;
   }
   static uint64_t padded( uint64_t n ) { return ( n + 7 ) / 8 * 8; }
+
+  static ModelOptions without_random_weights( ModelOptions o, const SettingsType& s )
+  {
+    o.randomize = s.randomize_parameters;
+    return o;
+  }
 
   void allocate_weights()
   {

@@ -58,6 +58,9 @@ def host_lib() -> C.CDLL:
             "glint_stage_scratch": (vp, [vp, C.c_int]),
             "glint_stage_sync": (None, [vp]),
             "glint_stage_prefill": (C.c_int, [vp, u32, vp, vp, u32, u32, vp, vp, vp, vp]),
+            "glint_stage_load": (C.c_int, [vp, C.c_char_p]),
+            "glint_last_error": (C.c_char_p, []),
+            "glint_model_dir_walk": (C.c_int64, [C.c_char_p, C.c_int, u32, u32, u32, C.c_char_p, vp, C.c_uint64]),
             "glint_book_manager_new": (vp, [u64]),
             "glint_book_manager_delete": (None, [vp]),
             "glint_book_manager_free": (u64, [vp]),
@@ -103,6 +106,12 @@ class Stage:
             self.close()
         except Exception:       # interpreter shutdown: module globals may already be gone
             pass
+
+    def load(self, model_dir: str) -> None:
+        """Copies the tensors this stage hosts out of a model directory in the reference's format
+        (CONFIG, BASEWEIGHTS_<FP16|FP32>, LAYER<i>_<FP16|FP32>)."""
+        if host_lib().glint_stage_load(self._h, os.fsencode(model_dir)) != 0:
+            raise GlintError(host_lib().glint_last_error().decode(errors="replace"))
 
     # ---- weights
     def set_layer_tensor(self, layer: int, name: str, arr: np.ndarray) -> None:
@@ -269,6 +278,24 @@ class BookPagedContext:
         out = (C.c_uint64 * 2)()
         allocated = host_lib().glint_book_paged_prepare(self._c, layer, token_pos, int(can_release), out)
         return int(allocated), int(out[0]), int(out[1])
+
+
+def model_dir_walk(config: str, dtype: str, first_layer: int, n_hosted: int, with_cls: bool, model_dir: str):
+    """Host-only: validates CONFIG and the weight files a stage of layers [first_layer, first_layer +
+    n_hosted) would open, and lists the tensors it would copy as dicts (is_base, layer, tensor name,
+    byte offset in its file, elements).  Raises GlintError with the loader's message on failure."""
+    cap = 1024
+    rec = np.zeros((cap, 5), dtype=np.uint64)
+    n = host_lib().glint_model_dir_walk(config.encode(), 0 if dtype == "f16" else 1, first_layer, n_hosted,
+                                        FLAG_CLS if with_cls else 0, os.fsencode(model_dir), rec.ctypes.data, cap)
+    if n < 0:
+        raise GlintError(host_lib().glint_last_error().decode(errors="replace"))
+    out = []
+    for r in rec[:n]:
+        is_base = bool(r[0])
+        out.append(dict(is_base=is_base, layer=int(r[1]), tensor=(BASE_TENSORS if is_base else LAYER_TENSORS)[int(r[2])],
+                        offset=int(r[3]), elements=int(r[4])))
+    return out
 
 
 def book_head_offset(hosted, layer: int, pos: int, head: int, value: bool) -> Optional[int]:
