@@ -24,6 +24,8 @@ struct StageBase
   virtual void set_layer_tensor( size_t layer, size_t k, const void* host, uint64_t n ) = 0;
   virtual void set_base_tensor( size_t k, const void* host, uint64_t n ) = 0;
   virtual std::string load_dir( const char* model_dir ) = 0;
+  virtual std::string set_state_bytes( const void* bytes, uint64_t len ) = 0;
+  virtual std::string get_state_bytes() = 0;
   virtual void new_state( uint32_t batch, uint32_t next_layer, int next_stage ) = 0;
   virtual void set_prompt( size_t i, uint32_t context_id, uint32_t token, uint32_t pos, float temp, uint32_t plen, uint32_t mcl ) = 0;
   virtual void discard( size_t i ) = 0;
@@ -61,6 +63,22 @@ struct StageImpl : StageBase
   {
   }
   std::string load_dir( const char* model_dir ) override { return load_model_dir( model, model_dir ); }
+  // a state as it arrives from / leaves for the neighbouring stage (models/common/state.hh:512-594)
+  std::string set_state_bytes( const void* bytes, uint64_t len ) override
+  {
+    std::string why;
+    State parsed;
+    if ( !State::parse( std::string_view( static_cast<const char*>( bytes ), len ), parsed, &why ) ) {
+      return why;
+    }
+    if ( parsed.dtype() != dtype_of<DType>() && parsed.next_stage() != InferenceStage::Attention ) {
+      return "state data type does not match the stage";
+    }
+    state = std::move( parsed );
+    held.clear();
+    return {};
+  }
+  std::string get_state_bytes() override { return state.serialize(); }
 
   void set_layer_tensor( size_t layer, size_t k, const void* host, uint64_t n ) override
   {
@@ -287,6 +305,11 @@ struct BookManager
 using PagedBookContext = glint::DynamicContext<BookConfig, float16_t, CountingRegion>;
 
 thread_local std::string g_last_error;
+thread_local std::string g_bytes; // result of the last call that returns bytes
+
+// host-only: states of one fixed shape for the tests of the wire format and of refill / split / merge
+using BookState = BatchedInferenceState<configs::Test_Tiny>;
+BookState* as_state( void* h ) { return static_cast<BookState*>( h ); }
 
 } // namespace
 
@@ -466,6 +489,102 @@ uint64_t glint_book_key_head_offset( const uint8_t* hosted, uint32_t layer, uint
   }
   auto tc = lc.token( pos );
   return static_cast<uint64_t>( ( value ? tc.value_head( head ) : tc.key_head( head ) ) - base );
+}
+
+// ---- stage state on the wire --------------------------------------------------------------------
+int glint_stage_set_state_bytes( void* h, const void* bytes, uint64_t len )
+{
+  g_last_error = static_cast<StageBase*>( h )->set_state_bytes( bytes, len );
+  return g_last_error.empty() ? 0 : -1;
+}
+// the serialized state stays valid until the next call on this thread
+const void* glint_stage_get_state_bytes( void* h, uint64_t* len )
+{
+  g_bytes = static_cast<StageBase*>( h )->get_state_bytes();
+  *len = g_bytes.size();
+  return g_bytes.data();
+}
+
+// ---- host-only states (shape of "test-tiny": dim 32, kv_dim 16) -----------------------------------
+void* glint_state_new( uint32_t batch, int dtype, uint32_t route_id, uint32_t model_id )
+{
+  return new BookState( batch, dtype == 0 ? DataType::Float16 : DataType::Float32, route_id, model_id );
+}
+void* glint_state_parse( const void* bytes, uint64_t len )
+{
+  auto* s = new BookState();
+  if ( !BookState::parse( std::string_view( static_cast<const char*>( bytes ), len ), *s, &g_last_error ) ) {
+    delete s;
+    return nullptr;
+  }
+  return s;
+}
+void glint_state_delete( void* h ) { delete as_state( h ); }
+const void* glint_state_serialize( void* h, uint64_t* len )
+{
+  g_bytes = as_state( h )->serialize();
+  *len = g_bytes.size();
+  return g_bytes.data();
+}
+void glint_state_set_meta( void* h, uint64_t id, uint32_t next_layer, int next_stage, int next_tier, uint32_t next_rank, int is_sharded )
+{
+  auto* s = as_state( h );
+  s->set_id( id );
+  s->set_next_layer( next_layer );
+  s->set_next_stage( static_cast<InferenceStage>( next_stage ) );
+  s->set_next_tier( (int8_t)next_tier );
+  s->set_next_rank( (uint8_t)next_rank );
+  s->set_is_sharded( is_sharded != 0 );
+}
+void glint_state_set_prompt( void* h, uint32_t i, const uint8_t prompt_id[32], uint32_t context_id, uint32_t token, uint32_t token_pos, float temperature,
+                             uint32_t prompt_length, uint32_t max_completion_length, int kv_tier, uint32_t kv_rank )
+{
+  PromptID id;
+  std::memcpy( id.hash.data(), prompt_id, 32 );
+  as_state( h )->set_prompt( i, id, context_id, token, token_pos, temperature, prompt_length, max_completion_length, (int8_t)kv_tier, (uint8_t)kv_rank );
+}
+void glint_state_discard( void* h, uint32_t i ) { as_state( h )->discard( i ); }
+void glint_state_set_finished( void* h, uint32_t i ) { as_state( h )->set_finished( i ); }
+int glint_state_check_finished( void* h, uint32_t i ) { return as_state( h )->check_finished( i ) ? 1 : 0; }
+uint64_t glint_state_free_slots( void* h ) { return as_state( h )->free_slots(); }
+uint32_t glint_state_batch_size( void* h ) { return as_state( h )->batch_size(); }
+int glint_state_all_assigned( void* h ) { return as_state( h )->all_assigned_to_nodes() ? 1 : 0; }
+// which: 0 activations, 1 queries, 2 kvs; allocates when asked to and absent; *bytes = 0 when absent
+void* glint_state_buffer( void* h, int which, uint64_t* bytes, int allocate )
+{
+  auto* s = as_state( h );
+  DataBuffer* b = which == 0 ? &s->activations() : which == 1 ? &s->queries() : &s->kvs();
+  const bool present = which == 0 ? s->has_activations() : which == 1 ? s->has_queries() : s->has_kvs();
+  if ( allocate && !present ) {
+    if ( which == 0 ) {
+      s->allocate_activations();
+    } else if ( which == 1 ) {
+      s->allocate_queries();
+    } else {
+      s->allocate_kvs();
+    }
+  }
+  *bytes = b->len();
+  return b->data();
+}
+int glint_state_replenish_from( void* h, void* other ) { return as_state( h )->replenish_from( *as_state( other ) ) ? 1 : 0; }
+void glint_state_merge( void* h, void* other ) { as_state( h )->merge( std::move( *as_state( other ) ) ); }
+// rows [0, n) and [n, batch) as two new states
+void glint_state_split( void* h, uint64_t n, void** first, void** second )
+{
+  auto [a, b] = as_state( h )->split( n );
+  *first = new BookState( std::move( a ) );
+  *second = new BookState( std::move( b ) );
+}
+// splits `h` (left empty) by kv placement; up to `cap` new states in `out`, returns how many pieces there are
+uint64_t glint_state_split_on_kv( void* h, void** out, uint64_t cap )
+{
+  auto pieces = BookState::split_on_kv( std::move( *as_state( h ) ) );
+  const uint64_t n = pieces.size();
+  for ( uint64_t i = 0; i < n && i < cap; i++ ) {
+    out[i] = new BookState( std::move( pieces[i] ) );
+  }
+  return n;
 }
 
 } // extern "C"

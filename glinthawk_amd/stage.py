@@ -60,6 +60,8 @@ def host_lib() -> C.CDLL:
             "glint_stage_prefill": (C.c_int, [vp, u32, vp, vp, u32, u32, vp, vp, vp, vp]),
             "glint_stage_load": (C.c_int, [vp, C.c_char_p]),
             "glint_last_error": (C.c_char_p, []),
+            "glint_stage_set_state_bytes": (C.c_int, [vp, vp, C.c_uint64]),
+            "glint_stage_get_state_bytes": (vp, [vp, C.POINTER(C.c_uint64)]),
             "glint_model_dir_walk": (C.c_int64, [C.c_char_p, C.c_int, u32, u32, u32, C.c_char_p, vp, C.c_uint64]),
             "glint_book_manager_new": (vp, [u64]),
             "glint_book_manager_delete": (None, [vp]),
@@ -106,6 +108,19 @@ class Stage:
             self.close()
         except Exception:       # interpreter shutdown: module globals may already be gone
             pass
+
+    def set_state_bytes(self, raw: bytes) -> None:
+        """Replaces the stage's batched state by one in the reference's wire format (as it arrives from the
+        previous stage)."""
+        buf = C.create_string_buffer(raw, len(raw))
+        if host_lib().glint_stage_set_state_bytes(self._h, C.cast(buf, C.c_void_p), len(raw)) != 0:
+            raise GlintError(host_lib().glint_last_error().decode(errors="replace"))
+
+    def get_state_bytes(self) -> bytes:
+        """The stage's batched state in the reference's wire format (what the next stage receives)."""
+        n = C.c_uint64(0)
+        p = host_lib().glint_stage_get_state_bytes(self._h, C.byref(n))
+        return C.string_at(p, n.value)
 
     def load(self, model_dir: str) -> None:
         """Copies the tensors this stage hosts out of a model directory in the reference's format
