@@ -53,9 +53,22 @@ def build_host() -> str | None:
     return HOST_LIB
 
 
+def build_tools() -> list[str]:
+    """profile-stage-hip and profile-gemm-hip: the reference's profiling front ends for this target."""
+    built = []
+    for src in sorted(glob.glob(os.path.join(HOST, "bin", "*.cc"))):
+        name = os.path.splitext(os.path.basename(src))[0].replace("_", "-") + "-hip"
+        exe = os.path.join(LIB_DIR, name)
+        _run([HIPCC, *COMMON_FLAGS, "-std=c++20", "-x", "c++", "-I" + HOST, "-o", exe, src,
+              "-L" + LIB_DIR, "-lglint_hip", "-Wl,-rpath,$ORIGIN", "-pthread"])
+        built.append(exe)
+    return built
+
+
 def build_all() -> None:
     build_kernels()
     build_host()
+    build_tools()
 
 
 if __name__ == "__main__":

@@ -6,10 +6,12 @@
 // A null buffer is the *empty* context (make_empty = true): ops skip such rows.
 #pragma once
 
+#include <algorithm>
 #include <array>
 #include <concepts>
 #include <cstddef>
 #include <optional>
+#include <vector>
 
 #include "glint/config.hh"
 
@@ -164,6 +166,7 @@ class DynamicContext : public Context<Config, DType>
 {
   std::optional<VirtualMemoryRegion> storage_ {};
   std::array<size_t, Config::n_layers> layer_allocated_offsets_ {};
+  std::vector<bool> block_committed_ {};
   size_t blocks_committed_ { 0 };
   size_t clears_ { 0 };
 
@@ -189,18 +192,35 @@ public:
     if ( can_release ) {
       storage_->clear();
       layer_allocated_offsets_.fill( 0 );
+      std::fill( block_committed_.begin(), block_committed_.end(), false );
       clears_++;
     }
     const auto layer = this->layer( layer_num );
     if ( layer.empty() ) {
       return true;
     }
+    // Blocks are 2 MiB pieces of the region counted from its base.  Every real shape has layer spans
+    // that are multiples of 2 MiB, so a layer's blocks start at the layer and this is the reference's
+    // rule (one more block whenever the needed length exceeds what the layer has).  Shapes smaller
+    // than that abort in the reference ("Out of bounds allocation"); here the last block is cut at
+    // the end of the region and a block shared by two layers is committed once.
     const size_t needed = ( token_pos + 1 ) * Config::kv_dim * 2 * sizeof( DType );
-    while ( needed > layer_allocated_offsets_[layer_num] ) {
-      const auto* at = reinterpret_cast<const uint8_t*>( layer.data() ) + layer_allocated_offsets_[layer_num];
-      storage_->allocate_span( at, BLOCK_SIZE );
-      layer_allocated_offsets_[layer_num] += BLOCK_SIZE;
-      blocks_committed_++;
+    if ( needed > layer_allocated_offsets_[layer_num] ) {
+      const size_t region_len = storage_->max_len();
+      const size_t layer_off = static_cast<size_t>( reinterpret_cast<const uint8_t*>( layer.data() ) - static_cast<const uint8_t*>( storage_->ptr() ) );
+      const size_t last_block = ( layer_off + needed - 1 ) / BLOCK_SIZE;
+      if ( block_committed_.size() < ( region_len + BLOCK_SIZE - 1 ) / BLOCK_SIZE ) {
+        block_committed_.resize( ( region_len + BLOCK_SIZE - 1 ) / BLOCK_SIZE, false );
+      }
+      for ( size_t b = layer_off / BLOCK_SIZE; b <= last_block; b++ ) {
+        if ( !block_committed_[b] ) {
+          const size_t begin = b * BLOCK_SIZE;
+          storage_->allocate_span( static_cast<const uint8_t*>( storage_->ptr() ) + begin, std::min( BLOCK_SIZE, region_len - begin ) );
+          block_committed_[b] = true;
+          blocks_committed_++;
+        }
+      }
+      layer_allocated_offsets_[layer_num] = std::min( ( last_block + 1 ) * BLOCK_SIZE, region_len ) - layer_off;
     }
     return true;
   }

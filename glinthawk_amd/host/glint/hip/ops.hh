@@ -11,6 +11,7 @@
 
 #include "glint/config.hh"
 #include "glint/context.hh"
+#include "glint/state.hh"
 #include "glint/types.hh"
 #include "glint_hip.h"
 
@@ -50,13 +51,33 @@ struct DeviceDeleter
   }
 };
 
+// From the first Operations object on, the state's host buffers (activations, queries, kvs) are
+// page-locked: their transfers need no staging copy.  Installed once per process.
+inline void use_pinned_state_buffers()
+{
+  static const bool installed = [] {
+    HostBufferPool::instance().set_source(
+      []( size_t n ) -> void* {
+        void* p = nullptr;
+        return gh_host_malloc( &p, n ) == GH_OK ? p : nullptr;
+      },
+      []( void* p ) { (void)gh_host_free( p ); } );
+    return true;
+  }();
+  (void)installed;
+}
+
 template<typename DType>
 class Operations
 {
 public:
   using DeviceUniquePtr = std::unique_ptr<DType, DeviceDeleter<DType>>;
 
-  Operations() { GLINT_GH( gh_init( 0 ) ); }
+  Operations()
+  {
+    GLINT_GH( gh_init( 0 ) );
+    use_pinned_state_buffers();
+  }
   ~Operations() = default;
   Operations( const Operations& ) = delete;
   Operations& operator=( const Operations& ) = delete;

@@ -274,15 +274,18 @@ public:
 
     // the wire dtype may differ from the attention dtype (fp16 activations, fp32 attention)
     import_converted( q_, states.queries().data(), states.queries().len(), states.dtype() );
-    if ( states.has_kvs() ) {
-      for ( size_t i = 0; i < states.batch_size(); i++ ) {
-        if ( states.active( i ) && !token_contexts_[i].empty() ) {
-          import_converted( token_contexts_[i].key(), states.kv( i ), 2 * Config::kv_dim * DataTypeSize( states.dtype() ), states.dtype() );
-        }
-      }
-    }
     if ( options_.fused_attention ) {
       upload_tables( contexts, { static_cast<size_t>( l ) } );
+    }
+    if ( states.has_kvs() ) {
+      // all rows in one transfer, then the append kernel scatters them into the slots (rows of
+      // inactive prompts have no token row and are skipped, like the reference's per-row loop)
+      import_converted( kv_, states.kvs().data(), states.kvs().len(), states.dtype() );
+      if ( options_.fused_attention ) {
+        GLINT_GH( gh_kv_append( token_rows_dev( 0 ), kv_, batch_, Config::kv_dim, hip::gh_type<DType>(), ops_.stream() ) );
+      } else {
+        ops_.copy_kv_cache( token_contexts_, kv_, batch_ );
+      }
     }
     attention_ops( 0 );
 
@@ -486,6 +489,13 @@ private:
   void post_attention_ops( const size_t layer )
   {
     const auto& w = layers_[layer];
+    if ( options_.fused_attention && options_.fused_projections ) {
+      // same three fused launches as in forward(): wo + residual + rmsnorm, w1|w3 + SiLU gate, w2 + residual
+      ops_.template matmul_accum<Config::dim, Config::dim>( x_, xb_, w.wo, batch_, xb_, w.rms_ffn_weight );
+      ops_.matmul_silu_gate( hb_, xb_, w.w1, batch_ );
+      ops_.template matmul_accum<Config::hidden_dim, Config::dim>( x_, hb_, w.w2, batch_, nullptr, nullptr );
+      return;
+    }
     ops_.template matmul<Config::dim, Config::dim>( xb2_, xb_, w.wo, batch_ );
     ops_.template accum<Config::dim>( x_, xb2_, batch_ );
     ops_.template rmsnorm<Config::dim>( xb_, x_, reinterpret_cast<float32_t*>( temp_ ), w.rms_ffn_weight, batch_ );

@@ -23,7 +23,10 @@
 #include <array>
 #include <cstdint>
 #include <cstring>
+#include <cstdlib>
 #include <deque>
+#include <map>
+#include <mutex>
 #include <sstream>
 #include <string>
 #include <string_view>
@@ -81,20 +84,139 @@ struct __attribute__( ( packed ) ) PromptData // models/common/state.hh:36-50
 static_assert( sizeof( StateMetadata ) == 32 );
 static_assert( sizeof( PromptData ) == 57 );
 
-// host buffer with the DataBuffer surface the driver uses (models/types.hh:78-125)
+// Host memory for the state buffers.  Freed buffers are kept by size and handed out again
+// (models/types.hh:58-76 has the same idea): a stage allocates the same few sizes every step.  The
+// memory comes from `malloc` unless a backend installs page-locked allocation with set_source()
+// (the hip target does, once the device is up: the activations then reach the GPU without a
+// staging copy).  Buffers are recycled only while the source that made them is still installed.
+class HostBufferPool
+{
+public:
+  using AllocFn = void* (*)( size_t );
+  using FreeFn = void ( * )( void* );
+
+  static HostBufferPool& instance()
+  {
+    // never destroyed: buffers may be returned during static destruction, and page-locked memory
+    // must not be freed after the device runtime has shut down
+    static HostBufferPool* pool = new HostBufferPool;
+    return *pool;
+  }
+
+  void set_source( AllocFn alloc, FreeFn free )
+  {
+    std::lock_guard<std::mutex> lock( mutex_ );
+    drop_unused();
+    alloc_ = alloc;
+    free_ = free;
+    generation_++;
+  }
+
+  struct Block
+  {
+    uint8_t* ptr { nullptr };
+    FreeFn free { nullptr };
+    uint64_t generation { 0 };
+  };
+
+  Block get( const size_t n )
+  {
+    if ( n == 0 ) {
+      return {};
+    }
+    std::lock_guard<std::mutex> lock( mutex_ );
+    auto it = unused_.find( n );
+    if ( it != unused_.end() && !it->second.empty() ) {
+      Block b = it->second.back();
+      it->second.pop_back();
+      reused_++;
+      return b;
+    }
+    void* p = alloc_( n );
+    if ( p == nullptr ) {
+      fatal( __FILE__, __LINE__, "HostBufferPool: out of host memory" );
+    }
+    return { static_cast<uint8_t*>( p ), free_, generation_ };
+  }
+
+  void put( const Block b, const size_t n )
+  {
+    if ( b.ptr == nullptr ) {
+      return;
+    }
+    std::lock_guard<std::mutex> lock( mutex_ );
+    if ( b.generation == generation_ && n >= MIN_POOLED ) {
+      unused_[n].push_back( b );
+    } else {
+      b.free( b.ptr );
+    }
+  }
+
+  uint64_t reused() const { return reused_; }
+
+private:
+  static constexpr size_t MIN_POOLED = 4096; // smaller buffers are cheap to allocate
+
+  HostBufferPool() = default;
+  void drop_unused()
+  {
+    for ( auto& [n, blocks] : unused_ ) {
+      for ( auto& b : blocks ) {
+        b.free( b.ptr );
+      }
+    }
+    unused_.clear();
+  }
+
+  std::mutex mutex_ {};
+  AllocFn alloc_ { &std::malloc };
+  FreeFn free_ { &std::free };
+  uint64_t generation_ { 0 };
+  std::map<size_t, std::vector<Block>> unused_ {};
+  uint64_t reused_ { 0 };
+};
+
+// host buffer with the DataBuffer surface the driver uses (models/types.hh:78-125); zero-filled when made
 class DataBuffer
 {
-  std::vector<uint8_t> bytes_ {};
+  HostBufferPool::Block block_ {};
+  uint64_t len_ { 0 };
 
 public:
   DataBuffer() = default;
   explicit DataBuffer( size_t n )
-    : bytes_( n )
+    : block_( HostBufferPool::instance().get( n ) )
+    , len_( n )
   {
+    if ( n > 0 ) {
+      std::memset( block_.ptr, 0, n );
+    }
   }
-  uint64_t len() const { return bytes_.size(); }
-  uint8_t* data() { return bytes_.data(); }
-  const uint8_t* data() const { return bytes_.data(); }
+  DataBuffer( const DataBuffer& ) = delete;
+  DataBuffer& operator=( const DataBuffer& ) = delete;
+  DataBuffer( DataBuffer&& other ) noexcept
+    : block_( other.block_ )
+    , len_( other.len_ )
+  {
+    other.block_ = {};
+    other.len_ = 0;
+  }
+  DataBuffer& operator=( DataBuffer&& other ) noexcept
+  {
+    if ( this != &other ) {
+      HostBufferPool::instance().put( block_, len_ );
+      block_ = other.block_;
+      len_ = other.len_;
+      other.block_ = {};
+      other.len_ = 0;
+    }
+    return *this;
+  }
+  ~DataBuffer() { HostBufferPool::instance().put( block_, len_ ); }
+
+  uint64_t len() const { return len_; }
+  uint8_t* data() { return block_.ptr; }
+  const uint8_t* data() const { return block_.ptr; }
 };
 
 template<typename Config>
