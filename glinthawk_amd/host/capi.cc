@@ -4,10 +4,13 @@
 #include <cstring>
 #include <deque>
 #include <memory>
+#include <chrono>
 #include <string>
+#include <thread>
 #include <vector>
 
 #include "glint/contextman.hh"
+#include "glint/kernel.hh"
 #include "glint/loader.hh"
 #include "glint/model.hh"
 
@@ -311,6 +314,106 @@ thread_local std::string g_bytes; // result of the last call that returns bytes
 using BookState = BatchedInferenceState<configs::Test_Tiny>;
 BookState* as_state( void* h ) { return static_cast<BookState*>( h ); }
 
+// ---------------------------------------------------------------------------------------------
+// compute kernel (push / pop / eventfd), type-erased; states cross as wire-format bytes
+// ---------------------------------------------------------------------------------------------
+struct KernelBase
+{
+  virtual ~KernelBase() = default;
+  virtual std::string push_bytes( const void* bytes, uint64_t len ) = 0;
+  virtual bool pop_bytes( std::string& out ) = 0;
+  virtual EventFD& event_fd() = 0;
+  virtual void slot_counts( uint64_t out[3] ) = 0;
+  virtual std::string load_dir( const char* ) { return "this kernel has no weights to load"; }
+};
+
+template<typename Model>
+struct KernelImpl : KernelBase
+{
+  BatchedComputeKernel<Model> kernel;
+  template<typename... Args>
+  explicit KernelImpl( Args&&... args )
+    : kernel( std::forward<Args>( args )... )
+  {
+  }
+  std::string push_bytes( const void* bytes, uint64_t len ) override
+  {
+    typename BatchedComputeKernel<Model>::BatchedState state;
+    std::string why;
+    if ( !BatchedComputeKernel<Model>::BatchedState::parse( std::string_view( static_cast<const char*>( bytes ), len ), state, &why ) ) {
+      return why;
+    }
+    if ( state.batch_size() == 0 || state.batch_size() > kernel.model().settings().concurrency_limit ) {
+      return "batch size outside the kernel's concurrency limit";
+    }
+    kernel.push( std::move( state ) );
+    return {};
+  }
+  bool pop_bytes( std::string& out ) override
+  {
+    typename BatchedComputeKernel<Model>::BatchedState state;
+    if ( !kernel.pop( state ) ) {
+      return false;
+    }
+    out = state.serialize();
+    return true;
+  }
+  EventFD& event_fd() override { return kernel.event_fd(); }
+  void slot_counts( uint64_t out[3] ) override
+  {
+    out[0] = kernel.context_manager().free();
+    out[1] = kernel.context_manager().allocated();
+    out[2] = kernel.context_manager().total();
+  }
+  std::string load_dir( const char* dir ) override
+  {
+    if constexpr ( requires( Model& m ) { m.base_weights(); } ) {
+      return load_model_dir( kernel.model(), dir );
+    } else {
+      return KernelBase::load_dir( dir );
+    }
+  }
+};
+
+// host-only model for the queue tests: no device, forward() advances every active row by one
+// token and takes a data-dependent nap so that the two threads interleave differently every time
+struct EchoContext : glint::Context<configs::Test_Tiny, float16_t>
+{
+  EchoContext() = default;
+  template<typename Settings>
+  explicit EchoContext( const Settings& s, bool make_empty = false )
+  {
+    this->set_buffer( s, make_empty ? nullptr : reinterpret_cast<float16_t*>( uintptr_t { 1 } << 40 ) );
+  }
+};
+struct EchoModel
+{
+  using ConfigType = configs::Test_Tiny;
+  using ContextType = EchoContext;
+  using SettingsType = StageSettings<configs::Test_Tiny>;
+  using StateType = BatchedInferenceState<configs::Test_Tiny>;
+  SettingsType settings_;
+  explicit EchoModel( const SettingsType& s )
+    : settings_( s )
+  {
+  }
+  const SettingsType& settings() const { return settings_; }
+  void forward( StateType& states, const std::vector<std::shared_ptr<EchoContext>>& contexts )
+  {
+    GLINT_CHECK( contexts.size() == states.batch_size() );
+    uint32_t nap = 0;
+    for ( size_t i = 0; i < states.batch_size(); i++ ) {
+      GLINT_CHECK( states.active( i ) != contexts[i]->empty() ); // active rows got a slot, the others the shared empty context
+      if ( states.active( i ) ) {
+        nap += states.token( i );
+        states.set_token( i, states.token( i ) + 1 );
+        states.set_token_pos( i, states.token_pos( i ) + 1 );
+      }
+    }
+    std::this_thread::sleep_for( std::chrono::microseconds( ( nap % 7 ) * 30 ) );
+  }
+};
+
 } // namespace
 
 extern "C" {
@@ -586,5 +689,66 @@ uint64_t glint_state_split_on_kv( void* h, void** out, uint64_t cap )
   }
   return n;
 }
+
+// ---- compute kernel -----------------------------------------------------------------------------
+// same arguments as glint_stage_create; the model sits behind push / pop / eventfd on two threads
+void* glint_kernel_create( const char* config, int dtype, uint32_t first_layer, uint32_t n_hosted, uint32_t concurrency, uint32_t max_contexts, uint32_t flags,
+                           uint64_t seed, float weight_std )
+{
+  const std::string name( config );
+  ModelOptions o;
+  o.fused_attention = flags & 1u;
+  o.fused_projections = !( flags & 8u );
+  o.seed = seed;
+  o.weight_std = weight_std;
+  const bool with_cls = flags & 2u;
+#define GLINT_CASE( NAME, CFG )                                                                                              \
+  if ( name == NAME ) {                                                                                                      \
+    const auto s = StageSettings<configs::CFG>::slice( first_layer, n_hosted, concurrency, max_contexts, with_cls );           \
+    if ( dtype == 0 ) {                                                                                                      \
+      using M = Llama2<configs::CFG, float16_t, hip::LlamaOperations<configs::CFG, float16_t>, hip::Context<configs::CFG, float16_t>>; \
+      return static_cast<KernelBase*>( new KernelImpl<M>( s, o ) );                                                           \
+    }                                                                                                                        \
+    using M = Llama2<configs::CFG, float32_t, hip::LlamaOperations<configs::CFG, float32_t>, hip::Context<configs::CFG, float32_t>>; \
+    return static_cast<KernelBase*>( new KernelImpl<M>( s, o ) );                                                             \
+  }
+  GLINT_CASE( "llama2-70b-4k", Llama2_70B_Chat_4K )
+  GLINT_CASE( "llama2-7b", Llama2_7B_Chat )
+  GLINT_CASE( "stories15m", Stories_15M )
+  GLINT_CASE( "test-gqa4", Test_GQA4 )
+  GLINT_CASE( "test-tiny", Test_Tiny )
+#undef GLINT_CASE
+  return nullptr;
+}
+// host-only kernel around a model that just advances tokens (shape of "test-tiny")
+void* glint_kernel_create_echo( uint32_t concurrency, uint32_t max_contexts )
+{
+  return static_cast<KernelBase*>( new KernelImpl<EchoModel>( StageSettings<configs::Test_Tiny>::slice( 0, 2, concurrency, max_contexts ) ) );
+}
+void glint_kernel_destroy( void* h ) { delete static_cast<KernelBase*>( h ); }
+int glint_kernel_load( void* h, const char* model_dir )
+{
+  g_last_error = static_cast<KernelBase*>( h )->load_dir( model_dir );
+  return g_last_error.empty() ? 0 : -1;
+}
+int glint_kernel_push( void* h, const void* bytes, uint64_t len )
+{
+  g_last_error = static_cast<KernelBase*>( h )->push_bytes( bytes, len );
+  return g_last_error.empty() ? 0 : -1;
+}
+// NULL when nothing has finished; otherwise the serialized state, valid until the next call on this thread
+const void* glint_kernel_pop( void* h, uint64_t* len )
+{
+  if ( !static_cast<KernelBase*>( h )->pop_bytes( g_bytes ) ) {
+    *len = 0;
+    return nullptr;
+  }
+  *len = g_bytes.size();
+  return g_bytes.data();
+}
+int glint_kernel_event_fd( void* h ) { return static_cast<KernelBase*>( h )->event_fd().fd_num(); }
+// 1 and the number of states finished since the last read, or 0 when none
+int glint_kernel_read_event( void* h, uint64_t* count ) { return static_cast<KernelBase*>( h )->event_fd().read_event( count ) ? 1 : 0; }
+void glint_kernel_slot_counts( void* h, uint64_t out[3] ) { static_cast<KernelBase*>( h )->slot_counts( out ); }
 
 } // extern "C"
