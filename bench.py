@@ -44,7 +44,16 @@ WORKLOADS = {
 SHAPES = {
     "llama2-70b-4k": dict(dim=8192, n_heads=64, n_kv_heads=8, hidden_dim=28672, seq_len=4096, n_layers=80),
     "llama2-7b": dict(dim=4096, n_heads=32, n_kv_heads=32, hidden_dim=11008, seq_len=2048, n_layers=32),
+    "llama2-13b-4k": dict(dim=5120, n_heads=40, n_kv_heads=40, hidden_dim=13824, seq_len=4096, n_layers=40),
 }
+# the two remaining one-GPU configurations of BASELINE.json; not the headline, different step definitions
+OTHER_WORKLOADS = {
+    "llama2-13b-prefill-8x2048": "Llama2-13B MHA shape (seq 4096), one stage of 10 layers, fp16: batched prefill of 8 prompts x 2048 "
+                                 "tokens per step, then 64 decode steps",
+    "llama2-70b-churn-256": "Llama2-70B GQA shape, one stage of 10 layers, fp16: 256 context slots with lengths U[16,4096]; every "
+                            "step decodes all slots, then 10 % of them finish and are refilled in place with 128-token prefills",
+}
+MFMA_PEAK_TFLOPS = 2500.0
 
 
 def attention_bytes(shape, batch, keys, elem=2):
@@ -150,6 +159,163 @@ def gpu_bench(workload, steps, warmup):
     return res
 
 
+def layer_matmul_flops(shape, tokens):
+    d, h = shape["dim"], shape["hidden_dim"]
+    kv_dim = d // (shape["n_heads"] // shape["n_kv_heads"])
+    return 2 * tokens * (2 * d * d + 2 * d * kv_dim + 3 * d * h)
+
+
+def prefill_bench(steps, warmup):
+    """BASELINE configuration 3.  One step = one batched prefill of 8 x 2048 prompt tokens through 10 layers
+    (activations in and out over the boundary, like forward()); afterwards 64 decode steps on the same contexts."""
+    import numpy as np
+
+    from glinthawk_amd import ops, stage as S
+
+    name, first, n_hosted, batch, T = "llama2-13b-4k", 10, 10, 8, 2048
+    shape = SHAPES[name]
+    ops.init(0)
+    st = S.Stage(name, "f16", first, n_hosted, batch, batch, seed=3)
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((batch * T, shape["dim"])).astype(np.float16)
+    ids = [100 + i for i in range(batch)]
+
+    def one_step():
+        res = st.prefill(ids, [0] * batch, T, first, activations=x)
+        assert res is not None
+        return res[0]
+
+    for _ in range(warmup):
+        one_step()
+    ops.sync()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        out = one_step()
+    ops.sync()
+    t1 = time.perf_counter()
+    assert np.isfinite(out.astype(np.float32)).all()
+    ms = (t1 - t0) * 1e3 / steps
+    decode_steps = 64
+    acts = x[:batch].copy()
+    t0 = time.perf_counter()
+    for k in range(decode_steps):
+        st.new_state(batch, next_layer=first)
+        for i in range(batch):
+            st.set_prompt(i, ids[i], 1, T + k)
+        st.activations(allocate=True)[:] = acts.reshape(-1)
+        assert st.forward()
+    ops.sync()
+    t1 = time.perf_counter()
+    decode_ms = (t1 - t0) * 1e3 / decode_steps
+    flops = n_hosted * (layer_matmul_flops(shape, batch * T) + batch * 4 * shape["dim"] * T * (T + 1) // 2)
+    dev = ops.device_name()
+    st.close()
+    return {
+        "metric": "prefill prompt tokens/s (+ decode ms/step), Llama2-13B shape, 8 x 2048 tokens, 10 layers",
+        "value": round(batch * T / (ms * 1e-3), 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": round(ms, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": "llama2-13b-prefill-8x2048", "description": OTHER_WORKLOADS["llama2-13b-prefill-8x2048"], "device": dev},
+        "decode_ms_per_step": round(decode_ms, 3), "decode_tokens_per_s": round(batch / (decode_ms * 1e-3), 1),
+        "roofline": {"bound": "mfma", "achieved": round(flops / (ms * 1e-3) / 1e12, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(flops / (ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4), "traffic": None,
+                     "kernel": "whole prefill pass incl. host transfers (projection GEMMs + causal attention flops / step time)",
+                     "algorithmic_flops_per_step": flops},
+        "cpu_baseline": None,
+    }
+
+
+def churn_bench(steps, warmup):
+    """BASELINE configuration 5.  One step = decode of all 256 slots (ragged lengths), then the slots drawn
+    to finish (10 %, seeded) restart in place: a 128-token batched prefill into the same slot."""
+    import numpy as np
+
+    from glinthawk_amd import _lib, ops, stage as S
+
+    name, first, n_hosted, slots, refill = "llama2-70b-4k", 10, 10, 256, 128
+    shape = SHAPES[name]
+    ops.init(0)
+    L = _lib.lib()
+    st = S.Stage(name, "f16", first, n_hosted, slots, slots, seed=5)
+    rng = np.random.default_rng(5)
+    pos = rng.integers(16, 4096, slots)
+    ids = [1000 + i for i in range(slots)]
+    st.new_state(slots, next_layer=first)
+    for i in range(slots):
+        st.set_prompt(i, ids[i], 1, int(pos[i]))
+    assert st.acquire_contexts()
+    kv_dim = shape["dim"] // (shape["n_heads"] // shape["n_kv_heads"])
+    for i in range(slots):
+        for l in range(first, first + n_hosted):
+            _lib.check(L.gh_fill_normal(st.context_layer_ptr(i, l), shape["seq_len"] * 2 * kv_dim, 0.0, 1.0, 7 + i * 131 + l, _lib.GH_F16, None))
+    slot_of = [st.context_slot(i) for i in range(slots)]
+    acts = rng.standard_normal((slots, shape["dim"])).astype(np.float16)
+    prompt = rng.standard_normal((slots * refill, shape["dim"])).astype(np.float16)
+    decoded = prefilled = restarts = 0
+    keys_read = 0
+    t_decode = t_prefill = 0.0
+
+    def one_step(count):
+        nonlocal decoded, prefilled, restarts, keys_read, t_decode, t_prefill
+        t0 = time.perf_counter()
+        st.new_state(slots, next_layer=first)
+        for i in range(slots):
+            st.set_prompt(i, ids[i], 1, int(pos[i]))
+        st.activations(allocate=True)[:] = acts.reshape(-1)
+        assert st.forward()
+        t1 = time.perf_counter()
+        assert [st.context_slot(i) for i in (0, slots // 2, slots - 1)] == [slot_of[0], slot_of[slots // 2], slot_of[slots - 1]]
+        if count:
+            decoded += slots
+            keys_read += int((pos + 1).sum())
+            t_decode += t1 - t0
+        pos[:] = pos + 1
+        done = (rng.random(slots) < 0.10) | (pos >= shape["seq_len"] - 1)
+        gone = np.nonzero(done)[0]
+        if len(gone):
+            t0 = time.perf_counter()
+            res = st.prefill([ids[i] for i in gone], [0] * len(gone), refill, first, activations=prompt[:len(gone) * refill],
+                             want_activations=False)
+            assert res is not None
+            st.sync()
+            t1 = time.perf_counter()
+            pos[gone] = refill
+            if count:
+                prefilled += len(gone) * refill
+                restarts += len(gone)
+                t_prefill += t1 - t0
+
+    for _ in range(warmup):
+        one_step(False)
+    ops.sync()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        one_step(True)
+    ops.sync()
+    t1 = time.perf_counter()
+    counts = st.slot_counts()
+    assert counts == dict(free=0, allocated=slots, total=slots), counts
+    ms = (t1 - t0) * 1e3 / steps
+    dev = ops.device_name()
+    st.close()
+    kv_bytes = keys_read * 2 * kv_dim * 2 * n_hosted
+    return {
+        "metric": "tokens/s (decode + refill prefill), ragged slot churn, Llama2-70B GQA shape, 256 slots, 10 layers",
+        "value": round((decoded + prefilled) / (t1 - t0), 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": round(ms, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": "llama2-70b-churn-256", "description": OTHER_WORKLOADS["llama2-70b-churn-256"], "device": dev},
+        "decode_tokens_per_s": round(decoded / t_decode, 1), "decode_ms_per_step": round(t_decode * 1e3 / steps, 3),
+        "prefill_tokens_per_s": round(prefilled / max(t_prefill, 1e-9), 1), "prefill_ms_per_step": round(t_prefill * 1e3 / steps, 3),
+        "restarts": restarts, "mean_keys_per_slot": round(keys_read / max(decoded, 1), 1),
+        "roofline": {"bound": "hbm", "achieved": round((kv_bytes + steps * n_hosted * layer_weight_bytes(shape)) / t_decode / 1e9, 1),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round((kv_bytes + steps * n_hosted * layer_weight_bytes(shape)) / t_decode / 1e9 / HBM_PEAK_GBPS, 4),
+                     "traffic": None, "kernel": "whole decode step (cached K/V read once + weights once) / decode time"},
+        "cpu_baseline": None,
+    }
+
+
 def cpu_baseline(workload):
     """The oracle (port of the reference's fp32 amd64/OpenMP path) on ONE layer of the workload,
     fp32 weights and fp32 K/V like the reference's CPU build, median of 3 after one warm-up; the
@@ -214,7 +380,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="llama2-70b-gqa-b64-ctx4096", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="llama2-70b-gqa-b64-ctx4096", choices=sorted(WORKLOADS) + sorted(OTHER_WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="also run a plain D2D copy of this many MiB (reference point for profiler byte counters)")
@@ -229,6 +395,12 @@ def main():
         from glinthawk_amd import ops
         ops.init(0)
         calibration_copy(args.calibration_copy_mib << 20)
+    if args.workload == "llama2-13b-prefill-8x2048":
+        print(json.dumps(prefill_bench(args.steps, args.warmup)))
+        return
+    if args.workload == "llama2-70b-churn-256":
+        print(json.dumps(churn_bench(args.steps, args.warmup)))
+        return
     g = gpu_bench(args.workload, args.steps, args.warmup)
     cfg_name, first, n_hosted, batch, keys, desc = WORKLOADS[args.workload]
 

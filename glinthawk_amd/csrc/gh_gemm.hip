@@ -21,6 +21,9 @@ void gemm_stream_plan( uint64_t s, uint64_t r, uint64_t b, uint32_t* splits_out,
 int gemm_stream_launch( __half* xout, float* partial, const __half* x, const __half* w, uint64_t s, uint64_t r, uint64_t b, uint32_t splits,
                         uint32_t k_per_split, bool write_partials, hipStream_t st );
 void gemm_stream_tuning( int target_wgs, int depth );
+// 256 x 256 tile kernel for products with enough tiles (gh_gemm_tile256.hip)
+bool gemm_tile256_applicable( uint64_t s, uint64_t r, uint64_t b, const void* x, const void* w, const void* xout );
+int gemm_tile256_launch( __half* xout, float* partial, const __half* x, const __half* w, uint64_t s, uint64_t r, uint64_t b, hipStream_t st );
 // large-batch (prefill) kernel (gh_gemm_tile.hip)
 bool gemm_tile_applicable( uint64_t s, uint64_t r, uint64_t b, const void* x, const void* w, const void* xout );
 void gemm_tile_plan( uint64_t s, uint64_t r, uint64_t b, uint32_t* splits_out, uint32_t* k_per_split_out );
@@ -254,6 +257,18 @@ int gemm_partials( void* xout, const void* x, const void* w, uint64_t s, uint64_
   GH_REQUIRE( dt == GH_F16, "gh_matmul: unsupported dtype %d", (int)dt );
 
   // many tokens at once (prefill): the MFMA-bound tile kernel; few (decode): the weight-streaming one
+  if ( ( g_force_kernel == 0 || g_force_kernel == 4 ) && gemm_tile256_applicable( s, r, b, x, w, xout ? xout : x ) ) {
+    float* ws = nullptr;
+    if ( want_partials ) {
+      if ( int rc = ensure_workspace( b * r * sizeof( float ), &ws ) ) {
+        return rc;
+      }
+      *partial_out = ws;
+      *splits_out = 1;
+    }
+    return gemm_tile256_launch( static_cast<__half*>( xout ), ws, static_cast<const __half*>( x ), static_cast<const __half*>( w ), s, r, b, st );
+  }
+  GH_REQUIRE( g_force_kernel != 4, "gh_matmul: the 256 x 256 tile kernel needs b >= 192, at least 192 tiles (1024 when s < 8192), s %% 64 == 0 and 16-byte aligned operands" );
   if ( ( g_force_kernel == 0 || g_force_kernel == 3 ) && gemm_tile_applicable( s, r, b, x, w, xout ? xout : x ) ) {
     uint32_t splits = 1, k_per_split = 0;
     gemm_tile_plan( s, r, b, &splits, &k_per_split );

@@ -160,6 +160,42 @@ def test_matmul_many_rows(dt, b, s, r):
     assert_close(got, want, what=f"matmul {dt} {b}x{s}x{r}")
 
 
+# enough 256 x 256 tiles for the second tile kernel (forced, and whatever the dispatcher picks), ragged edges
+@pytest.mark.parametrize("force", [4, 0])
+@pytest.mark.parametrize("b,s,r", [(3000, 8192, 4100), (8200, 128, 8190), (700, 8256, 18000)])
+def test_matmul_256_tiles(force, b, s, r):
+    from glinthawk_amd import _lib
+    rng = np.random.default_rng(26)
+    x = rng.standard_normal((b, s)).astype(np.float16)
+    w = (rng.standard_normal((r, s)) / np.sqrt(s)).astype(np.float16)
+    _lib.lib().gh_gemm_set_tuning(force, 0, 0)
+    try:
+        got = ops.matmul(torch.from_numpy(x).cuda(), torch.from_numpy(w).cuda())
+    finally:
+        _lib.lib().gh_gemm_set_tuning(0, 0, 0)
+    want = (torch.from_numpy(x).cuda().float() @ torch.from_numpy(w).cuda().float().t())
+    err = (got.float() - want).abs()
+    assert got.shape == (b, r) and err.max().item() < 2e-2 and (err.mean() / want.abs().mean()).item() < 1e-3
+    # a strip against the CPU oracle as well
+    want_cpu = O.matmul(x[:8].astype(np.float32), w.astype(np.float32))
+    assert_close(got[:8].cpu().numpy(), want_cpu, what=f"matmul 256-tile {b}x{s}x{r}")
+
+
+def test_matmul_256_tile_one_hot_layout():
+    from glinthawk_amd import _lib
+    s, r, b = 8192, 12544, 1030            # 49 x 5 = 245 tiles, ragged in both directions
+    w = torch.arange(r * s, dtype=torch.float32, device="cuda").reshape(r, s).remainder(1000).half()
+    x = torch.zeros((b, s), dtype=torch.float16, device="cuda")
+    cols = [(7919 * i + 3) % s for i in range(b)]
+    x[torch.arange(b), torch.tensor(cols)] = 1
+    _lib.lib().gh_gemm_set_tuning(4, 0, 0)
+    try:
+        got = ops.matmul(x, w)
+    finally:
+        _lib.lib().gh_gemm_set_tuning(0, 0, 0)
+    assert torch.equal(got, w[:, cols].t().contiguous())
+
+
 def test_matmul_many_rows_layout_one_hot():
     # x rows that select single columns of w: the tile kernel must return them bit for bit
     s, r, b = 320, 200, 260
