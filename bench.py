@@ -382,6 +382,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="llama2-70b-gqa-b64-ctx4096", choices=sorted(WORKLOADS) + sorted(OTHER_WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--attn-variant", default="auto", choices=["auto", "generic", "valu", "mfma"],
+                    help="decode attention kernel the stage uses (measurement of the alternatives; auto = the library's choice)")
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="also run a plain D2D copy of this many MiB (reference point for profiler byte counters)")
     args = ap.parse_args()
@@ -395,6 +397,10 @@ def main():
         from glinthawk_amd import ops
         ops.init(0)
         calibration_copy(args.calibration_copy_mib << 20)
+    if args.attn_variant != "auto":
+        from glinthawk_amd import _lib, ops
+        ops.init(0)
+        _lib.check(_lib.lib().gh_attn_set_auto_variant({"generic": 1, "valu": 2, "mfma": 3}[args.attn_variant]))
     if args.workload == "llama2-13b-prefill-8x2048":
         print(json.dumps(prefill_bench(args.steps, args.warmup)))
         return
@@ -428,7 +434,8 @@ def main():
         "dtype": "f16",
         "data": "synthetic",
         "config": {"workload": args.workload, "description": desc, "stage_config": cfg_name, "first_layer": first,
-                   "hosted_layers": n_hosted, "batch": batch, "keys_per_context": keys, "device": g["device"]},
+                   "hosted_layers": n_hosted, "batch": batch, "keys_per_context": keys, "device": g["device"],
+                   "attn_variant": args.attn_variant},
         "attn_op_ms": round(attn_op_ms, 5),
         "attn_kernel_ms": round(g["attn_kernel_ms"], 5),
         "attn_merge_ms": round(g["attn_merge_ms"], 5),

@@ -102,6 +102,7 @@ SIGNATURES = {
     "gh_attn_pv": (_i, [_vp, _vp, _vp, _u64, _vp, _shp, _i, _vp]),
     "gh_attn_pv_host": (_i, [_vp, _vp, _vp, _u64, _vp, _shp, _i, _vp]),
     "gh_attn_set_chunk": (_i, [_u32]),
+    "gh_attn_set_auto_variant": (_i, [_i]),
     "gh_attn_decode_workspace": (_u64, [_u64, _u32, _shp]),
     "gh_attn_decode": (_i, [_vp, _vp, _vp, _vp, _u64, _u32, _shp, _i, _vp, _u64, _i, _vp]),
     "gh_attn_decode_host": (_i, [_vp, _vp, _vp, _vp, _u64, _shp, _i, _vp, _u64, _i, _vp]),

@@ -30,6 +30,7 @@ constexpr float LOG2E = 1.4426950408889634f;
 constexpr int HS = 128; // head size of the fast kernels
 
 uint32_t g_chunk_override = 0;
+int g_auto_variant = GH_ATTN_AUTO; // what GH_ATTN_AUTO resolves to when the shape allows it (gh_attn_set_auto_variant)
 
 typedef _Float16 f16x4 __attribute__( ( ext_vector_type( 4 ) ) );
 typedef _Float16 f16x8 __attribute__( ( ext_vector_type( 8 ) ) );
@@ -665,7 +666,13 @@ Plan make_plan( uint64_t batch, uint32_t max_pos, const gh_shape* s, gh_dtype dt
 {
   Plan p;
   p.variant = variant;
-  if ( variant == GH_ATTN_AUTO ) {
+  if ( variant == GH_ATTN_AUTO && g_auto_variant == GH_ATTN_GENERIC ) {
+    p.variant = GH_ATTN_GENERIC;
+  } else if ( variant == GH_ATTN_AUTO && g_auto_variant == GH_ATTN_VALU && fast_ok( s, dt ) && valu_gqa_ok( s->gqa_size ) ) {
+    p.variant = GH_ATTN_VALU;
+  } else if ( variant == GH_ATTN_AUTO && g_auto_variant == GH_ATTN_MFMA && fast_ok( s, dt ) && mfma_gqa_ok( s->gqa_size ) ) {
+    p.variant = GH_ATTN_MFMA;
+  } else if ( variant == GH_ATTN_AUTO ) {
     if ( fast_ok( s, dt ) && mfma_gqa_ok( s->gqa_size ) && s->gqa_size >= 4 ) {
       p.variant = GH_ATTN_MFMA;
     } else if ( fast_ok( s, dt ) && valu_gqa_ok( s->gqa_size ) ) {
@@ -729,6 +736,13 @@ void launch_mfma( dim3 grid, hipStream_t st, const void* q, const void* const* r
 using namespace gh;
 
 extern "C" {
+
+int gh_attn_set_auto_variant( int variant )
+{
+  GH_REQUIRE( variant >= GH_ATTN_AUTO && variant <= GH_ATTN_MFMA, "gh_attn_set_auto_variant: unknown variant %d", variant );
+  g_auto_variant = variant;
+  return GH_OK;
+}
 
 int gh_attn_set_chunk( uint32_t tokens_per_split )
 {

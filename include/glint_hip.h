@@ -203,6 +203,8 @@ typedef enum gh_attn_variant
 
 /* tokens per split of the fused kernel; 0 (default) lets the library choose from the batch shape */
 int gh_attn_set_chunk( uint32_t tokens_per_split );
+/* measurement hook: which kernel GH_ATTN_AUTO picks where the shape permits it (GH_ATTN_AUTO restores the library's choice) */
+int gh_attn_set_auto_variant( int variant );
 uint64_t gh_attn_decode_workspace( uint64_t batch, uint32_t max_pos, const gh_shape* shape );
 int gh_attn_decode( const void* q, const void* const* layer_rows_dev, const uint32_t* pos_dev, void* xb, uint64_t batch,
                     uint32_t max_pos, const gh_shape* shape, gh_dtype dt, void* workspace, uint64_t workspace_bytes,
