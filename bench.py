@@ -177,11 +177,14 @@ def prefill_bench(steps, warmup):
     ops.init(0)
     st = S.Stage(name, "f16", first, n_hosted, batch, batch, seed=3)
     rng = np.random.default_rng(3)
-    x = rng.standard_normal((batch * T, shape["dim"])).astype(np.float16)
+    # the boundary's host buffers, page-locked like the states' own buffers
+    x = ops.pinned_empty((batch * T, shape["dim"]), np.float16)
+    x[:] = rng.standard_normal(x.shape).astype(np.float16)
+    y = ops.pinned_empty((batch * T, shape["dim"]), np.float16)
     ids = [100 + i for i in range(batch)]
 
     def one_step():
-        res = st.prefill(ids, [0] * batch, T, first, activations=x)
+        res = st.prefill(ids, [0] * batch, T, first, activations=x, out=y)
         assert res is not None
         return res[0]
 
@@ -250,7 +253,8 @@ def churn_bench(steps, warmup):
             _lib.check(L.gh_fill_normal(st.context_layer_ptr(i, l), shape["seq_len"] * 2 * kv_dim, 0.0, 1.0, 7 + i * 131 + l, _lib.GH_F16, None))
     slot_of = [st.context_slot(i) for i in range(slots)]
     acts = rng.standard_normal((slots, shape["dim"])).astype(np.float16)
-    prompt = rng.standard_normal((slots * refill, shape["dim"])).astype(np.float16)
+    prompt = ops.pinned_empty((slots * refill, shape["dim"]), np.float16)
+    prompt[:] = rng.standard_normal(prompt.shape).astype(np.float16)
     decoded = prefilled = restarts = 0
     keys_read = 0
     t_decode = t_prefill = 0.0

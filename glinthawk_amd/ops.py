@@ -257,5 +257,23 @@ def attn_set_chunk(tokens: int) -> None:
     check(lib().gh_attn_set_chunk(tokens), "gh_attn_set_chunk")
 
 
+def pinned_empty(shape, dtype):
+    """A numpy array in page-locked host memory (gh_host_malloc): transfers to and from the device need
+    no staging copy.  The memory is released when the array and every view of it are gone."""
+    import ctypes as C
+    import weakref
+
+    import numpy as np
+
+    dt = np.dtype(dtype)
+    n = int(np.prod(shape)) * dt.itemsize
+    ptr = C.c_void_p()
+    check(lib().gh_host_malloc(C.byref(ptr), max(n, 1)), "gh_host_malloc")
+    buf = (C.c_uint8 * max(n, 1)).from_address(ptr.value)
+    arr = np.frombuffer(buf, dtype=dt, count=int(np.prod(shape))).reshape(shape)
+    weakref.finalize(buf, lambda p=ptr.value: lib().gh_host_free(C.c_void_p(p)))
+    return arr
+
+
 def sync() -> None:
     check(lib().gh_sync(None), "gh_sync")

@@ -218,14 +218,14 @@ class Stage:
         host_lib().glint_stage_sync(self._h)
 
     def prefill(self, context_ids, start_pos, n_tokens: int, first_layer: int = 0, token_ids=None, activations=None,
-                want_activations: bool = True, want_next_tokens: bool = False):
+                want_activations: bool = True, want_next_tokens: bool = False, out=None):
         """Batched prefill of `n_tokens` tokens per context.  Returns (activations_out or None,
         next_tokens or None); None overall when the contexts could not be served."""
         batch = len(context_ids)
         ids = np.ascontiguousarray(np.asarray(context_ids, dtype=np.uint32))
         start = np.ascontiguousarray(np.asarray(start_pos, dtype=np.uint32))
         toks = None if token_ids is None else np.ascontiguousarray(np.asarray(token_ids, dtype=np.uint32).reshape(-1))
-        acts = None if activations is None else np.ascontiguousarray(activations, dtype=self.np_dtype)
+        acts = None if activations is None else np.ascontiguousarray(activations, dtype=self.np_dtype)   # no copy when already so
         if toks is not None:
             assert toks.size == batch * n_tokens
         dim = None if acts is None else acts.reshape(batch * n_tokens, -1).shape[1]
@@ -233,7 +233,9 @@ class Stage:
         if want_activations:
             if dim is None:
                 raise ValueError("pass dim via activations or call with want_activations=False")
-            out = np.empty((batch * n_tokens, dim), dtype=self.np_dtype)
+            if out is None:
+                out = np.empty((batch * n_tokens, dim), dtype=self.np_dtype)
+            assert out.dtype == self.np_dtype and out.size == batch * n_tokens * dim and out.flags["C_CONTIGUOUS"]
         nxt = np.zeros(batch, dtype=np.uint32) if want_next_tokens else None
         rc = host_lib().glint_stage_prefill(self._h, batch, ids.ctypes.data, start.ctypes.data, n_tokens, first_layer,
                                             None if toks is None else toks.ctypes.data,

@@ -18,7 +18,9 @@ def _init():
 
 
 @pytest.mark.parametrize("dt", [torch.float16, torch.float32])
-@pytest.mark.parametrize("b,s,r", [(4, 288, 288), (64, 1024, 512), (5, 768, 1000), (3, 100, 36)])
+@pytest.mark.parametrize("b,s,r", [(4, 288, 288), (64, 1024, 512), (5, 768, 1000), (3, 100, 36),
+                                   # more rows than one streaming slab: the tile kernels write the partials
+                                   (100, 512, 260), (256, 1024, 512), (300, 4096, 1000), (768, 8192, 16384)])
 def test_matmul_accum_and_norm(dt, b, s, r):
     g = torch.Generator(device="cuda").manual_seed(1)
     x = torch.randn((b, s), generator=g, device="cuda").to(dt)
@@ -45,7 +47,7 @@ def test_matmul_accum_and_norm(dt, b, s, r):
 
 
 @pytest.mark.parametrize("dt", [torch.float16, torch.float32])
-@pytest.mark.parametrize("b,s,hidden", [(4, 288, 768), (64, 512, 1536), (3, 100, 50)])
+@pytest.mark.parametrize("b,s,hidden", [(4, 288, 768), (64, 512, 1536), (3, 100, 50), (130, 512, 1536), (512, 8192, 12544)])
 def test_matmul_silu_gate(dt, b, s, hidden):
     g = torch.Generator(device="cuda").manual_seed(2)
     x = torch.randn((b, s), generator=g, device="cuda").to(dt)
