@@ -33,7 +33,7 @@ HBM_PEAK_GBPS = 8000.0
 # scaled by what it reads for a 1 GiB copy).  Only valid for the workload it was measured on.
 MEASURED_TRAFFIC = {"llama2-70b-gqa-b64-ctx4096": 1086918181}
 
-# the configurations of BASELINE.json that fit one GPU as a single stage
+# the decode configurations that fit one GPU as a single stage (the first is the headline)
 WORKLOADS = {
     # name: (stage config, first layer, hosted layers, batch, keys attended, description)
     "llama2-70b-gqa-b64-ctx4096": ("llama2-70b-4k", 10, 10, 64, 4096,
@@ -46,7 +46,7 @@ SHAPES = {
     "llama2-7b": dict(dim=4096, n_heads=32, n_kv_heads=32, hidden_dim=11008, seq_len=2048, n_layers=32),
     "llama2-13b-4k": dict(dim=5120, n_heads=40, n_kv_heads=40, hidden_dim=13824, seq_len=4096, n_layers=40),
 }
-# the two remaining one-GPU configurations of BASELINE.json; not the headline, different step definitions
+# the prefill-heavy and the slot-churn configuration: not the headline, different step definitions
 OTHER_WORKLOADS = {
     "llama2-13b-prefill-8x2048": "Llama2-13B MHA shape (seq 4096), one stage of 10 layers, fp16: batched prefill of 8 prompts x 2048 "
                                  "tokens per step, then 64 decode steps",
@@ -166,7 +166,7 @@ def layer_matmul_flops(shape, tokens):
 
 
 def prefill_bench(steps, warmup):
-    """BASELINE configuration 3.  One step = one batched prefill of 8 x 2048 prompt tokens through 10 layers
+    """The prefill-heavy configuration.  One step = one batched prefill of 8 x 2048 prompt tokens through 10 layers
     (activations in and out over the boundary, like forward()); afterwards 64 decode steps on the same contexts."""
     import numpy as np
 
@@ -229,7 +229,7 @@ def prefill_bench(steps, warmup):
 
 
 def churn_bench(steps, warmup):
-    """BASELINE configuration 5.  One step = decode of all 256 slots (ragged lengths), then the slots drawn
+    """The slot-churn configuration.  One step = decode of all 256 slots (ragged lengths), then the slots drawn
     to finish (10 %, seeded) restart in place: a 128-token batched prefill into the same slot."""
     import numpy as np
 
@@ -394,7 +394,7 @@ def main():
 
     if args.gpus != 1:
         print("bench.py: this build runs one pipeline stage on ONE GPU; --gpus must be 1 "
-              "(the path shards by context with no collective, see DESIGN.md)", file=sys.stderr)
+              "(the path shards by context, slot -> GPU, with no collective; only the one-GPU share is built)", file=sys.stderr)
         sys.exit(2)
 
     if args.calibration_copy_mib > 0:
