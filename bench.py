@@ -139,6 +139,21 @@ def gpu_bench(workload, steps, warmup):
     out = st.activations().astype(np.float32)
     assert np.all(np.isfinite(out)), "stage output is not finite"
 
+    # what a plain device-to-device copy reaches on this box (bytes read + bytes written per second):
+    # the practical ceiling beside the published peak
+    src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").zero_()
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(10):
+        dst.copy_(src)
+    e1.record()
+    torch.cuda.synchronize()
+    copy_gbps = 10 * 2 * src.numel() / (e0.elapsed_time(e1) * 1e-3) / 1e9
+    del src, dst
+
     ms_per_step = (t1 - t0) * 1e3 / steps
     launches = max(1, n.value)
     kernel_ms = k_ms.value / launches
@@ -154,6 +169,7 @@ def gpu_bench(workload, steps, warmup):
         stage_bytes=stage_bytes,
         batch=batch,
         device=ops.device_name(),
+        copy_gbps=copy_gbps,
     )
     st.close()
     return res
@@ -425,6 +441,8 @@ def main():
         "value": round(value, 1),
         "unit": "GB/s",
         "pct_of_peak": round(100 * value / HBM_PEAK_GBPS, 2),
+        "copy_ceiling_gbps": round(g["copy_gbps"], 1),
+        "pct_of_copy_ceiling": round(100 * value / g["copy_gbps"], 2),
         "stage_tokens_per_s": round(tokens_per_s, 1),
         "stage_roofline_frac": round(stage_roofline_ms / g["ms_per_step"], 4),
         "stage_bytes_per_step": g["stage_bytes"],
