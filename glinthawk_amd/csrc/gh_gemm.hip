@@ -21,6 +21,8 @@ void gemm_stream_plan( uint64_t s, uint64_t r, uint64_t b, uint32_t* splits_out,
 int gemm_stream_launch( __half* xout, float* partial, const __half* x, const __half* w, uint64_t s, uint64_t r, uint64_t b, uint32_t splits,
                         uint32_t k_per_split, bool write_partials, hipStream_t st );
 void gemm_stream_tuning( int target_wgs, int depth );
+bool gemm_stream_gate_applicable( uint64_t s, uint64_t hidden, uint64_t b, const void* x, const void* w13, const void* hb );
+int gemm_stream_gate_launch( __half* hb, const __half* x, const __half* w13, uint64_t s, uint64_t hidden, uint64_t b, hipStream_t st );
 // 256 x 256 tile kernel for products with enough tiles (gh_gemm_tile256.hip)
 bool gemm_tile256_applicable( uint64_t s, uint64_t r, uint64_t b, const void* x, const void* w, const void* xout );
 int gemm_tile256_launch( __half* xout, float* partial, const __half* x, const __half* w, uint64_t s, uint64_t r, uint64_t b, hipStream_t st );
@@ -235,6 +237,18 @@ namespace gh {
 // Runs the GEMM proper.  With `want_partials` the result is always left as fp32 partial sums
 // `[splits][b][r]` in the library's workspace (*partial_out, *splits_out) for a fused epilogue;
 // otherwise the kernel may store DType results straight into `xout` (*splits_out == 0 then).
+// w1, w3 and the SiLU gate in one launch of the streaming kernel, where gemm_partials() would pick that
+// kernel without a K split.  *done = false: nothing was launched, the caller takes the two-kernel route.
+int gemm_gate_one_launch( void* hb, const void* x, const void* w13, uint64_t s, uint64_t hidden, uint64_t b, gh_dtype dt, hipStream_t st, bool* done )
+{
+  *done = false;
+  if ( dt != GH_F16 || ( g_force_kernel != 0 && g_force_kernel != 2 ) || b > 64 || !gemm_stream_gate_applicable( s, hidden, b, x, w13, hb ) ) {
+    return GH_OK;
+  }
+  *done = true;
+  return gemm_stream_gate_launch( static_cast<__half*>( hb ), static_cast<const __half*>( x ), static_cast<const __half*>( w13 ), s, hidden, b, st );
+}
+
 int gemm_partials( void* xout, const void* x, const void* w, uint64_t s, uint64_t r, uint64_t b, gh_dtype dt, hipStream_t st, bool want_partials,
                    float** partial_out, uint32_t* splits_out )
 {

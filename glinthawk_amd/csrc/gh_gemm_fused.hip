@@ -9,6 +9,7 @@ namespace gh {
 
 int gemm_partials( void* xout, const void* x, const void* w, uint64_t s, uint64_t r, uint64_t b, gh_dtype dt, hipStream_t st, bool want_partials,
                    float** partial_out, uint32_t* splits_out );
+int gemm_gate_one_launch( void* hb, const void* x, const void* w13, uint64_t s, uint64_t hidden, uint64_t b, gh_dtype dt, hipStream_t st, bool* done );
 
 namespace {
 
@@ -234,6 +235,13 @@ int gh_matmul_silu_gate( void* hb, const void* x, const void* w13, uint64_t s, u
   }
   GH_REQUIRE( hb != nullptr, "gh_matmul_silu_gate: NULL output" );
   hipStream_t st = as_stream( stream );
+  bool done = false;
+  if ( int rc = gemm_gate_one_launch( hb, x, w13, s, hidden_dim, b, dt, st, &done ) ) {
+    return rc;
+  }
+  if ( done ) {
+    return GH_OK;
+  }
   float* partial = nullptr;
   uint32_t splits = 0;
   if ( int rc = gemm_partials( nullptr, x, w13, s, 2 * hidden_dim, b, dt, st, true, &partial, &splits ) ) {

@@ -109,8 +109,16 @@ __device__ __forceinline__ void half_mfma( f32x16 acc[2], const uint4* wtile, co
   }
 }
 
+// what a work-group does with its accumulators
+constexpr int MODE_PLAIN = 0; // round and store xout(b, r)
+constexpr int MODE_SPLIT = 1; // fp32 partials of a K range
+constexpr int MODE_GATE = 2;  // w = [w1 rows | w3 rows], r = rows of each: store DType(silu(DType(y1)) * DType(y3))
+
 // grid: (row blocks x column slabs, 1, k splits).  s % 256 == 0, 16-byte aligned operands.
-template<bool SPLIT>
+// MODE_GATE: a work-group takes 64 output rows; waves 0, 1 stream them from w1, waves 2, 3 the same
+// rows from w3, so that the two factors of an output element sit in the same lane and accumulator
+// register of a wave pair and meet through LDS after the K loop (no K split in this mode).
+template<int MODE>
 __global__ __launch_bounds__( 256, 2 ) void gemm_stream_kernel( __half* __restrict__ xout,
                                                              float* __restrict__ partial,
                                                              const __half* __restrict__ x,
@@ -134,11 +142,12 @@ __global__ __launch_bounds__( 256, 2 ) void gemm_stream_kernel( __half* __restri
     const uint32_t idx = blockIdx.x >> 3;
     col_slab = idx % n_col_slabs;
     row_block = ( idx / n_col_slabs ) * 8 + ( blockIdx.x & 7 );
-    if ( row_block * WG_ROWS >= r ) {
+    if ( row_block * ( MODE == MODE_GATE ? WG_ROWS / 2 : WG_ROWS ) >= r ) {
       return; // padding of the grid to a multiple of 8 row blocks (whole work-group)
     }
   }
-  const uint32_t row0 = row_block * WG_ROWS + wave * 32;
+  const uint32_t row0 = MODE == MODE_GATE ? row_block * ( WG_ROWS / 2 ) + ( wave & 1 ) * 32 : row_block * WG_ROWS + wave * 32; // output row
+  const uint32_t w_row0 = MODE == MODE_GATE ? ( wave >> 1 ) * r + row0 : row0;
   const uint32_t col0 = col_slab * COLS;
   const uint32_t k_begin = blockIdx.z * k_per_split;
   const uint32_t k_end = min( s, k_begin + k_per_split );
@@ -148,7 +157,7 @@ __global__ __launch_bounds__( 256, 2 ) void gemm_stream_kernel( __half* __restri
   // descriptors bounded to the wave's rows / the work-group's columns: anything past the matrix reads as zero
   const uint32_t w_rows = row0 < r ? min( 32u, r - row0 ) : 0u;
   const uint32_t x_cols = col0 < b ? min( (uint32_t)COLS, b - col0 ) : 0u;
-  const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc( const_cast<__half*>( w + (uint64_t)row0 * s ), 0, (int)( w_rows * ld_bytes ), 0x00020000 );
+  const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc( const_cast<__half*>( w + (uint64_t)w_row0 * s ), 0, (int)( w_rows * ld_bytes ), 0x00020000 );
   const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc( const_cast<__half*>( x + (uint64_t)col0 * s ), 0, (int)( x_cols * ld_bytes ), 0x00020000 );
   const uint32_t w_lane = ( lane >> 4 ) * ld_bytes + ( lane & 15 ) * 16;
   const uint32_t x_lane = ( threadIdx.x >> 4 ) * ld_bytes + ( threadIdx.x & 15 ) * 16;
@@ -202,6 +211,56 @@ __global__ __launch_bounds__( 256, 2 ) void gemm_stream_kernel( __half* __restri
   }
   // acc[t][v]: row = 8*(v/4) + 4*(lane/32) + v%4 of the wave's 32, column = 32*t + lane%32
   const uint32_t g2 = lane >> 5;
+  if ( MODE == MODE_GATE ) {
+    // waves 2, 3 hand DType(y3) to waves 0, 1 through the activation tile's LDS (16 KiB = 2 x 2 x 16 x 64 floats)
+    float* gate = reinterpret_cast<float*>( s_x[0] );
+    __syncthreads(); // every wave is done reading the activation tiles
+    if ( wave >= 2 ) {
+#pragma unroll
+      for ( int t = 0; t < 2; t++ ) {
+#pragma unroll
+        for ( int v = 0; v < 16; v++ ) {
+          gate[( ( ( wave & 1 ) * 2 + t ) * 16 + v ) * 64 + lane] = __half2float( __float2half_rn( acc[t][v] ) );
+        }
+      }
+    }
+    __syncthreads();
+    if ( wave >= 2 ) {
+      return;
+    }
+#pragma unroll
+    for ( int t = 0; t < 2; t++ ) {
+      const uint32_t col = col0 + 32 * t + ( lane & 31 );
+#pragma unroll
+      for ( int q4 = 0; q4 < 4; q4++ ) {
+        const uint32_t row = row0 + 8 * q4 + 4 * g2;
+        union
+        {
+          uint2 raw;
+          __half h[4];
+        } o;
+#pragma unroll
+        for ( int i = 0; i < 4; i++ ) {
+          const float y1 = __half2float( __float2half_rn( acc[t][4 * q4 + i] ) );
+          const float y3 = gate[( ( wave * 2 + t ) * 16 + 4 * q4 + i ) * 64 + lane];
+          o.h[i] = __float2half_rn( y1 / ( 1.0f + __expf( -y1 ) ) * y3 );
+        }
+        if ( col < b ) {
+          __half* dst = xout + (uint64_t)col * r + row;
+          if ( row + 3 < r ) {
+            *reinterpret_cast<uint2*>( dst ) = o.raw;
+          } else {
+            for ( int i = 0; i < 4; i++ ) {
+              if ( row + i < r ) {
+                dst[i] = o.h[i];
+              }
+            }
+          }
+        }
+      }
+    }
+    return;
+  }
 #pragma unroll
   for ( int t = 0; t < 2; t++ ) {
     const uint32_t col = col0 + 32 * t + ( lane & 31 );
@@ -211,7 +270,7 @@ __global__ __launch_bounds__( 256, 2 ) void gemm_stream_kernel( __half* __restri
 #pragma unroll
     for ( int q4 = 0; q4 < 4; q4++ ) {
       const uint32_t row = row0 + 8 * q4 + 4 * g2;
-      if ( SPLIT ) {
+      if ( MODE == MODE_SPLIT ) {
         float* dst = partial + ( (uint64_t)blockIdx.z * b + col ) * r + row;
         if ( row + 3 < r ) {
           *reinterpret_cast<float4*>( dst ) = make_float4( acc[t][4 * q4], acc[t][4 * q4 + 1], acc[t][4 * q4 + 2], acc[t][4 * q4 + 3] );
@@ -253,9 +312,9 @@ void launch( dim3 grid, hipStream_t st, bool split, __half* xout, float* partial
              uint32_t k_per_split, uint32_t n_col_slabs )
 {
   if ( split ) {
-    gemm_stream_kernel<true><<<grid, 256, 0, st>>>( xout, partial, x, w, s, r, b, k_per_split, n_col_slabs );
+    gemm_stream_kernel<MODE_SPLIT><<<grid, 256, 0, st>>>( xout, partial, x, w, s, r, b, k_per_split, n_col_slabs );
   } else {
-    gemm_stream_kernel<false><<<grid, 256, 0, st>>>( xout, partial, x, w, s, r, b, k_per_split, n_col_slabs );
+    gemm_stream_kernel<MODE_PLAIN><<<grid, 256, 0, st>>>( xout, partial, x, w, s, r, b, k_per_split, n_col_slabs );
   }
 }
 
@@ -299,6 +358,30 @@ int gemm_stream_launch( __half* xout, float* partial, const __half* x, const __h
   GH_REQUIRE( gx < ( 1ull << 31 ) && splits <= 65535, "gh_matmul: grid too large" );
   const dim3 grid( (unsigned)gx, 1, splits );
   launch( grid, st, write_partials, xout, partial, x, w, (uint32_t)s, (uint32_t)r, (uint32_t)b, k_per_split, (uint32_t)col_slabs );
+  GH_LAUNCH_CHECK();
+  return GH_OK;
+}
+
+// hb(b, hidden) = DType(silu(DType(x . w1^T)) * DType(x . w3^T)), w13 = w1 rows then w3 rows, in one launch.
+// Only without a K split: the caller checks gemm_stream_gate_applicable first.
+bool gemm_stream_gate_applicable( uint64_t s, uint64_t hidden, uint64_t b, const void* x, const void* w13, const void* hb )
+{
+  if ( !gemm_stream_applicable( s, 2 * hidden, b, x, w13, hb ) ) {
+    return false;
+  }
+  uint32_t splits = 1, k_per_split = 0;
+  gemm_stream_plan( s, 2 * hidden, b, &splits, &k_per_split );
+  return splits == 1;
+}
+
+int gemm_stream_gate_launch( __half* hb, const __half* x, const __half* w13, uint64_t s, uint64_t hidden, uint64_t b, hipStream_t st )
+{
+  const uint64_t row_blocks = ( hidden + WG_ROWS / 2 - 1 ) / ( WG_ROWS / 2 );
+  const uint64_t col_slabs = ( b + COLS - 1 ) / COLS;
+  const uint64_t gx = col_slabs == 1 ? row_blocks : ( row_blocks + 7 ) / 8 * 8 * col_slabs;
+  GH_REQUIRE( gx < ( 1ull << 31 ), "gh_matmul_silu_gate: grid too large" );
+  gemm_stream_kernel<MODE_GATE><<<dim3( (unsigned)gx, 1, 1 ), 256, 0, st>>>( hb, nullptr, x, w13, (uint32_t)s, (uint32_t)hidden, (uint32_t)b, (uint32_t)s,
+                                                                         (uint32_t)col_slabs );
   GH_LAUNCH_CHECK();
   return GH_OK;
 }

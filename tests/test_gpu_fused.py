@@ -47,7 +47,9 @@ def test_matmul_accum_and_norm(dt, b, s, r):
 
 
 @pytest.mark.parametrize("dt", [torch.float16, torch.float32])
-@pytest.mark.parametrize("b,s,hidden", [(4, 288, 768), (64, 512, 1536), (3, 100, 50), (130, 512, 1536), (512, 8192, 12544)])
+@pytest.mark.parametrize("b,s,hidden", [(4, 288, 768), (64, 512, 1536), (3, 100, 50), (130, 512, 1536), (512, 8192, 12544),
+                                        # enough row tiles for one launch without a K split: both factors in one kernel
+                                        (64, 512, 16384), (5, 256, 16404), (33, 1024, 28672)])
 def test_matmul_silu_gate(dt, b, s, hidden):
     g = torch.Generator(device="cuda").manual_seed(2)
     x = torch.randn((b, s), generator=g, device="cuda").to(dt)
@@ -60,6 +62,11 @@ def test_matmul_silu_gate(dt, b, s, hidden):
     # separate calls, so the fp32 sums can differ in the last bit before rounding
     tol = 2e-3 if dt == torch.float16 else 2e-6
     assert torch.allclose(got.float(), hb.float(), rtol=tol, atol=tol)
+    if b * hidden * s <= 64 * 512 * 16384:
+        xh, wh = x.float().cpu().numpy(), w13.float().cpu().numpy()
+        want = O.matmul(xh, np.ascontiguousarray(wh[:hidden]))
+        O.silu(want, O.matmul(xh, np.ascontiguousarray(wh[hidden:])))
+        assert_close(got.float().cpu().numpy(), want, what="fused w1, w3, silu")
 
 
 @pytest.mark.parametrize("dt", [torch.float16, torch.float32])
