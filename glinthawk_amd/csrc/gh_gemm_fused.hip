@@ -101,6 +101,101 @@ __global__ __launch_bounds__( EPI_THREADS ) void epi_accum_norm_kernel( T* __res
   }
 }
 
+// The same for rows of at most 8192 f16 elements (r % 4 == 0, 8-byte aligned rows): a thread owns
+// two groups of four columns for the whole kernel.  Every load -- partials, residual, norm weight --
+// is issued before the first use, and the updated residual stays in registers across the row
+// reduction, so the kernel is two memory round trips deep instead of four.
+__global__ __launch_bounds__( EPI_THREADS ) void epi_accum_norm_row8k_kernel( __half* __restrict__ residual,
+                                                                             const float* __restrict__ partial,
+                                                                             uint32_t r,
+                                                                             uint32_t b,
+                                                                             uint32_t splits,
+                                                                             __half* __restrict__ norm_out,
+                                                                             const __half* __restrict__ norm_weight )
+{
+  __shared__ float smem[EPI_THREADS / WAVE];
+  const uint32_t row = blockIdx.x;
+  const uint64_t n = (uint64_t)b * r;
+  __half* res = residual + (uint64_t)row * r;
+  const float* prow = partial + (uint64_t)row * r;
+  union H4
+  {
+    uint2 raw;
+    __half h[4];
+  };
+  float4 acc[2];
+  H4 old[2], nw[2];
+  bool live[2];
+#pragma unroll
+  for ( int it = 0; it < 2; it++ ) {
+    const uint32_t j = ( it * EPI_THREADS + threadIdx.x ) * 4;
+    live[it] = j < r;
+    acc[it] = make_float4( 0.0f, 0.0f, 0.0f, 0.0f );
+    old[it].raw = make_uint2( 0, 0 );
+    nw[it].raw = make_uint2( 0, 0 );
+    if ( live[it] ) {
+      old[it].raw = *reinterpret_cast<const uint2*>( res + j );
+      if ( norm_out != nullptr ) {
+        nw[it].raw = *reinterpret_cast<const uint2*>( norm_weight + j );
+      }
+    }
+  }
+  for ( uint32_t k = 0; k < splits; k++ ) {
+#pragma unroll
+    for ( int it = 0; it < 2; it++ ) {
+      if ( live[it] ) {
+        const float4 p = *reinterpret_cast<const float4*>( prow + (uint64_t)k * n + ( it * EPI_THREADS + threadIdx.x ) * 4 );
+        acc[it].x += p.x;
+        acc[it].y += p.y;
+        acc[it].z += p.z;
+        acc[it].w += p.w;
+      }
+    }
+  }
+  float ss = 0.0f;
+  float v[2][4];
+#pragma unroll
+  for ( int it = 0; it < 2; it++ ) {
+    const float y[4] = { acc[it].x, acc[it].y, acc[it].z, acc[it].w };
+    H4 o;
+#pragma unroll
+    for ( int e = 0; e < 4; e++ ) {
+      o.h[e] = __float2half_rn( __half2float( old[it].h[e] ) + __half2float( __float2half_rn( y[e] ) ) ); // xb2 = DType(matmul), then accum
+      v[it][e] = __half2float( o.h[e] );
+      ss += v[it][e] * v[it][e];
+    }
+    if ( live[it] ) {
+      *reinterpret_cast<uint2*>( res + ( it * EPI_THREADS + threadIdx.x ) * 4 ) = o.raw;
+    }
+  }
+  if ( norm_out == nullptr ) {
+    return;
+  }
+  ss = wave_sum( ss );
+  if ( threadIdx.x % WAVE == 0 ) {
+    smem[threadIdx.x / WAVE] = ss;
+  }
+  __syncthreads();
+  ss = 0.0f;
+  for ( int w = 0; w < EPI_THREADS / WAVE; w++ ) {
+    ss += smem[w];
+  }
+  ss = ss / (float)r + 1e-5f;
+  const float inv = 1.0f / sqrtf( ss );
+  __half* o = norm_out + (uint64_t)row * r;
+#pragma unroll
+  for ( int it = 0; it < 2; it++ ) {
+    if ( live[it] ) {
+      H4 out;
+#pragma unroll
+      for ( int e = 0; e < 4; e++ ) {
+        out.h[e] = __float2half_rn( __half2float( nw[it].h[e] ) * ( inv * v[it][e] ) );
+      }
+      *reinterpret_cast<uint2*>( o + ( it * EPI_THREADS + threadIdx.x ) * 4 ) = out.raw;
+    }
+  }
+}
+
 // hb(b, hidden) = DType( silu(DType(y1)) * DType(y3) ), partial rows [0, hidden) = w1, [hidden, 2 hidden) = w3
 template<typename T>
 __global__ __launch_bounds__( 256 ) void epi_silu_gate_kernel( T* __restrict__ hb, const float* __restrict__ partial, uint32_t hidden, uint32_t b, uint32_t splits )
@@ -211,7 +306,11 @@ int gh_matmul_accum( void* residual, const void* x, const void* w, uint64_t s, u
   if ( int rc = gemm_partials( nullptr, x, w, s, r, b, dt, st, true, &partial, &splits ) ) {
     return rc;
   }
-  if ( dt == GH_F16 ) {
+  const bool rows_8byte = ( ( reinterpret_cast<uintptr_t>( residual ) | reinterpret_cast<uintptr_t>( norm_out ) | reinterpret_cast<uintptr_t>( norm_weight ) ) & 7u ) == 0;
+  if ( dt == GH_F16 && r % 4 == 0 && r <= 2 * 4 * EPI_THREADS && rows_8byte ) {
+    epi_accum_norm_row8k_kernel<<<(unsigned)b, EPI_THREADS, 0, st>>>( static_cast<__half*>( residual ), partial, (uint32_t)r, (uint32_t)b, splits,
+                                                                     static_cast<__half*>( norm_out ), static_cast<const __half*>( norm_weight ) );
+  } else if ( dt == GH_F16 ) {
     epi_accum_norm_kernel<__half><<<(unsigned)b, EPI_THREADS, 0, st>>>( static_cast<__half*>( residual ), partial, (uint32_t)r, (uint32_t)b, splits,
                                                                static_cast<__half*>( norm_out ), static_cast<const __half*>( norm_weight ) );
   } else {
