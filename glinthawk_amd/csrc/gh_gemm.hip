@@ -17,9 +17,9 @@ namespace gh {
 
 // streaming decode kernel (gh_gemm_stream.hip)
 bool gemm_stream_applicable( uint64_t s, uint64_t r, uint64_t b, const void* x, const void* w, const void* xout );
-void gemm_stream_plan( uint64_t s, uint64_t r, uint64_t b, uint32_t* splits_out, uint32_t* k_per_split_out );
+void gemm_stream_plan( uint64_t s, uint64_t r, uint64_t b, uint32_t* splits_out, uint32_t* k_per_split_out, uint32_t* rows_per_wg_out );
 int gemm_stream_launch( __half* xout, float* partial, const __half* x, const __half* w, uint64_t s, uint64_t r, uint64_t b, uint32_t splits,
-                        uint32_t k_per_split, bool write_partials, hipStream_t st );
+                        uint32_t k_per_split, uint32_t rows_per_wg, bool write_partials, hipStream_t st );
 void gemm_stream_tuning( int target_wgs, int depth );
 bool gemm_stream_gate_applicable( uint64_t s, uint64_t hidden, uint64_t b, const void* x, const void* w13, const void* hb );
 int gemm_stream_gate_launch( __half* hb, const __half* x, const __half* w13, uint64_t s, uint64_t hidden, uint64_t b, hipStream_t st );
@@ -299,8 +299,8 @@ int gemm_partials( void* xout, const void* x, const void* w, uint64_t s, uint64_
   GH_REQUIRE( g_force_kernel != 3, "gh_matmul: the tile kernel needs b > 64, s %% 8 == 0 and 16-byte aligned operands" );
 
   if ( g_force_kernel != 1 && gemm_stream_applicable( s, r, b, x, w, xout ? xout : x ) ) {
-    uint32_t splits = 1, k_per_split = 0;
-    gemm_stream_plan( s, r, b, &splits, &k_per_split );
+    uint32_t splits = 1, k_per_split = 0, rows_per_wg = 0;
+    gemm_stream_plan( s, r, b, &splits, &k_per_split, &rows_per_wg );
     float* ws = nullptr;
     const bool partial = want_partials || splits > 1;
     if ( partial ) {
@@ -311,7 +311,7 @@ int gemm_partials( void* xout, const void* x, const void* w, uint64_t s, uint64_
       *splits_out = splits;
     }
     return gemm_stream_launch( static_cast<__half*>( xout ), ws, static_cast<const __half*>( x ), static_cast<const __half*>( w ), s, r, b, splits, k_per_split,
-                               partial, st );
+                               rows_per_wg, partial, st );
   }
   GH_REQUIRE( g_force_kernel != 2, "gh_matmul: the streaming kernel needs s %% 256 == 0, r %% 4 == 0 and 16-byte aligned operands" );
 

@@ -20,6 +20,9 @@
 // are summed by gemm_reduce_kernel (gh_gemm.hip).
 #include "gh_common.h"
 
+#include <cmath>
+#include <type_traits>
+
 namespace gh {
 
 typedef _Float16 f16x8 __attribute__( ( ext_vector_type( 8 ) ) );
@@ -38,6 +41,13 @@ struct WSlab
   uint4 v[2][8];
 };
 
+// Weights are read once: the non-temporal hint keeps them from displacing the activations, which
+// every work-group re-reads, from the L2 (measured: 7 to 10 % on the 70B projections).
+__device__ __forceinline__ uint4 buffer_load16_stream( __amdgpu_buffer_rsrc_t rsrc, uint32_t lane_offset, uint32_t uniform_offset )
+{
+  return __builtin_bit_cast( uint4, __builtin_amdgcn_raw_buffer_load_b128( rsrc, lane_offset, uniform_offset, 2 /* nt */ ) );
+}
+
 __device__ __forceinline__ uint4 buffer_load16( __amdgpu_buffer_rsrc_t rsrc, uint32_t lane_offset, uint32_t uniform_offset )
 {
   return __builtin_bit_cast( uint4, __builtin_amdgcn_raw_buffer_load_b128( rsrc, lane_offset, uniform_offset, 0 ) );
@@ -50,8 +60,8 @@ __device__ __forceinline__ void load_w_slab( WSlab& dst, __amdgpu_buffer_rsrc_t 
   for ( int j = 0; j < 8; j++ ) {
     const uint32_t row_offset = 4 * j * ld_bytes + kb;
     // both halves of the row back to back: 512 contiguous bytes per row reach the memory system together
-    dst.v[0][j] = buffer_load16( rsrc, lane_offset, row_offset );
-    dst.v[1][j] = buffer_load16( rsrc, lane_offset + 2 * HALF_K, row_offset );
+    dst.v[0][j] = buffer_load16_stream( rsrc, lane_offset, row_offset );
+    dst.v[1][j] = buffer_load16_stream( rsrc, lane_offset + 2 * HALF_K, row_offset );
   }
 }
 
@@ -127,7 +137,8 @@ __global__ __launch_bounds__( 256, 2 ) void gemm_stream_kernel( __half* __restri
                                                              uint32_t r,
                                                              uint32_t b,
                                                              uint32_t k_per_split,
-                                                             uint32_t n_col_slabs )
+                                                             uint32_t n_col_slabs,
+                                                             uint32_t rows_per_wave )
 {
   __shared__ uint4 s_x[2][COLS * 16]; // 2 x 16 KiB
   __shared__ uint4 s_w[4][32 * 16];   // 4 x 8 KiB, one per wave
@@ -142,11 +153,12 @@ __global__ __launch_bounds__( 256, 2 ) void gemm_stream_kernel( __half* __restri
     const uint32_t idx = blockIdx.x >> 3;
     col_slab = idx % n_col_slabs;
     row_block = ( idx / n_col_slabs ) * 8 + ( blockIdx.x & 7 );
-    if ( row_block * ( MODE == MODE_GATE ? WG_ROWS / 2 : WG_ROWS ) >= r ) {
+    if ( row_block * ( MODE == MODE_GATE ? 2 : 4 ) * rows_per_wave >= r ) {
       return; // padding of the grid to a multiple of 8 row blocks (whole work-group)
     }
   }
-  const uint32_t row0 = MODE == MODE_GATE ? row_block * ( WG_ROWS / 2 ) + ( wave & 1 ) * 32 : row_block * WG_ROWS + wave * 32; // output row
+  // a wave owns rows_per_wave (<= 32, a multiple of 4) rows of its 32-row MFMA tile; the others read as zero and are not stored
+  const uint32_t row0 = MODE == MODE_GATE ? ( row_block * 2 + ( wave & 1 ) ) * rows_per_wave : ( row_block * 4 + wave ) * rows_per_wave; // output row
   const uint32_t w_row0 = MODE == MODE_GATE ? ( wave >> 1 ) * r + row0 : row0;
   const uint32_t col0 = col_slab * COLS;
   const uint32_t k_begin = blockIdx.z * k_per_split;
@@ -155,7 +167,7 @@ __global__ __launch_bounds__( 256, 2 ) void gemm_stream_kernel( __half* __restri
   uint4* wtile = s_w[wave];
 
   // descriptors bounded to the wave's rows / the work-group's columns: anything past the matrix reads as zero
-  const uint32_t w_rows = row0 < r ? min( 32u, r - row0 ) : 0u;
+  const uint32_t w_rows = row0 < r ? min( rows_per_wave, r - row0 ) : 0u;
   const uint32_t x_cols = col0 < b ? min( (uint32_t)COLS, b - col0 ) : 0u;
   const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc( const_cast<__half*>( w + (uint64_t)w_row0 * s ), 0, (int)( w_rows * ld_bytes ), 0x00020000 );
   const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc( const_cast<__half*>( x + (uint64_t)col0 * s ), 0, (int)( x_cols * ld_bytes ), 0x00020000 );
@@ -175,38 +187,47 @@ __global__ __launch_bounds__( 256, 2 ) void gemm_stream_kernel( __half* __restri
   // other.  Loads retire in order, so the issue order matters: the weight loads of slab i+1 go out
   // first in iteration i, the activation halves of slab i+1 follow as their registers are staged;
   // everything iteration i+1 waits for is then older than the weight loads it issues itself.
+  //
+  // The loop body has no conditional loads and no joins: the compiler counts outstanding loads per
+  // path and, where paths with different counts meet, waits for the smaller count -- which here
+  // would mean waiting for the slab that was just requested.  So the prologue issues in the same
+  // order as an iteration leaves things (weights, then activations), the loads behind the last slab
+  // are still issued but aimed past the descriptors' bounds (they return zero without touching
+  // memory), and the loop is left by `break`.
+  constexpr uint32_t PAST_THE_END = 0x80000000u; // + lane and row offsets (< 2^30) stays below 2^32 and above any descriptor's size
   const uint32_t n_slabs = ( k_end - k_begin ) / SLAB_K; // K ranges are multiples of SLAB_K
   uint32_t cur = ( ( row_block + blockIdx.z ) * 3u ) % n_slabs; // rotated start, see the header
   WSlab wr[2];
   XSlab xr;
   {
     const uint32_t kb = ( k_begin + cur * SLAB_K ) * 2;
+    load_w_slab( wr[0], w_rsrc, w_lane, ld_bytes, kb );
     load_x_half( xr, x_rsrc, x_lane, ld_bytes, kb, 0 );
     load_x_half( xr, x_rsrc, x_lane, ld_bytes, kb, 1 );
-    load_w_slab( wr[0], w_rsrc, w_lane, ld_bytes, kb );
   }
-  for ( uint32_t j0 = 0; j0 < n_slabs; j0 += 2 ) {
+  uint32_t j = 0;
+  auto consume = [&]( auto set_tag ) {
+    constexpr int set = decltype( set_tag )::value;
+    cur = cur + 1 == n_slabs ? 0 : cur + 1;
+    const uint32_t kb = j + 1 < n_slabs ? ( k_begin + cur * SLAB_K ) * 2 : PAST_THE_END;
+    load_w_slab( wr[set ^ 1], w_rsrc, w_lane, ld_bytes, kb );
 #pragma unroll
-    for ( int set = 0; set < 2; set++ ) {
-      const uint32_t j = j0 + set;
-      if ( j < n_slabs ) { // uniform across the work-group
-        cur = cur + 1 == n_slabs ? 0 : cur + 1;
-        const bool more = j + 1 < n_slabs;
-        const uint32_t kb = ( k_begin + cur * SLAB_K ) * 2;
-        if ( more ) {
-          load_w_slab( wr[set ^ 1], w_rsrc, w_lane, ld_bytes, kb );
-        }
-#pragma unroll
-        for ( int h = 0; h < 2; h++ ) {
-          stage_x_half( s_x[h], xr, h );
-          stage_w_half( wtile, wr[set], h );
-          if ( more ) {
-            load_x_half( xr, x_rsrc, x_lane, ld_bytes, kb, h ); // same registers, next slab
-          }
-          __syncthreads();
-          half_mfma( acc, wtile, s_x[h] );
-        }
-      }
+    for ( int h = 0; h < 2; h++ ) {
+      stage_x_half( s_x[h], xr, h );
+      stage_w_half( wtile, wr[set], h );
+      load_x_half( xr, x_rsrc, x_lane, ld_bytes, kb, h ); // same registers, next slab
+      __syncthreads();
+      half_mfma( acc, wtile, s_x[h] );
+    }
+  };
+  for ( ;; ) { // exits are uniform across the work-group
+    consume( std::integral_constant<int, 0> {} );
+    if ( ++j == n_slabs ) {
+      break;
+    }
+    consume( std::integral_constant<int, 1> {} );
+    if ( ++j == n_slabs ) {
+      break;
     }
   }
   // acc[t][v]: row = 8*(v/4) + 4*(lane/32) + v%4 of the wave's 32, column = 32*t + lane%32
@@ -245,7 +266,7 @@ __global__ __launch_bounds__( 256, 2 ) void gemm_stream_kernel( __half* __restri
           const float y3 = gate[( ( wave * 2 + t ) * 16 + 4 * q4 + i ) * 64 + lane];
           o.h[i] = __float2half_rn( y1 / ( 1.0f + __expf( -y1 ) ) * y3 );
         }
-        if ( col < b ) {
+        if ( col < b && 8 * q4 + 4 * g2 < rows_per_wave ) {
           __half* dst = xout + (uint64_t)col * r + row;
           if ( row + 3 < r ) {
             *reinterpret_cast<uint2*>( dst ) = o.raw;
@@ -270,6 +291,9 @@ __global__ __launch_bounds__( 256, 2 ) void gemm_stream_kernel( __half* __restri
 #pragma unroll
     for ( int q4 = 0; q4 < 4; q4++ ) {
       const uint32_t row = row0 + 8 * q4 + 4 * g2;
+      if ( 8 * q4 + 4 * g2 >= rows_per_wave ) {
+        continue;
+      }
       if ( MODE == MODE_SPLIT ) {
         float* dst = partial + ( (uint64_t)blockIdx.z * b + col ) * r + row;
         if ( row + 3 < r ) {
@@ -309,12 +333,12 @@ __global__ __launch_bounds__( 256, 2 ) void gemm_stream_kernel( __half* __restri
 int g_target_wgs = 256;
 
 void launch( dim3 grid, hipStream_t st, bool split, __half* xout, float* partial, const __half* x, const __half* w, uint32_t s, uint32_t r, uint32_t b,
-             uint32_t k_per_split, uint32_t n_col_slabs )
+             uint32_t k_per_split, uint32_t n_col_slabs, uint32_t rows_per_wave )
 {
   if ( split ) {
-    gemm_stream_kernel<MODE_SPLIT><<<grid, 256, 0, st>>>( xout, partial, x, w, s, r, b, k_per_split, n_col_slabs );
+    gemm_stream_kernel<MODE_SPLIT><<<grid, 256, 0, st>>>( xout, partial, x, w, s, r, b, k_per_split, n_col_slabs, rows_per_wave );
   } else {
-    gemm_stream_kernel<MODE_PLAIN><<<grid, 256, 0, st>>>( xout, partial, x, w, s, r, b, k_per_split, n_col_slabs );
+    gemm_stream_kernel<MODE_PLAIN><<<grid, 256, 0, st>>>( xout, partial, x, w, s, r, b, k_per_split, n_col_slabs, rows_per_wave );
   }
 }
 
@@ -326,38 +350,62 @@ bool gemm_stream_applicable( uint64_t s, uint64_t r, uint64_t b, const void* x, 
   return s % SLAB_K == 0 && s < ( 1u << 24 ) && r % 4 == 0 && ( ( reinterpret_cast<uintptr_t>( x ) | reinterpret_cast<uintptr_t>( w ) | reinterpret_cast<uintptr_t>( xout ) ) & 15u ) == 0;
 }
 
-// picks the K split; returns the number of splits and k per split
-void gemm_stream_plan( uint64_t s, uint64_t r, uint64_t b, uint32_t* splits_out, uint32_t* k_per_split_out )
+// Picks the K split and the rows per work-group.
+//
+// What the choice has to get right (measured on the 70B shapes with cold weights, per-work-group
+// time stamps): a CU pulls about 1/256 of the chip's bandwidth whatever runs on it, so a launch is
+// as slow as its busiest CU (320 equal work-groups on 256 CUs: 48 us; the same bytes as 240: 38 us);
+// a CU needs about 72 KiB of loads in flight to reach that rate, and a work-group keeps one
+// register slab (rows x 512 bytes) in flight, so two small tiles or one full tile per CU;
+// every split adds an fp32 partial tile per output element, written and read again; and a
+// work-group's first slab arrives late.  The row tile only shrinks below 128 where there is no K
+// split to balance the launch with (a wave keeps its 32-row MFMA tile and leaves rows unused).
+void gemm_stream_plan( uint64_t s, uint64_t r, uint64_t b, uint32_t* splits_out, uint32_t* k_per_split_out, uint32_t* rows_per_wg_out )
 {
-  const uint64_t tiles = ( ( r + WG_ROWS - 1 ) / WG_ROWS ) * ( ( b + COLS - 1 ) / COLS );
-  uint32_t splits = 1;
-  if ( tiles < (uint64_t)g_target_wgs ) {
-    // two work-groups per CU hide each other's staging and MFMA phases, but only pay off while every
-    // work-group still streams at least 8 slabs; otherwise one per CU with at least 4 slabs each
-    const uint32_t two_per_cu = (uint32_t)( ( 2 * g_target_wgs + tiles - 1 ) / tiles );
-    if ( s / two_per_cu >= 8 * SLAB_K ) {
-      splits = two_per_cu;
-    } else {
-      splits = (uint32_t)( ( g_target_wgs + tiles - 1 ) / tiles );
-      const uint32_t max_by_k = (uint32_t)std::max<uint64_t>( 1, s / ( 4 * SLAB_K ) );
-      splits = std::min( splits, max_by_k );
+  const uint64_t col_slabs = ( b + COLS - 1 ) / COLS;
+  const double n_cu = (double)g_target_wgs;
+  const uint64_t total_slabs = s / SLAB_K;
+  double best_cost = 0.0;
+  uint32_t best_rows = WG_ROWS, best_splits = 1, best_kps = (uint32_t)s;
+  bool have = false;
+  for ( uint32_t rows = WG_ROWS; rows >= 96; rows -= 16 ) {
+    const uint64_t tiles = ( ( r + rows - 1 ) / rows ) * col_slabs;
+    for ( uint32_t want = 1; want <= 16 && want <= total_slabs; want++ ) {
+      const uint64_t kps = ( total_slabs + want - 1 ) / want * SLAB_K;
+      const uint32_t splits = (uint32_t)( ( s + kps - 1 ) / kps );
+      if ( splits != want || ( splits > 1 && ( kps < 4 * SLAB_K || rows != WG_ROWS ) ) ) {
+        continue; // the same plan as a smaller `want`; too little K per work-group to pipeline; small tiles only without a split
+      }
+      const double slab_bytes = (double)rows * SLAB_K * 2.0;
+      const double per_cu = std::ceil( (double)( tiles * splits ) / n_cu );
+      const double busiest = per_cu * (double)rows * (double)kps * 2.0;
+      const double rate = std::min( 1.0, std::min( per_cu, 2.0 ) * slab_bytes / ( 72.0 * 1024.0 ) );
+      const double partials = splits > 1 ? 2.0 * splits * (double)b * (double)r * 4.0 / n_cu : 0.0;
+      const double cost = busiest / rate + partials + per_cu * slab_bytes;
+      if ( !have || cost < best_cost ) {
+        have = true;
+        best_cost = cost;
+        best_rows = rows;
+        best_splits = splits;
+        best_kps = (uint32_t)kps;
+      }
     }
   }
-  uint32_t k_per_split = (uint32_t)( ( s + splits - 1 ) / splits );
-  k_per_split = ( k_per_split + SLAB_K - 1 ) / SLAB_K * SLAB_K;
-  *splits_out = (uint32_t)( ( s + k_per_split - 1 ) / k_per_split );
-  *k_per_split_out = k_per_split;
+  *splits_out = best_splits;
+  *k_per_split_out = best_kps;
+  *rows_per_wg_out = best_rows;
 }
 
 int gemm_stream_launch( __half* xout, float* partial, const __half* x, const __half* w, uint64_t s, uint64_t r, uint64_t b, uint32_t splits,
-                        uint32_t k_per_split, bool write_partials, hipStream_t st )
+                        uint32_t k_per_split, uint32_t rows_per_wg, bool write_partials, hipStream_t st )
 {
-  const uint64_t row_blocks = ( r + WG_ROWS - 1 ) / WG_ROWS;
+  GH_REQUIRE( rows_per_wg % 16 == 0 && rows_per_wg >= 16 && rows_per_wg <= WG_ROWS, "gh_matmul: bad row tile %u", rows_per_wg );
+  const uint64_t row_blocks = ( r + rows_per_wg - 1 ) / rows_per_wg;
   const uint64_t col_slabs = ( b + COLS - 1 ) / COLS;
   const uint64_t gx = col_slabs == 1 ? row_blocks : ( row_blocks + 7 ) / 8 * 8 * col_slabs;
   GH_REQUIRE( gx < ( 1ull << 31 ) && splits <= 65535, "gh_matmul: grid too large" );
   const dim3 grid( (unsigned)gx, 1, splits );
-  launch( grid, st, write_partials, xout, partial, x, w, (uint32_t)s, (uint32_t)r, (uint32_t)b, k_per_split, (uint32_t)col_slabs );
+  launch( grid, st, write_partials, xout, partial, x, w, (uint32_t)s, (uint32_t)r, (uint32_t)b, k_per_split, (uint32_t)col_slabs, rows_per_wg / 4 );
   GH_LAUNCH_CHECK();
   return GH_OK;
 }
@@ -369,19 +417,23 @@ bool gemm_stream_gate_applicable( uint64_t s, uint64_t hidden, uint64_t b, const
   if ( !gemm_stream_applicable( s, 2 * hidden, b, x, w13, hb ) ) {
     return false;
   }
-  uint32_t splits = 1, k_per_split = 0;
-  gemm_stream_plan( s, 2 * hidden, b, &splits, &k_per_split );
+  uint32_t splits = 1, k_per_split = 0, rows = 0;
+  gemm_stream_plan( s, 2 * hidden, b, &splits, &k_per_split, &rows );
   return splits == 1;
 }
 
 int gemm_stream_gate_launch( __half* hb, const __half* x, const __half* w13, uint64_t s, uint64_t hidden, uint64_t b, hipStream_t st )
 {
-  const uint64_t row_blocks = ( hidden + WG_ROWS / 2 - 1 ) / ( WG_ROWS / 2 );
+  uint32_t splits = 1, k_per_split = 0, rows = 0;
+  gemm_stream_plan( s, 2 * hidden, b, &splits, &k_per_split, &rows );
+  GH_REQUIRE( splits == 1, "gh_matmul_silu_gate: the one-launch form does not split K" );
+  const uint32_t rows_per_wave = rows / 4; // two waves on w1, two on w3: rows / 2 output rows per work-group
+  const uint64_t row_blocks = ( hidden + 2 * rows_per_wave - 1 ) / ( 2 * rows_per_wave );
   const uint64_t col_slabs = ( b + COLS - 1 ) / COLS;
   const uint64_t gx = col_slabs == 1 ? row_blocks : ( row_blocks + 7 ) / 8 * 8 * col_slabs;
   GH_REQUIRE( gx < ( 1ull << 31 ), "gh_matmul_silu_gate: grid too large" );
   gemm_stream_kernel<MODE_GATE><<<dim3( (unsigned)gx, 1, 1 ), 256, 0, st>>>( hb, nullptr, x, w13, (uint32_t)s, (uint32_t)hidden, (uint32_t)b, (uint32_t)s,
-                                                                         (uint32_t)col_slabs );
+                                                                         (uint32_t)col_slabs, rows_per_wave );
   GH_LAUNCH_CHECK();
   return GH_OK;
 }

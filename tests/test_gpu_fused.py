@@ -137,7 +137,9 @@ def test_stage_with_and_without_fused_projections(name, dtype):
         assert a.forward() and b.forward()
         la = d2h(a.scratch_ptr("logits"), (batch, cfg.vocab_size), np_dt).astype(np.float32)
         lb = d2h(b.scratch_ptr("logits"), (batch, cfg.vocab_size), np_dt).astype(np.float32)
-        tol = 4e-3 if dtype == "f16" else 2e-5       # only the rmsnorm reduction order differs between the two
+        # the two differ in reduction order only: the rmsnorm sum, and the K split of a concatenated
+        # projection against the split of its parts (an fp16 rounding can flip and travel through the layers)
+        tol = 8e-3 if dtype == "f16" else 2e-5
         np.testing.assert_allclose(la, lb, rtol=tol, atol=tol)
         assert_close(la, want, mean_rel=2e-3 if dtype == "f16" else 1e-3, what=f"{name} fused-projection logits step {step}")
         tokens = [a.row(i)["token"] for i in range(batch)]
