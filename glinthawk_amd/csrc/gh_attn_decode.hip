@@ -245,6 +245,12 @@ __device__ __forceinline__ float row16_sum( float v )
 }
 
 __device__ __forceinline__ uint4 load16( const __half* p ) { return *reinterpret_cast<const uint4*>( p ); }
+// cache rows are read once per launch: non-temporal, so that they do not push the queries and partials out of the L2
+typedef uint32_t u32x4_t __attribute__( ( ext_vector_type( 4 ) ) );
+__device__ __forceinline__ uint4 load16_stream( const __half* p )
+{
+  return __builtin_bit_cast( uint4, __builtin_nontemporal_load( reinterpret_cast<const u32x4_t*>( p ) ) );
+}
 
 __device__ __forceinline__ float dot8( const uint4& a, const uint4& b, float acc )
 {
@@ -325,8 +331,8 @@ __global__ __launch_bounds__( 256 ) void attn_decode_valu_kernel( const __half* 
     const uint32_t tok = t0 + 4 * j + r;
     const bool ok = tok < job.t_end;
     const __half* row = kp + (uint64_t)tok * row_elems;
-    kn[j] = ok ? load16( row ) : zero4;
-    vn[j] = ok ? load16( row + v_off ) : zero4;
+    kn[j] = ok ? load16_stream( row ) : zero4;
+    vn[j] = ok ? load16_stream( row + v_off ) : zero4;
   }
 
   for ( uint32_t it = 0; it < n_tiles; it++ ) {
@@ -345,8 +351,8 @@ __global__ __launch_bounds__( 256 ) void attn_decode_valu_kernel( const __half* 
       const uint32_t tok = t_next + 4 * j + r;
       const bool ok = more && tok < job.t_end;
       const __half* row = kp + (uint64_t)tok * row_elems;
-      kn[j] = ok ? load16( row ) : zero4;
-      vn[j] = ok ? load16( row + v_off ) : zero4;
+      kn[j] = ok ? load16_stream( row ) : zero4;
+      vn[j] = ok ? load16_stream( row + v_off ) : zero4;
     }
 
     float s[4][G];
@@ -516,8 +522,8 @@ __global__ __launch_bounds__( 256 ) void attn_decode_mfma_kernel( const __half* 
     const uint32_t tok = t0 + 4 * g4 + i;
     const bool ok = tok < job.t_end;
     const __half* row = kp + (uint64_t)tok * row_elems;
-    kn[i] = ok ? load16( row ) : zero4;
-    vn[i] = ok ? load16( row + v_off ) : zero4;
+    kn[i] = ok ? load16_stream( row ) : zero4;
+    vn[i] = ok ? load16_stream( row + v_off ) : zero4;
   }
 
   for ( uint32_t it = 0; it < n_tiles; it++ ) {
@@ -538,8 +544,8 @@ __global__ __launch_bounds__( 256 ) void attn_decode_mfma_kernel( const __half* 
       const uint32_t tok = t_next + 4 * g4 + i;
       const bool ok = more && tok < job.t_end;
       const __half* row = kp + (uint64_t)tok * row_elems;
-      kn[i] = ok ? load16( row ) : zero4;
-      vn[i] = ok ? load16( row + v_off ) : zero4;
+      kn[i] = ok ? load16_stream( row ) : zero4;
+      vn[i] = ok ? load16_stream( row + v_off ) : zero4;
     }
     __builtin_amdgcn_fence( __ATOMIC_RELEASE, "wavefront" );
     __builtin_amdgcn_wave_barrier();
