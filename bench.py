@@ -33,7 +33,7 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch of the dominant kernel, from the FETCH_SIZE / WRITE_SIZE counter passes
 # summarised in profiles/attn_decode_mfma_llama2-70b-gqa-b64-ctx4096_hbm_counters.md (each counter
 # scaled by what it reads for a 1 GiB copy).  Only valid for the workload it was measured on.
-MEASURED_TRAFFIC = {"llama2-70b-gqa-b64-ctx4096": 1086918181}
+MEASURED_TRAFFIC = {"llama2-70b-gqa-b64-ctx4096": 1086915785}
 
 # the decode configurations that fit one GPU as a single stage (the first is the headline)
 WORKLOADS = {
