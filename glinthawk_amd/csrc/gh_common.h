@@ -40,6 +40,8 @@ int fail( int status, const char* fmt, ... ) __attribute__( ( format( printf, 2,
 #define GH_LAUNCH_CHECK() GH_HIP( hipGetLastError() )
 
 int ensure_init();
+// compute units of the device the library was initialised on (256 before initialisation)
+int cu_count();
 
 inline hipStream_t as_stream( gh_stream s ) { return reinterpret_cast<hipStream_t>( s ); }
 

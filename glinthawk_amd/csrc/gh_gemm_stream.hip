@@ -193,7 +193,8 @@ __global__ __launch_bounds__( 256, 2 ) void gemm_stream_kernel( __half* __restri
   // would mean waiting for the slab that was just requested.  So the prologue issues in the same
   // order as an iteration leaves things (weights, then activations), the loads behind the last slab
   // are still issued but aimed past the descriptors' bounds (they return zero without touching
-  // memory), and the loop is left by `break`.
+  // memory: the scalar offset is part of the range check on this hardware, which gh_init verifies),
+  // and the loop is left by `break`.
   constexpr uint32_t PAST_THE_END = 0x80000000u; // + lane and row offsets (< 2^30) stays below 2^32 and above any descriptor's size
   const uint32_t n_slabs = ( k_end - k_begin ) / SLAB_K; // K ranges are multiples of SLAB_K
   uint32_t cur = ( ( row_block + blockIdx.z ) * 3u ) % n_slabs; // rotated start, see the header
@@ -330,7 +331,7 @@ __global__ __launch_bounds__( 256, 2 ) void gemm_stream_kernel( __half* __restri
   }
 }
 
-int g_target_wgs = 256;
+int g_target_wgs = 0; // tuning override of the CU count the plan balances for (0: the device's)
 
 void launch( dim3 grid, hipStream_t st, bool split, __half* xout, float* partial, const __half* x, const __half* w, uint32_t s, uint32_t r, uint32_t b,
              uint32_t k_per_split, uint32_t n_col_slabs, uint32_t rows_per_wave )
@@ -363,7 +364,7 @@ bool gemm_stream_applicable( uint64_t s, uint64_t r, uint64_t b, const void* x, 
 void gemm_stream_plan( uint64_t s, uint64_t r, uint64_t b, uint32_t* splits_out, uint32_t* k_per_split_out, uint32_t* rows_per_wg_out )
 {
   const uint64_t col_slabs = ( b + COLS - 1 ) / COLS;
-  const double n_cu = (double)g_target_wgs;
+  const double n_cu = (double)( g_target_wgs > 0 ? g_target_wgs : cu_count() );
   const uint64_t total_slabs = s / SLAB_K;
   double best_cost = 0.0;
   uint32_t best_rows = WG_ROWS, best_splits = 1, best_kps = (uint32_t)s;

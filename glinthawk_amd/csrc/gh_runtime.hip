@@ -16,6 +16,7 @@ thread_local char g_error[512] = "";
 std::mutex g_mutex;
 bool g_ready = false;
 int g_device = -1;
+int g_cu_count = 256; // compute units of the initialised device (a full MI355X: 256)
 char g_arch[128] = "";
 
 // ---- staging ring ------------------------------------------------------------------------------
@@ -56,6 +57,37 @@ int fail( int status, const char* fmt, ... )
   return status;
 }
 
+// The GEMM kernels bound their buffer loads by the descriptor's size and put row and
+// K offsets into the scalar offset operand, including offsets that are meant to fall outside.  That
+// is only safe if the scalar offset takes part in the hardware's range check (it does on gfx950;
+// the compiler's contract for the intrinsic does not promise it), so initialisation checks it once
+// on memory where either answer is harmless.
+__global__ void buffer_bounds_probe_kernel( const uint32_t* buf, uint32_t* out, uint32_t scalar_offset )
+{
+  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc( const_cast<uint32_t*>( buf ), 0, 1024, 0x00020000 );
+  const uint32_t so = __builtin_amdgcn_readfirstlane( scalar_offset );
+  out[threadIdx.x] = __builtin_amdgcn_raw_buffer_load_b32( rsrc, threadIdx.x * 4, so, 0 );
+}
+
+int check_buffer_bounds()
+{
+  uint32_t* buf = nullptr;
+  GH_HIP( hipMalloc( reinterpret_cast<void**>( &buf ), 4096 + 64 * 4 ) );
+  uint32_t* out = buf + 1024;
+  GH_HIP( hipMemset( buf, 0x5a, 4096 + 64 * 4 ) );
+  buffer_bounds_probe_kernel<<<1, 64>>>( buf, out, 2048 ); // descriptor: 1024 bytes; the loads land at 2048.. of a 4096-byte block
+  GH_HIP( hipGetLastError() );
+  uint32_t host[64];
+  GH_HIP( hipMemcpy( host, out, sizeof( host ), hipMemcpyDeviceToHost ) );
+  GH_HIP( hipFree( buf ) );
+  for ( uint32_t v : host ) {
+    if ( v != 0 ) {
+      return fail( GH_ERR_DEVICE, "this device does not range-check the scalar offset of buffer loads; the kernels of this library rely on it" );
+    }
+  }
+  return GH_OK;
+}
+
 static int init_locked( int device )
 {
   int count = 0;
@@ -74,15 +106,21 @@ static int init_locked( int device )
   if ( strncmp( prop.gcnArchName, "gfx950", 6 ) != 0 ) {
     return fail( GH_ERR_NO_DEVICE, "device %d is %s; this library holds gfx950 code only", device, prop.gcnArchName );
   }
+  if ( int rc = check_buffer_bounds() ) {
+    return rc;
+  }
   for ( int i = 0; i < STAGE_SLOTS; i++ ) {
     GH_HIP( hipHostMalloc( reinterpret_cast<void**>( &g_slots[i].pinned ), STAGE_SLOT_BYTES, hipHostMallocDefault ) );
     GH_HIP( hipMalloc( reinterpret_cast<void**>( &g_slots[i].device ), STAGE_SLOT_BYTES ) );
     GH_HIP( hipEventCreateWithFlags( &g_slots[i].done, hipEventDisableTiming ) );
   }
   g_device = device;
+  g_cu_count = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
   g_ready = true;
   return GH_OK;
 }
+
+int cu_count() { return g_cu_count; }
 
 int ensure_init()
 {
