@@ -1,8 +1,9 @@
 // Projection GEMMs fused with the ops that follow them in the reference's layer
 // (models/llama2/model.hh:326-427).  The GEMM kernel leaves fp32 partial sums [splits][b][r]; one
-// epilogue kernel per call sums the splits and applies the follow-up ops, so a layer needs 10
-// launches instead of 21.  Rounding points are those of the unfused sequence: every matmul result
-// is rounded to DType first (the reference stores it), later math is fp32 with one rounding per store.
+// epilogue kernel per call sums the splits and applies the follow-up ops (w1, w3 and the SiLU gate
+// are a single launch when no K split is needed), so a layer needs 9 launches instead of 21.
+// Rounding points are those of the unfused sequence: every matmul result is rounded to DType first
+// (the reference stores it), later math is fp32 with one rounding per store.
 #include "gh_common.h"
 
 namespace gh {

@@ -2,9 +2,12 @@
 // (64 columns per column slab), f16 storage, fp32 accumulate.  Every weight element is read from HBM
 // exactly once, so the kernel is built like a streaming read:
 //
-//   work-group = 4 waves = 128 weight rows x one K range; wave = 32 rows x all 64 batch columns
+//   work-group = 4 waves = up to 128 weight rows x one K range; wave = up to 32 rows x all 64 batch
+//               columns (the planner may give a wave fewer rows of its 32-row MFMA tile so that the
+//               number of work-groups suits the number of CUs)
 //   weights     global -> registers with fully coalesced 16-byte buffer loads (scalar row/k offsets,
-//               rows past the end read as zero by the descriptor's bound).  A register slab is 32 rows
+//               rows past the end read as zero by the descriptor's bound), non-temporal: they are
+//               read once and should not displace the activations from L2.  A register slab is 32 rows
 //               x 256 k, 512 contiguous bytes per row per visit.  Two register sets: slab i+1 is in
 //               flight while slab i is consumed.  From registers each 128-k half goes through a
 //               wave-private LDS tile (XOR-swizzled 16-byte chunks) into MFMA operand order.
@@ -17,7 +20,8 @@
 //   math        v_mfma_f32_32x32x16_f16: A = 32 weight rows, B = 32 batch columns, two column tiles
 //
 // K is split across work-groups when there are too few row slabs to fill the chip; the fp32 partials
-// are summed by gemm_reduce_kernel (gh_gemm.hip).
+// are summed by gemm_reduce_kernel (gh_gemm.hip) or by the fused epilogues (gh_gemm_fused.hip).
+// Without a split, w1 and w3 can share a launch that applies the SiLU gate itself (MODE_GATE).
 #include "gh_common.h"
 
 #include <cmath>

@@ -506,7 +506,7 @@ private:
     ops_.template accum<Config::dim>( x_, xb_, batch_ );
   }
 
-  // One whole layer with the projections fused with their follow-up ops: 10 launches instead of 21.
+  // One whole layer with the projections fused with their follow-up ops: 9 or 10 launches instead of 21.
   // Expects xb_ = rmsnorm(x_) * rms_att_weight on entry; leaves the same for the next layer when
   // `next_att_norm` is given.
   void fused_layer_ops( const size_t layer, const size_t table_index, const DType* next_att_norm )
