@@ -207,6 +207,38 @@ def test_matmul_many_rows_layout_one_hot():
     assert torch.equal(got, w[:, cols].t().contiguous())
 
 
+def _streaming_shapes():
+    rng = np.random.default_rng(77)
+    shapes = [(64, 8192, 10240), (64, 2048, 57344), (33, 1024, 28672), (200, 512, 1100)]   # 3 splits; 112-row tiles; ragged batch; 4 column slabs
+    for _ in range(20):
+        shapes.append((int(rng.integers(1, 200)), 256 * int(rng.integers(1, 24)), 4 * int(rng.integers(1, 5000))))
+    return shapes
+
+
+@pytest.mark.parametrize("b,s,r", _streaming_shapes())
+def test_matmul_streaming_kernel_sweep(b, s, r):
+    """The weight-streaming kernel forced on shapes that walk through its plans: K splits, row tiles
+    below 128, ragged last row blocks, one to four column slabs.  One-hot activations make the check
+    bit exact (every output is one weight), a random product bounds the arithmetic."""
+    from glinthawk_amd import _lib
+    g = torch.Generator(device="cuda").manual_seed(b * 7 + r)
+    w = (torch.randn((r, s), generator=g, device="cuda") / s ** 0.5).half()
+    hot = torch.zeros((b, s), dtype=torch.float16, device="cuda")
+    cols = torch.tensor([(7919 * i + 3) % s for i in range(b)], device="cuda")
+    hot[torch.arange(b, device="cuda"), cols] = 1
+    x = torch.randn((b, s), generator=g, device="cuda").half()
+    _lib.lib().gh_gemm_set_tuning(2, 0, 0)
+    try:
+        got_hot = ops.matmul(hot, w)
+        got = ops.matmul(x, w)
+    finally:
+        _lib.lib().gh_gemm_set_tuning(0, 0, 0)
+    assert torch.equal(got_hot, w[:, cols].t().contiguous())
+    want = x.float() @ w.float().t()
+    err = (got.float() - want).abs()
+    assert err.max().item() < 2e-2 and (err.mean() / want.abs().mean()).item() < 1e-3
+
+
 def test_matmul_layout_one_hot():
     s, r = 256, 192
     w = torch.arange(r * s, dtype=torch.float32).reshape(r, s).remainder(1000).half().cuda()
