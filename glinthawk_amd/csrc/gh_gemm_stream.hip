@@ -378,7 +378,7 @@ void gemm_stream_plan( uint64_t s, uint64_t r, uint64_t b, uint32_t* splits_out,
     for ( uint32_t want = 1; want <= 16 && want <= total_slabs; want++ ) {
       const uint64_t kps = ( total_slabs + want - 1 ) / want * SLAB_K;
       const uint32_t splits = (uint32_t)( ( s + kps - 1 ) / kps );
-      if ( splits != want || ( splits > 1 && ( kps < 4 * SLAB_K || rows != WG_ROWS ) ) ) {
+      if ( splits != want || ( splits > 1 && ( kps < 2 * SLAB_K || rows != WG_ROWS ) ) ) {
         continue; // the same plan as a smaller `want`; too little K per work-group to pipeline; small tiles only without a split
       }
       const double slab_bytes = (double)rows * SLAB_K * 2.0;
