@@ -419,7 +419,7 @@ int gemm_stream_launch( __half* xout, float* partial, const __half* x, const __h
 // Only without a K split: the caller checks gemm_stream_gate_applicable first.
 bool gemm_stream_gate_applicable( uint64_t s, uint64_t hidden, uint64_t b, const void* x, const void* w13, const void* hb )
 {
-  if ( !gemm_stream_applicable( s, 2 * hidden, b, x, w13, hb ) ) {
+  if ( hidden % 4 != 0 || !gemm_stream_applicable( s, 2 * hidden, b, x, w13, hb ) ) { // 8-byte output stores
     return false;
   }
   uint32_t splits = 1, k_per_split = 0, rows = 0;

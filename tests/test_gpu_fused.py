@@ -49,7 +49,8 @@ def test_matmul_accum_and_norm(dt, b, s, r):
 @pytest.mark.parametrize("dt", [torch.float16, torch.float32])
 @pytest.mark.parametrize("b,s,hidden", [(4, 288, 768), (64, 512, 1536), (3, 100, 50), (130, 512, 1536), (512, 8192, 12544),
                                         # enough row tiles for one launch without a K split: both factors in one kernel
-                                        (64, 512, 16384), (5, 256, 16404), (33, 1024, 28672)])
+                                        (64, 512, 16384), (5, 256, 16404), (33, 1024, 28672),
+                                        (5, 256, 16386)])     # rows not a multiple of 4: the two-kernel route
 def test_matmul_silu_gate(dt, b, s, hidden):
     g = torch.Generator(device="cuda").manual_seed(2)
     x = torch.randn((b, s), generator=g, device="cuda").to(dt)
