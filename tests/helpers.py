@@ -57,3 +57,13 @@ class Arena:
 
     def refresh_host(self):
         self.host = self.dev.cpu().numpy()
+
+
+def half_ulp_diff(a: np.ndarray, b: np.ndarray):
+    """Largest distance in fp16 units in the last place between two float16 arrays, and the fraction of
+    elements that differ at all (both arrays finite)."""
+    def ordered(x):
+        i = np.ascontiguousarray(x).view(np.int16).astype(np.int32)
+        return np.where(i < 0, -32768 - i, i)
+    d = np.abs(ordered(a) - ordered(b))
+    return int(d.max()), float((d > 0).mean())

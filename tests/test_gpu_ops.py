@@ -9,7 +9,7 @@ import torch
 import oracle as O
 from glinthawk_amd import Shape, ops
 from glinthawk_amd._lib import GH_ATTN_AUTO, GH_ATTN_GENERIC, GH_ATTN_MFMA, GH_ATTN_VALU, GlintError
-from helpers import Arena, assert_close, errors, oracle_cfg
+from helpers import half_ulp_diff, Arena, assert_close, errors, oracle_cfg
 
 pytestmark = pytest.mark.gpu
 
@@ -63,6 +63,10 @@ def test_rmsnorm(dt, tol, batch, size):
     got = ops.rmsnorm(dx, dw).cpu().numpy()
     want = O.rmsnorm(x, w)
     np.testing.assert_allclose(got.astype(np.float64), want.astype(np.float64), rtol=tol, atol=tol)
+    if dt == "f16":
+        # against the fp16-storage instantiation: same rounding points, only the order of the sum of squares differs
+        worst, differing = half_ulp_diff(got, want)
+        assert worst <= 1 and differing < 0.01, (worst, differing)
     want32 = O.rmsnorm(x.astype(np.float32), w.astype(np.float32))
     assert_close(got, want32, what="rmsnorm vs fp32 path")
     # in place
@@ -80,6 +84,10 @@ def test_silu(dt, tol, batch, hidden):
     ops.silu(dx, dy)
     O.silu(x, y)
     np.testing.assert_allclose(dx.cpu().numpy().astype(np.float64), x.astype(np.float64), rtol=tol, atol=tol)
+    if dt == "f16":
+        # one rounding per element on both sides; the exponential is the only difference
+        worst, differing = half_ulp_diff(dx.cpu().numpy(), x)
+        assert worst <= 1 and differing < 1e-3, (worst, differing)
 
 
 @pytest.mark.parametrize("dt", ["f16", "f32"])
@@ -298,6 +306,13 @@ def test_rope(dt, tol, shape, host_tables):
     got_cache = arena.dev.cpu().numpy()
     np.testing.assert_allclose(dq.cpu().numpy().astype(np.float64), q.astype(np.float64), rtol=tol, atol=tol)
     np.testing.assert_allclose(got_cache.astype(np.float64), want_cache.astype(np.float64), rtol=tol, atol=tol)
+    if dt == "f16":
+        # fp32 rotation and one rounding on both sides: at most the last bit (fused against separate multiply-add)
+        present_rows = [i for i in range(batch) if present[i]]
+        worst, _ = half_ulp_diff(dq.cpu().numpy()[present_rows], q[present_rows])
+        assert worst <= 1, worst
+        worst, _ = half_ulp_diff(got_cache, want_cache)
+        assert worst <= 1, worst
     # V halves and all other rows are untouched bit for bit
     U = np.uint16 if dt == "f16" else np.uint32
     mask = np.ones(got_cache.shape, bool)
