@@ -9,8 +9,11 @@
 // 16 exactly like the decode kernel (K through a wave-private swizzled LDS tile into
 // v_mfma_f32_16x16x32_f16 operand order, S^T lands in the A-operand order of
 // v_mfma_f32_16x16x16_f16, V transposed in registers), with a per-column causal mask.  The four
-// waves of a block take neighbouring query groups, so they read the same cache rows at about the
-// same time and share them through L2.
+// waves of a block take neighbouring query groups and need almost the same keys: the block streams
+// them once, 64 keys per step into an LDS stage (every wave fetches a quarter, the next step's rows
+// are in flight in registers meanwhile), and each wave works through the four 16-key tiles of the
+// stage that its queries can see.  Four blocks per CU: the per-tile chain of MFMA, softmax and
+// shuffles is latency-bound, so occupancy matters more than the 4 spilled registers it costs.
 //
 // Any other shape: the decode kernels are run on tables expanded to one entry per (context, token).
 #include "gh_common.h"
@@ -20,6 +23,9 @@ namespace {
 
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr int HS = 128;
+#ifndef PF_WGS_PER_CU
+#define PF_WGS_PER_CU 4
+#endif
 
 typedef _Float16 f16x4 __attribute__( ( ext_vector_type( 4 ) ) );
 typedef _Float16 f16x8 __attribute__( ( ext_vector_type( 8 ) ) );
@@ -58,7 +64,7 @@ __global__ __launch_bounds__( 256 ) void expand_tables_kernel( const void* const
 
 // q, xb: (batch * n_tokens, n_kv_heads * G * 128), row index = context * n_tokens + token
 template<int G>
-__global__ __launch_bounds__( 256 ) void attn_prefill_mfma_kernel( const __half* __restrict__ q,
+__global__ __launch_bounds__( 256, PF_WGS_PER_CU ) void attn_prefill_mfma_kernel( const __half* __restrict__ q,
                                                                    const __half* const* __restrict__ layer_rows,
                                                                    const uint32_t* __restrict__ start_pos,
                                                                    __half* __restrict__ xb,
@@ -67,7 +73,8 @@ __global__ __launch_bounds__( 256 ) void attn_prefill_mfma_kernel( const __half*
                                                                    uint32_t groups_per_head, // ceil(n_tokens / (16 / G))
                                                                    float scale_log2e )
 {
-  __shared__ uint4 s_k[4][16 * 16];
+  __shared__ uint4 s_kt[64 * 16]; // 64 keys x 256 bytes, 16-byte chunks XOR-swizzled per 16-key tile
+  __shared__ uint4 s_vt[64 * 16]; // the same keys' value rows, plain
   constexpr uint32_t TPG = 16 / G; // tokens per query group
 
   const uint32_t wave = threadIdx.x >> 6;
@@ -83,22 +90,25 @@ __global__ __launch_bounds__( 256 ) void attn_prefill_mfma_kernel( const __half*
   const uint32_t ctx = bid / n_kv_heads;
   const uint32_t group = quad * 4 + wave;
   const __half* base = layer_rows[ctx];
-  if ( group >= groups_per_head || base == nullptr ) {
-    return; // wave-uniform; only wave-private LDS below, no block barrier
+  if ( base == nullptr ) {
+    return; // the whole work-group
   }
+  const bool wave_ok = group < groups_per_head; // a wave without queries still loads its share of every tile
   const uint32_t n_heads = n_kv_heads * G;
   const uint64_t row_elems = 2ull * n_kv_heads * HS;
   const uint32_t v_off = n_kv_heads * HS;
   const uint32_t start = start_pos[ctx];
-  uint4* tile = s_k[wave];
 
   // this lane's query column: token tq, head gq; invalid beyond n_tokens
   const uint32_t tq = group * TPG + c / G;
   const uint32_t gq = c % G;
-  const bool col_ok = tq < n_tokens;
+  const bool col_ok = wave_ok && tq < n_tokens;
   const int32_t qpos = col_ok ? (int32_t)( start + tq ) : -1; // last visible key of the column
   const uint32_t last_tok = min( n_tokens, ( group + 1 ) * TPG ) - 1;
-  const uint32_t t_end = start + last_tok + 1; // keys [0, t_end) are visible to some column of the group
+  const uint32_t t_end = wave_ok ? start + last_tok + 1 : 0; // keys [0, t_end) are visible to some column of the group
+  // the work-group streams the keys its last group needs; every wave loads a quarter of each 64-key tile
+  const uint32_t last_group = min( groups_per_head, quad * 4 + 4 ) - 1;
+  const uint32_t wg_end = start + min( n_tokens, ( last_group + 1 ) * TPG );
 
   f16x8 qb[4];
   {
@@ -126,86 +136,99 @@ __global__ __launch_bounds__( 256 ) void attn_prefill_mfma_kernel( const __half*
   uint4 kn[4], vn[4];
 #pragma unroll
   for ( int i = 0; i < 4; i++ ) {
-    const uint32_t tok = 4 * g4 + i;
-    const bool ok = tok < t_end;
+    const uint32_t tok = 16 * wave + 4 * g4 + i;
+    const bool ok = tok < wg_end;
     const __half* row = kp + (uint64_t)tok * row_elems;
     kn[i] = ok ? load16( row ) : zero4;
     vn[i] = ok ? load16( row + v_off ) : zero4;
   }
 
-  for ( uint32_t t0 = 0; t0 < t_end; t0 += 16 ) {
-    uint4 vc[4];
-#pragma unroll
-    for ( int i = 0; i < 4; i++ ) {
-      const uint32_t tl = 4 * g4 + i;
-      tile[tl * 16 + ( c ^ tl )] = kn[i];
-      vc[i] = vn[i];
+  for ( uint32_t tile0 = 0; tile0 < wg_end; tile0 += 64 ) {
+    uint4* kt = s_kt;
+    uint4* vt = s_vt;
+    if ( tile0 != 0 ) {
+      __syncthreads(); // every wave is done with the previous tile
     }
 #pragma unroll
     for ( int i = 0; i < 4; i++ ) {
-      const uint32_t tok = t0 + 16 + 4 * g4 + i;
-      const bool ok = tok < t_end;
+      const uint32_t tl = 4 * g4 + i;
+      kt[( 16 * wave + tl ) * 16 + ( c ^ tl )] = kn[i];
+      vt[( 16 * wave + tl ) * 16 + c] = vn[i];
+    }
+#pragma unroll
+    for ( int i = 0; i < 4; i++ ) {
+      const uint32_t tok = tile0 + 64 + 16 * wave + 4 * g4 + i;
+      const bool ok = tok < wg_end;
       const __half* row = kp + (uint64_t)tok * row_elems;
       kn[i] = ok ? load16( row ) : zero4;
       vn[i] = ok ? load16( row + v_off ) : zero4;
     }
-    __builtin_amdgcn_fence( __ATOMIC_RELEASE, "wavefront" );
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence( __ATOMIC_ACQUIRE, "wavefront" );
+    __syncthreads();
 
-    f32x4 st = f32x4 { 0.0f, 0.0f, 0.0f, 0.0f };
-#pragma unroll
-    for ( int kk = 0; kk < 4; kk++ ) {
-      const uint4 kf = tile[c * 16 + ( ( 4 * kk + g4 ) ^ c )];
-      st = __builtin_amdgcn_mfma_f32_16x16x32_f16( __builtin_bit_cast( f16x8, kf ), qb[kk], st, 0, 0, 0 );
-    }
-    __builtin_amdgcn_fence( __ATOMIC_RELEASE, "wavefront" );
-    __builtin_amdgcn_wave_barrier();
-
-    // st[i] = score of key t0 + 4*g4 + i for query column c; causal mask per column
-    float s[4];
-    float mt = -INFINITY;
-#pragma unroll
-    for ( int i = 0; i < 4; i++ ) {
-      const int32_t key = (int32_t)( t0 + 4 * g4 + i );
-      s[i] = key <= qpos ? st[i] * scale_log2e : -INFINITY;
-      mt = fmaxf( mt, s[i] );
-    }
-    mt = fmaxf( mt, __shfl_xor( mt, 16, WAVE ) );
-    mt = fmaxf( mt, __shfl_xor( mt, 32, WAVE ) );
-    const float m_new = fmaxf( m, mt );
-    const float m_safe = m_new == -INFINITY ? 0.0f : m_new; // padding columns never see a key
-    const float alpha = fast_exp2( m - m_safe );
-    float p[4];
-#pragma unroll
-    for ( int i = 0; i < 4; i++ ) {
-      p[i] = fast_exp2( s[i] - m_safe );
-    }
-    l = l * alpha + ( p[0] + p[1] ) + ( p[2] + p[3] );
-    m = m_new;
-
-    if ( __builtin_amdgcn_ballot_w64( alpha != 1.0f ) != 0 ) {
+    for ( uint32_t sub = 0; sub < 4; sub++ ) {
+      const uint32_t t0 = tile0 + 16 * sub;
+      if ( t0 >= t_end ) {
+        break; // wave-uniform: nothing further is visible to this wave's queries
+      }
+      const uint4* tile = kt + 16 * sub * 16;
+      uint4 vc[4];
 #pragma unroll
       for ( int i = 0; i < 4; i++ ) {
-        const float a = __shfl( alpha, (int)( 4 * g4 + i ), WAVE );
+        vc[i] = vt[( 16 * sub + 4 * g4 + i ) * 16 + c];
+      }
+
+      f32x4 st = f32x4 { 0.0f, 0.0f, 0.0f, 0.0f };
 #pragma unroll
-        for ( int nn = 0; nn < 8; nn++ ) {
-          acc[nn][i] *= a;
+      for ( int kk = 0; kk < 4; kk++ ) {
+        const uint4 kf = tile[c * 16 + ( ( 4 * kk + g4 ) ^ c )];
+        st = __builtin_amdgcn_mfma_f32_16x16x32_f16( __builtin_bit_cast( f16x8, kf ), qb[kk], st, 0, 0, 0 );
+      }
+
+      // st[i] = score of key t0 + 4*g4 + i for query column c; causal mask per column
+      float s[4];
+      float mt = -INFINITY;
+#pragma unroll
+      for ( int i = 0; i < 4; i++ ) {
+        const int32_t key = (int32_t)( t0 + 4 * g4 + i );
+        s[i] = key <= qpos ? st[i] * scale_log2e : -INFINITY;
+        mt = fmaxf( mt, s[i] );
+      }
+      mt = fmaxf( mt, __shfl_xor( mt, 16, WAVE ) );
+      mt = fmaxf( mt, __shfl_xor( mt, 32, WAVE ) );
+      const float m_new = fmaxf( m, mt );
+      const float m_safe = m_new == -INFINITY ? 0.0f : m_new; // padding columns never see a key
+      const float alpha = fast_exp2( m - m_safe );
+      float p[4];
+#pragma unroll
+      for ( int i = 0; i < 4; i++ ) {
+        p[i] = fast_exp2( s[i] - m_safe );
+      }
+      l = l * alpha + ( p[0] + p[1] ) + ( p[2] + p[3] );
+      m = m_new;
+
+      if ( __builtin_amdgcn_ballot_w64( alpha != 1.0f ) != 0 ) {
+#pragma unroll
+        for ( int i = 0; i < 4; i++ ) {
+          const float a = __shfl( alpha, (int)( 4 * g4 + i ), WAVE );
+#pragma unroll
+          for ( int nn = 0; nn < 8; nn++ ) {
+            acc[nn][i] *= a;
+          }
         }
       }
-    }
 
-    const f16x4 pa = f16x4 { (_Float16)p[0], (_Float16)p[1], (_Float16)p[2], (_Float16)p[3] };
-    const uint32_t vw[4][4] = { { vc[0].x, vc[0].y, vc[0].z, vc[0].w },
-                                { vc[1].x, vc[1].y, vc[1].z, vc[1].w },
-                                { vc[2].x, vc[2].y, vc[2].z, vc[2].w },
-                                { vc[3].x, vc[3].y, vc[3].z, vc[3].w } };
+      const f16x4 pa = f16x4 { (_Float16)p[0], (_Float16)p[1], (_Float16)p[2], (_Float16)p[3] };
+      const uint32_t vw[4][4] = { { vc[0].x, vc[0].y, vc[0].z, vc[0].w },
+                                  { vc[1].x, vc[1].y, vc[1].z, vc[1].w },
+                                  { vc[2].x, vc[2].y, vc[2].z, vc[2].w },
+                                  { vc[3].x, vc[3].y, vc[3].z, vc[3].w } };
 #pragma unroll
-    for ( int w = 0; w < 4; w++ ) {
-      const uint2 lo = make_uint2( __builtin_amdgcn_perm( vw[1][w], vw[0][w], 0x05040100u ), __builtin_amdgcn_perm( vw[3][w], vw[2][w], 0x05040100u ) );
-      const uint2 hi = make_uint2( __builtin_amdgcn_perm( vw[1][w], vw[0][w], 0x07060302u ), __builtin_amdgcn_perm( vw[3][w], vw[2][w], 0x07060302u ) );
-      acc[2 * w] = __builtin_amdgcn_mfma_f32_16x16x16f16( pa, __builtin_bit_cast( f16x4, lo ), acc[2 * w], 0, 0, 0 );
-      acc[2 * w + 1] = __builtin_amdgcn_mfma_f32_16x16x16f16( pa, __builtin_bit_cast( f16x4, hi ), acc[2 * w + 1], 0, 0, 0 );
+      for ( int w = 0; w < 4; w++ ) {
+        const uint2 lo = make_uint2( __builtin_amdgcn_perm( vw[1][w], vw[0][w], 0x05040100u ), __builtin_amdgcn_perm( vw[3][w], vw[2][w], 0x05040100u ) );
+        const uint2 hi = make_uint2( __builtin_amdgcn_perm( vw[1][w], vw[0][w], 0x07060302u ), __builtin_amdgcn_perm( vw[3][w], vw[2][w], 0x07060302u ) );
+        acc[2 * w] = __builtin_amdgcn_mfma_f32_16x16x16f16( pa, __builtin_bit_cast( f16x4, lo ), acc[2 * w], 0, 0, 0 );
+        acc[2 * w + 1] = __builtin_amdgcn_mfma_f32_16x16x16f16( pa, __builtin_bit_cast( f16x4, hi ), acc[2 * w + 1], 0, 0, 0 );
+      }
     }
   }
 

@@ -130,8 +130,8 @@ int gh_silu( void* hb, const void* hb2, uint64_t hidden_dim, uint64_t batch, gh_
 int gh_argmax( uint32_t* out_host, uint32_t* out_dev, const void* v, uint64_t n, uint64_t batch, gh_dtype dt, gh_stream stream );
 /* Operations::matmul<s,r> / untemplated_matmul  arch/amd64/common/ops.hh:74-93,212-271 :
  * xout(b, r) = sum_p w(r, p) * x(b, p); w row-major (r, s); fp32 accumulate */
-/* tuning hook: kernel 0 auto / 1 small tiled / 2 streaming (decode) / 3 128x128 tile / 4 256x256 tile (many rows); target number of work-groups for the K split
- * (<= 0 keeps the current value); prefetch depth 2..4 of the streaming kernel (other values keep it) */
+/* tuning hook: kernel 0 auto / 1 small tiled / 2 streaming (decode) / 3 128x128 tile / 4 256x256 tile (many rows); the number of compute units the
+ * streaming kernel's K split is balanced for (<= 0 keeps the current value; the default is the device's own count); the third argument is ignored */
 int gh_gemm_set_tuning( int kernel, int target_workgroups, int depth );
 int gh_matmul( void* xout, const void* x, const void* w, uint64_t s, uint64_t r, uint64_t b, gh_dtype dt, gh_stream stream );
 /* A projection fused with the ops that follow it in the reference's layer; same arithmetic and the
