@@ -364,6 +364,14 @@ int gh_gemm_set_tuning( int kernel, int target_workgroups, int depth )
   return GH_OK;
 }
 
+int gh_gemm_stream_plan( uint64_t s, uint64_t r, uint64_t b, uint32_t* splits, uint32_t* k_per_split, uint32_t* rows_per_workgroup )
+{
+  GH_REQUIRE( splits && k_per_split && rows_per_workgroup, "gh_gemm_stream_plan: NULL output" );
+  GH_REQUIRE( s >= 256 && s % 256 == 0 && r > 0 && b > 0, "gh_gemm_stream_plan: the streaming kernel takes s %% 256 == 0, r > 0, b > 0" );
+  gemm_stream_plan( s, r, b, splits, k_per_split, rows_per_workgroup );
+  return GH_OK;
+}
+
 int gh_matmul( void* xout, const void* x, const void* w, uint64_t s, uint64_t r, uint64_t b, gh_dtype dt, gh_stream stream )
 {
   if ( int rc = ensure_init() ) {

@@ -133,6 +133,9 @@ int gh_argmax( uint32_t* out_host, uint32_t* out_dev, const void* v, uint64_t n,
 /* tuning hook: kernel 0 auto / 1 small tiled / 2 streaming (decode) / 3 128x128 tile / 4 256x256 tile (many rows); the number of compute units the
  * streaming kernel's K split is balanced for (<= 0 keeps the current value; the default is the device's own count); the third argument is ignored */
 int gh_gemm_set_tuning( int kernel, int target_workgroups, int depth );
+/* host-only query: how the weight-streaming kernel would cut an (r x s) . (b x s)^T product for the initialised device (256 compute
+ * units before initialisation): number of K ranges, k per range (a multiple of 256), weight rows per work-group */
+int gh_gemm_stream_plan( uint64_t s, uint64_t r, uint64_t b, uint32_t* splits, uint32_t* k_per_split, uint32_t* rows_per_workgroup );
 int gh_matmul( void* xout, const void* x, const void* w, uint64_t s, uint64_t r, uint64_t b, gh_dtype dt, gh_stream stream );
 /* A projection fused with the ops that follow it in the reference's layer; same arithmetic and the
  * same rounding points as the separate calls (every matmul result is rounded to DType first).
