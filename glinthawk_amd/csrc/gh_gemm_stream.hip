@@ -110,7 +110,7 @@ __device__ __forceinline__ void half_mfma( f32x16 acc[2], const uint4* wtile, co
 {
   const uint32_t lane = threadIdx.x & 63;
   const uint32_t r = lane & 31, g2 = lane >> 5;
-#pragma unroll 2
+#pragma unroll
   for ( int s = 0; s < 8; s++ ) {
     const uint32_t ch = 2 * s + g2;
     const f16x8 a = __builtin_bit_cast( f16x8, wtile[r * 16 + ( ch ^ ( r & 15 ) )] );
