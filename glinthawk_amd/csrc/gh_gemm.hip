@@ -282,7 +282,7 @@ int gemm_partials( void* xout, const void* x, const void* w, uint64_t s, uint64_
     }
     return gemm_tile256_launch( static_cast<__half*>( xout ), ws, static_cast<const __half*>( x ), static_cast<const __half*>( w ), s, r, b, st );
   }
-  GH_REQUIRE( g_force_kernel != 4, "gh_matmul: the 256 x 256 tile kernel needs b >= 192, at least 192 tiles (1024 when s < 8192), s %% 64 == 0 and 16-byte aligned operands" );
+  GH_REQUIRE( g_force_kernel != 4, "gh_matmul: the 256 x 256 tile kernel needs b >= 192, at least 192 tiles with a last round that is not mostly empty, s %% 64 == 0 and 16-byte aligned operands" );
   if ( ( g_force_kernel == 0 || g_force_kernel == 3 ) && gemm_tile_applicable( s, r, b, x, w, xout ? xout : x ) ) {
     uint32_t splits = 1, k_per_split = 0;
     gemm_tile_plan( s, r, b, &splits, &k_per_split );
