@@ -139,13 +139,17 @@ __global__ __launch_bounds__( T256_THREADS, 1 ) void gemm_tile256_kernel( __half
   for ( uint32_t j = 0; j < n_steps; j++ ) {
     const uint4* wt = s_w[j & 1];
     const uint4* xt = s_x[j & 1];
+    __builtin_amdgcn_s_setprio( 1 );
     mfma_k16( wt, xt, 0 );
     mfma_k16( wt, xt, 1 );
+    __builtin_amdgcn_s_setprio( 0 );
     stage( ( j & 1 ) ^ 1 );
     load8( wreg, w_rsrc, voff, ld_bytes, ( j + 2 ) * TKS * 2 );
     load8( xreg, x_rsrc, voff, ld_bytes, ( j + 2 ) * TKS * 2 );
+    __builtin_amdgcn_s_setprio( 1 );
     mfma_k16( wt, xt, 2 );
     mfma_k16( wt, xt, 3 );
+    __builtin_amdgcn_s_setprio( 0 );
     __syncthreads();
   }
   // acc[rt][t][v]: row = tile_row0 + 64*wr + 32*rt + 8*(v/4) + 4*(lane/32) + v%4, token = tile_col0 + 128*wc + 32*t + lane%32
