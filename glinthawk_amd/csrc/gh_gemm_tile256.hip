@@ -7,13 +7,15 @@
 //                 2 x 4 accumulators of v_mfma_f32_32x32x16_f16 (128 registers), two waves per SIMD.
 //                 With one wave per SIMD (four waves of 64 x 256, the first version of this kernel)
 //                 every stall of a memory or LDS instruction also holds back that wave's MFMAs:
-//                 0.82-0.97 PFLOP/s however the operands were fetched; two waves per SIMD: 0.9-1.03.
+//                 0.82-0.97 PFLOP/s however the operands were fetched; two waves per SIMD: 0.9-1.08.
 //   operands    both go global -> registers (one 64-k step ahead, coalesced 128-byte row segments,
 //                 four 16-byte loads per thread and operand) -> LDS (two stages, XOR-swizzled
 //                 16-byte chunks, no bank conflicts) -> MFMA operands
 //   schedule    step j multiplies out of stage j % 2; in the middle of its MFMAs the registers that
 //                 hold step j + 1 are written to the other stage and the loads of step j + 2 go
-//                 out, so the matrix pipe works through the copy; one barrier per step
+//                 out, so the matrix pipe works through the copy; one barrier per step; the wave's
+//                 priority is raised while it issues MFMAs, so that of two waves on a SIMD the one
+//                 with matrix work goes first
 //   tile order  as in the 128 x 128 kernel: each XCD owns every 8th row tile and walks patches of
 //                 tiles that are resident together
 #include "gh_common.h"
