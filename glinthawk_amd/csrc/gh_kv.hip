@@ -74,6 +74,85 @@ __global__ __launch_bounds__( 256 ) void rope_kernel( const uint32_t* __restrict
   }
 }
 
+// The same for f16 with 16-byte accesses: thread <-> (kv head j, four pairs 4m .. 4m+3).  Used when the head
+// size is a multiple of 8 and q and the tables are aligned; a cache row that is not 16-byte aligned
+// makes its block take two-byte accesses (same arithmetic, same rounding).
+__global__ __launch_bounds__( 256 ) void rope_f16x8_kernel( const uint32_t* __restrict__ pos,
+                                                            const __half* __restrict__ freq_real,
+                                                            const __half* __restrict__ freq_imag,
+                                                            __half* __restrict__ q,
+                                                            void* const* __restrict__ rows,
+                                                            uint32_t n_kv_heads,
+                                                            uint32_t gqa,
+                                                            uint32_t head_size )
+{
+  const uint32_t ctx = blockIdx.y;
+  __half* krow = static_cast<__half*>( rows[ctx] );
+  if ( krow == nullptr ) {
+    return;
+  }
+  const uint32_t half = head_size / 2;
+  const uint32_t groups = head_size / 8; // groups of four pairs per head
+  const uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if ( idx >= n_kv_heads * groups ) {
+    return;
+  }
+  const uint32_t j = idx / groups;
+  const uint32_t m = idx % groups;
+  const uint64_t p = pos[ctx];
+  union H4
+  {
+    uint2 raw;
+    __half h[4];
+  };
+  union H8
+  {
+    uint4 raw;
+    __half h[8];
+  };
+  H4 fr, fi;
+  fr.raw = *reinterpret_cast<const uint2*>( freq_real + p * half + 4 * m );
+  fi.raw = *reinterpret_cast<const uint2*>( freq_imag + p * half + 4 * m );
+  float c[4], sn[4];
+#pragma unroll
+  for ( int e = 0; e < 4; e++ ) {
+    c[e] = __half2float( fr.h[e] );
+    sn[e] = __half2float( fi.h[e] );
+  }
+  auto rotate = [&]( H8& v ) {
+#pragma unroll
+    for ( int e = 0; e < 4; e++ ) {
+      const float x0 = __half2float( v.h[2 * e] );
+      const float x1 = __half2float( v.h[2 * e + 1] );
+      v.h[2 * e] = __float2half_rn( x0 * c[e] - x1 * sn[e] );
+      v.h[2 * e + 1] = __float2half_rn( x0 * sn[e] + x1 * c[e] );
+    }
+  };
+  __half* kp = krow + (uint64_t)j * head_size + 8 * m;
+  H8 v;
+  if ( ( reinterpret_cast<uintptr_t>( krow ) & 15u ) == 0 ) { // uniform across the block
+    v.raw = *reinterpret_cast<const uint4*>( kp );
+    rotate( v );
+    *reinterpret_cast<uint4*>( kp ) = v.raw;
+  } else {
+#pragma unroll
+    for ( int e = 0; e < 8; e++ ) {
+      v.h[e] = kp[e];
+    }
+    rotate( v );
+#pragma unroll
+    for ( int e = 0; e < 8; e++ ) {
+      kp[e] = v.h[e];
+    }
+  }
+  __half* qp = q + (uint64_t)ctx * n_kv_heads * gqa * head_size + (uint64_t)j * gqa * head_size + 8 * m;
+  for ( uint32_t g = 0; g < gqa; g++ ) {
+    v.raw = *reinterpret_cast<const uint4*>( qp + g * head_size );
+    rotate( v );
+    *reinterpret_cast<uint4*>( qp + g * head_size ) = v.raw;
+  }
+}
+
 } // namespace
 } // namespace gh
 
@@ -133,7 +212,14 @@ int gh_rope( uint64_t batch, const uint32_t* pos_dev, const void* freq_real, con
   GH_REQUIRE( head_size % 2 == 0 && head_size > 0 && n_kv_heads > 0 && gqa_size > 0 && batch <= 65535, "gh_rope: bad shape" );
   const unsigned threads = n_kv_heads * ( head_size / 2 );
   const dim3 grid( ( threads + 255 ) / 256, (unsigned)batch );
-  if ( dt == GH_F16 ) {
+  const bool vec_ok = dt == GH_F16 && head_size % 8 == 0 && ( reinterpret_cast<uintptr_t>( q ) & 15u ) == 0
+                      && ( ( reinterpret_cast<uintptr_t>( freq_real ) | reinterpret_cast<uintptr_t>( freq_imag ) ) & 7u ) == 0;
+  if ( vec_ok ) {
+    const unsigned vthreads = n_kv_heads * ( head_size / 8 );
+    const dim3 vgrid( ( vthreads + 255 ) / 256, (unsigned)batch );
+    rope_f16x8_kernel<<<vgrid, 256, 0, as_stream( stream )>>>( pos_dev, static_cast<const __half*>( freq_real ), static_cast<const __half*>( freq_imag ),
+                                                             static_cast<__half*>( q ), token_rows_dev, n_kv_heads, gqa_size, head_size );
+  } else if ( dt == GH_F16 ) {
     rope_kernel<__half><<<grid, 256, 0, as_stream( stream )>>>( pos_dev, static_cast<const __half*>( freq_real ), static_cast<const __half*>( freq_imag ),
                                                               static_cast<__half*>( q ), token_rows_dev, n_kv_heads, gqa_size, head_size );
   } else if ( dt == GH_F32 ) {
