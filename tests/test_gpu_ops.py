@@ -322,6 +322,30 @@ def test_rope(dt, tol, shape, host_tables):
     assert np.array_equal(got_cache.view(U)[mask], arena.host.view(U)[mask])
 
 
+def test_rope_cache_row_not_16_byte_aligned():
+    """The f16 kernel takes 16-byte accesses when it can; a cache row at an odd element offset has to come out the same."""
+    shape = GQA8
+    re32, im32 = O.rope_tables(shape.seq_len, shape.head_size)
+    re, im = re32.astype(np.float16), im32.astype(np.float16)
+    rng = np.random.default_rng(21)
+    q = rng.standard_normal((2, shape.dim)).astype(np.float16)
+    rows = rng.standard_normal((2, 2 * shape.kv_dim + 8)).astype(np.float16)
+    drows = torch.from_numpy(rows).cuda()
+    dq = torch.from_numpy(q).cuda()
+    pos = [7, shape.seq_len - 1]
+    ptrs = [drows[0].data_ptr() + 2, drows[1].data_ptr()]          # first row starts one element in
+    ops.rope(torch.tensor(pos, dtype=torch.int32, device="cuda"), torch.from_numpy(re).cuda(), torch.from_numpy(im).cuda(), dq, ops.row_table(ptrs), shape)
+    want_rows = [rows[0, 1:1 + 2 * shape.kv_dim].copy(), rows[1, :2 * shape.kv_dim].copy()]
+    O.apply_rope(oracle_cfg(shape), pos, re, im, q, want_rows)
+    got = drows.cpu().numpy()
+    assert half_ulp_diff(got[0, 1:1 + 2 * shape.kv_dim], want_rows[0])[0] <= 1
+    assert half_ulp_diff(got[1, :2 * shape.kv_dim], want_rows[1])[0] <= 1
+    assert half_ulp_diff(dq.cpu().numpy(), q)[0] <= 1
+    # nothing outside the K halves moved
+    assert np.array_equal(got[0, :1], rows[0, :1]) and np.array_equal(got[0, 1 + shape.kv_dim:], rows[0, 1 + shape.kv_dim:])
+    assert np.array_equal(got[1, shape.kv_dim:], rows[1, shape.kv_dim:])
+
+
 # ------------------------------------------------------------------ unfused attention ops
 @pytest.mark.parametrize("dt", ["f16", "f32"])
 @pytest.mark.parametrize("shape", [TINY, STORIES, GQA8], ids=["tiny", "stories15m", "gqa8"])
