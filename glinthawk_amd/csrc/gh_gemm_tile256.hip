@@ -7,15 +7,22 @@
 //                 2 x 4 accumulators of v_mfma_f32_32x32x16_f16 (128 registers), two waves per SIMD.
 //                 With one wave per SIMD (four waves of 64 x 256, the first version of this kernel)
 //                 every stall of a memory or LDS instruction also holds back that wave's MFMAs:
-//                 0.82-0.97 PFLOP/s however the operands were fetched; two waves per SIMD: 0.9-1.08.
-//   operands    both go global -> registers (one 64-k step ahead, coalesced 128-byte row segments,
-//                 four 16-byte loads per thread and operand) -> LDS (two stages, XOR-swizzled
-//                 16-byte chunks, no bank conflicts) -> MFMA operands
-//   schedule    step j multiplies out of stage j % 2; in the middle of its MFMAs the registers that
-//                 hold step j + 1 are written to the other stage and the loads of step j + 2 go
-//                 out, so the matrix pipe works through the copy; one barrier per step; the wave's
-//                 priority is raised while it issues MFMAs, so that of two waves on a SIMD the one
-//                 with matrix work goes first
+//                 0.82-0.97 PFLOP/s however the operands were fetched.
+//   operands    both go global -> LDS without passing through registers (`buffer_load ... lds`, 16
+//                 bytes per lane: a wave's instruction writes 1 KiB of LDS, lane l at + 16 l, so the
+//                 XOR swizzle that keeps the MFMA reads free of bank conflicts is applied to the
+//                 global address each lane fetches) -> MFMA operands; two 64-k stages
+//   schedule    step j multiplies out of stage j % 2 while the loads of step j + 1 fill the other
+//                 stage; the barrier that ends the step waits for them.  The fragments of the next
+//                 16 k are read from LDS before the MFMAs of the current 16 k are issued; the
+//                 wave's priority is raised while it issues MFMAs, so that of two waves on a SIMD
+//                 the one with matrix work goes first.  Against staging through registers (loads
+//                 one step ahead, ds_write in the middle of the MFMAs): 1.02 -> 1.15 PFLOP/s at
+//                 16384 x 8192 x 57344.
+//   what binds  with the loads taken out the loop runs at 1.8-2.1 PFLOP/s (2.1-2.3 without the
+//                 barrier as well); with every work-group reading the same L2-resident tile at
+//                 1.2: a step's 64 KiB arrive at about 16 bytes per clock and CU from L2, however
+//                 they are addressed, and that, not the matrix pipe or LDS, sets the step time.
 //   tile order  as in the 128 x 128 kernel: each XCD owns every 8th row tile and walks patches of
 //                 tiles that are resident together
 #include "gh_common.h"
@@ -26,6 +33,7 @@ namespace gh {
 
 typedef _Float16 f16x8 __attribute__( ( ext_vector_type( 8 ) ) );
 typedef float f32x16 __attribute__( ( ext_vector_type( 16 ) ) );
+typedef __attribute__( ( address_space( 3 ) ) ) void* lds_ptr;
 
 namespace {
 
@@ -33,10 +41,6 @@ constexpr int TM2 = 256; // weight rows per work-group: 4 waves x 64
 constexpr int TN2 = 256; // tokens per work-group
 constexpr int TKS = 64;  // k per step
 
-__device__ __forceinline__ uint4 bload( __amdgpu_buffer_rsrc_t rsrc, uint32_t voff, uint32_t soff )
-{
-  return __builtin_bit_cast( uint4, __builtin_amdgcn_raw_buffer_load_b128( rsrc, voff, soff, 0 ) );
-}
 __device__ __forceinline__ uint32_t swz( uint32_t row, uint32_t chunk ) { return row * 8 + ( chunk ^ ( ( row >> 1 ) & 7 ) ); }
 
 struct TileOrder
@@ -45,19 +49,6 @@ struct TileOrder
 };
 
 constexpr int T256_THREADS = 512;
-
-struct Step8
-{
-  uint4 v[4]; // thread t: row t/8 + 64*i, chunk t%8
-};
-
-__device__ __forceinline__ void load8( Step8& d, __amdgpu_buffer_rsrc_t rsrc, uint32_t voff, uint32_t ld_bytes, uint32_t kb )
-{
-#pragma unroll
-  for ( int i = 0; i < 4; i++ ) {
-    d.v[i] = bload( rsrc, voff, 64 * i * ld_bytes + kb );
-  }
-}
 
 // grid: 8 * padded tiles per XCD.  s % 64 == 0, 16-byte aligned operands.  PARTIAL: fp32 (1, b, r) instead of xout.
 template<bool PARTIAL>
@@ -70,8 +61,10 @@ __global__ __launch_bounds__( T256_THREADS, 1 ) void gemm_tile256_kernel( __half
                                                                         uint32_t b,
                                                                         TileOrder ord )
 {
-  __shared__ uint4 s_x[2][TN2 * 8]; // 2 x 32 KiB
-  __shared__ uint4 s_w[2][TM2 * 8]; // 2 x 32 KiB
+  // Four separate arrays, not [2][...]: the compiler orders an LDS read behind an outstanding
+  // load-to-LDS only when it cannot tell their arrays apart.
+  __shared__ uint4 s_x0[TN2 * 8], s_x1[TN2 * 8]; // 2 x 32 KiB
+  __shared__ uint4 s_w0[TM2 * 8], s_w1[TM2 * 8]; // 2 x 32 KiB
   const uint32_t xcd = blockIdx.x & 7;
   const uint32_t idx = blockIdx.x >> 3;
   const uint32_t per_patch = ord.gm * ord.gn;
@@ -92,7 +85,10 @@ __global__ __launch_bounds__( T256_THREADS, 1 ) void gemm_tile256_kernel( __half
   const uint32_t x_cols = min( (uint32_t)TN2, b - tile_col0 );
   const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc( const_cast<__half*>( w + (uint64_t)tile_row0 * s ), 0, (int)( w_rows * ld_bytes ), 0x00020000 );
   const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc( const_cast<__half*>( x + (uint64_t)tile_col0 * s ), 0, (int)( x_cols * ld_bytes ), 0x00020000 );
-  const uint32_t voff = ( threadIdx.x >> 3 ) * ld_bytes + ( threadIdx.x & 7 ) * 16;
+  // A load-to-LDS writes lane l of a wave to (wave's base) + 16 l: thread t fills slot t % 8 of row
+  // t / 8 (+ 64 i), so it fetches the chunk that the swizzle keeps in that slot.
+  const uint32_t voff = ( threadIdx.x >> 3 ) * ld_bytes + ( ( threadIdx.x & 7 ) ^ ( ( threadIdx.x >> 4 ) & 7 ) ) * 16;
+  const uint32_t wave_slot0 = 8 * wave * 8; // first uint4 of the wave's 8 rows
 
   f32x16 acc[2][4];
 #pragma unroll
@@ -106,53 +102,68 @@ __global__ __launch_bounds__( T256_THREADS, 1 ) void gemm_tile256_kernel( __half
     }
   }
   const uint32_t n_steps = s / TKS;
-  Step8 wreg, xreg;
   const uint32_t fr = lane & 31, g2 = lane >> 5;
-  auto stage = [&]( uint32_t p ) { // registers -> LDS stage p
+  auto fetch = [&]( uint4* wt, uint4* xt, uint32_t kb ) { // global -> LDS stage, 8 x 1 KiB per wave
 #pragma unroll
     for ( int i = 0; i < 4; i++ ) {
-      const uint32_t row = ( threadIdx.x >> 3 ) + 64 * i;
-      s_w[p][swz( row, threadIdx.x & 7 )] = wreg.v[i];
-      s_x[p][swz( row, threadIdx.x & 7 )] = xreg.v[i];
+      __builtin_amdgcn_raw_ptr_buffer_load_lds( w_rsrc, (lds_ptr)( wt + wave_slot0 + 64 * i * 8 ), 16, voff, 64 * i * ld_bytes + kb, 0, 0 );
+      __builtin_amdgcn_raw_ptr_buffer_load_lds( x_rsrc, (lds_ptr)( xt + wave_slot0 + 64 * i * 8 ), 16, voff, 64 * i * ld_bytes + kb, 0, 0 );
     }
   };
-  auto mfma_k16 = [&]( const uint4* wt, const uint4* xt, int kk ) {
+  struct Frags
+  {
+    f16x8 a[2], bb[4];
+  };
+  auto read_k16 = [&]( Frags& f, const uint4* wt, const uint4* xt, int kk ) {
     const uint32_t ch = 2 * kk + g2;
-    const f16x8 a0 = __builtin_bit_cast( f16x8, wt[swz( 64 * wr + fr, ch )] );
-    const f16x8 a1 = __builtin_bit_cast( f16x8, wt[swz( 64 * wr + 32 + fr, ch )] );
+    f.a[0] = __builtin_bit_cast( f16x8, wt[swz( 64 * wr + fr, ch )] );
+    f.a[1] = __builtin_bit_cast( f16x8, wt[swz( 64 * wr + 32 + fr, ch )] );
 #pragma unroll
     for ( int t = 0; t < 4; t++ ) {
-      const f16x8 bb = __builtin_bit_cast( f16x8, xt[swz( 128 * wc + 32 * t + fr, ch )] );
-      acc[0][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16( a0, bb, acc[0][t], 0, 0, 0 );
-      acc[1][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16( a1, bb, acc[1][t], 0, 0, 0 );
+      f.bb[t] = __builtin_bit_cast( f16x8, xt[swz( 128 * wc + 32 * t + fr, ch )] );
     }
   };
-  load8( wreg, w_rsrc, voff, ld_bytes, 0 );
-  load8( xreg, x_rsrc, voff, ld_bytes, 0 );
-  stage( 0 );
-  load8( wreg, w_rsrc, voff, ld_bytes, TKS * 2 );
-  load8( xreg, x_rsrc, voff, ld_bytes, TKS * 2 );
-  __syncthreads();
-  // Step j computes out of stage j % 2 while the registers that hold step j + 1 are written to the
-  // other stage in the middle of its MFMAs (that stage was last read in step j - 1, behind a
-  // barrier) and the loads of step j + 2 go out: the matrix pipe keeps working through the copy.
-  // The loads behind the last step read the start of the next rows (bounded by the descriptors);
-  // what they bring is staged but never multiplied.
-  for ( uint32_t j = 0; j < n_steps; j++ ) {
-    const uint4* wt = s_w[j & 1];
-    const uint4* xt = s_x[j & 1];
+  auto mfma_k16 = [&]( const Frags& f ) {
+#pragma unroll
+    for ( int t = 0; t < 4; t++ ) {
+      acc[0][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16( f.a[0], f.bb[t], acc[0][t], 0, 0, 0 );
+      acc[1][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16( f.a[1], f.bb[t], acc[1][t], 0, 0, 0 );
+    }
+  };
+  // Step j multiplies out of stage j % 2 while the memory unit writes step j + 1 straight into the
+  // other stage (last read in step j - 1, behind a barrier); the barrier that ends the step also
+  // waits for those loads.  The loads behind the last step read the start of the next rows (bounded
+  // by the descriptors); what they bring is never multiplied.
+  auto step = [&]( const uint4* wt, const uint4* xt, uint4* wn, uint4* xn, uint32_t j ) {
+    Frags f0, f1;
+    read_k16( f0, wt, xt, 0 );
+    fetch( wn, xn, ( j + 1 ) * TKS * 2 );
+    read_k16( f1, wt, xt, 1 );
     __builtin_amdgcn_s_setprio( 1 );
-    mfma_k16( wt, xt, 0 );
-    mfma_k16( wt, xt, 1 );
+    mfma_k16( f0 );
     __builtin_amdgcn_s_setprio( 0 );
-    stage( ( j & 1 ) ^ 1 );
-    load8( wreg, w_rsrc, voff, ld_bytes, ( j + 2 ) * TKS * 2 );
-    load8( xreg, x_rsrc, voff, ld_bytes, ( j + 2 ) * TKS * 2 );
+    read_k16( f0, wt, xt, 2 );
     __builtin_amdgcn_s_setprio( 1 );
-    mfma_k16( wt, xt, 2 );
-    mfma_k16( wt, xt, 3 );
+    mfma_k16( f1 );
+    __builtin_amdgcn_s_setprio( 0 );
+    read_k16( f1, wt, xt, 3 );
+    __builtin_amdgcn_s_setprio( 1 );
+    mfma_k16( f0 );
+    mfma_k16( f1 );
     __builtin_amdgcn_s_setprio( 0 );
     __syncthreads();
+  };
+  fetch( s_w0, s_x0, 0 );
+  __syncthreads();
+  for ( uint32_t j = 0;; ) {
+    step( s_w0, s_x0, s_w1, s_x1, j );
+    if ( ++j == n_steps ) {
+      break;
+    }
+    step( s_w1, s_x1, s_w0, s_x0, j );
+    if ( ++j == n_steps ) {
+      break;
+    }
   }
   // acc[rt][t][v]: row = tile_row0 + 64*wr + 32*rt + 8*(v/4) + 4*(lane/32) + v%4, token = tile_col0 + 128*wc + 32*t + lane%32
 #pragma unroll
