@@ -26,6 +26,7 @@ int gemm_stream_gate_launch( __half* hb, const __half* x, const __half* w13, uin
 // 256 x 256 tile kernel for products with enough tiles (gh_gemm_tile256.hip)
 bool gemm_tile256_applicable( uint64_t s, uint64_t r, uint64_t b, const void* x, const void* w, const void* xout );
 int gemm_tile256_launch( __half* xout, float* partial, const __half* x, const __half* w, uint64_t s, uint64_t r, uint64_t b, hipStream_t st );
+void gemm_tile256_tuning( int rows );
 // large-batch (prefill) kernel (gh_gemm_tile.hip)
 bool gemm_tile_applicable( uint64_t s, uint64_t r, uint64_t b, const void* x, const void* w, const void* xout );
 void gemm_tile_plan( uint64_t s, uint64_t r, uint64_t b, uint32_t* splits_out, uint32_t* k_per_split_out );
@@ -357,10 +358,11 @@ using namespace gh;
 
 extern "C" {
 
-int gh_gemm_set_tuning( int kernel, int target_workgroups, int depth )
+int gh_gemm_set_tuning( int kernel, int target_workgroups, int tile_rows )
 {
   g_force_kernel = kernel;
-  gemm_stream_tuning( target_workgroups, depth );
+  gemm_stream_tuning( target_workgroups, 0 );
+  gemm_tile256_tuning( tile_rows );
   return GH_OK;
 }
 

@@ -1,13 +1,18 @@
-// Second MFMA-bound GEMM for many activation rows: a 256 x 256 output tile per work-group, i.e. per
-// CU, for products with enough such tiles to fill the chip.  A 256 x 256 tile needs half the operand
-// bytes per flop of a 128 x 128 one, and what limits a tile GEMM on this part is the CU's vector
-// memory path, not HBM or the matrix pipes.
+// Second MFMA-bound GEMM for many activation rows: a 256 x 256 or 384 x 256 (weight rows x tokens)
+// output tile per work-group, i.e. per CU, for products with enough such tiles to fill the chip.  A
+// 256 x 256 tile needs half the operand bytes per flop of a 128 x 128 one, and what limits a tile GEMM
+// on this part is the path from L2 into the CU, not HBM or the matrix pipes.
 //
-//   work-group  = 8 waves = 4 row groups x 2 token groups; a wave owns 64 weight rows x 128 tokens:
-//                 2 x 4 accumulators of v_mfma_f32_32x32x16_f16 (128 registers), two waves per SIMD.
+//   work-group  = 8 waves = 4 row groups x 2 token groups; a wave owns 64 or 96 weight rows x 128
+//                 tokens: 2 or 3 x 4 accumulators of v_mfma_f32_32x32x16_f16 (128 or 192 registers),
+//                 two waves per SIMD.
 //                 With one wave per SIMD (four waves of 64 x 256, the first version of this kernel)
 //                 every stall of a memory or LDS instruction also holds back that wave's MFMAs:
 //                 0.82-0.97 PFLOP/s however the operands were fetched.
+//   384 rows    bring 80 KiB per 64 k for 1.5 x the flops of 256 rows (64 KiB) and fill the LDS
+//                 (2 x 80 KiB) and the registers (one set of MFMA operands instead of two); a round
+//                 of them takes 1.32-1.49 x as long, so they win where their rounds fit the shape
+//                 at least as well (tile256_rows() below)
 //   operands    both go global -> LDS without passing through registers (`buffer_load ... lds`, 16
 //                 bytes per lane: a wave's instruction writes 1 KiB of LDS, lane l at + 16 l, so the
 //                 XOR swizzle that keeps the MFMA reads free of bank conflicts is applied to the
@@ -59,7 +64,8 @@ struct TileOrder
 constexpr int T256_THREADS = 512;
 
 // grid: 8 x (padded tiles of one XCD).  s % 64 == 0, 16-byte aligned operands.  PARTIAL: fp32 (1, b, r) instead of xout.
-template<bool PARTIAL>
+// NA: 32-row accumulator tiles per wave, 2 (256 weight rows per work-group) or 3 (384).
+template<bool PARTIAL, int NA>
 __global__ __launch_bounds__( T256_THREADS, 1 ) void gemm_tile256_kernel( __half* __restrict__ xout,
                                                                         float* __restrict__ partial,
                                                                         const __half* __restrict__ x,
@@ -71,8 +77,9 @@ __global__ __launch_bounds__( T256_THREADS, 1 ) void gemm_tile256_kernel( __half
 {
   // Four separate arrays, not [2][...]: the compiler orders an LDS read behind an outstanding
   // load-to-LDS only when it cannot tell their arrays apart.
+  constexpr int TM = 128 * NA; // weight rows per work-group: 4 waves x NA x 32
   __shared__ uint4 s_x0[TN2 * 8], s_x1[TN2 * 8]; // 2 x 32 KiB
-  __shared__ uint4 s_w0[TM2 * 8], s_w1[TM2 * 8]; // 2 x 32 KiB
+  __shared__ uint4 s_w0[TM * 8], s_w1[TM * 8];   // 2 x 32 KiB, or 2 x 48 KiB: all 160 KiB of the CU
   const uint32_t xcd = blockIdx.x & 7; // work-groups go to the XCDs in turn
   const uint32_t idx = blockIdx.x >> 3;
   uint32_t row_tile, token_tile;
@@ -101,10 +108,10 @@ __global__ __launch_bounds__( T256_THREADS, 1 ) void gemm_tile256_kernel( __half
   const uint32_t wave = __builtin_amdgcn_readfirstlane( threadIdx.x >> 6 );
   const uint32_t lane = threadIdx.x & 63;
   const uint32_t wr = wave >> 1, wc = wave & 1;
-  const uint32_t tile_row0 = row_tile * TM2;
+  const uint32_t tile_row0 = row_tile * TM;
   const uint32_t tile_col0 = token_tile * TN2;
   const uint32_t ld_bytes = s * 2;
-  const uint32_t w_rows = min( (uint32_t)TM2, r - tile_row0 );
+  const uint32_t w_rows = min( (uint32_t)TM, r - tile_row0 );
   const uint32_t x_cols = min( (uint32_t)TN2, b - tile_col0 );
   const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc( const_cast<__half*>( w + (uint64_t)tile_row0 * s ), 0, (int)( w_rows * ld_bytes ), 0x00020000 );
   const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc( const_cast<__half*>( x + (uint64_t)tile_col0 * s ), 0, (int)( x_cols * ld_bytes ), 0x00020000 );
@@ -113,9 +120,9 @@ __global__ __launch_bounds__( T256_THREADS, 1 ) void gemm_tile256_kernel( __half
   const uint32_t voff = ( threadIdx.x >> 3 ) * ld_bytes + ( ( threadIdx.x & 7 ) ^ ( ( threadIdx.x >> 4 ) & 7 ) ) * 16;
   const uint32_t wave_slot0 = 8 * wave * 8; // first uint4 of the wave's 8 rows
 
-  f32x16 acc[2][4];
+  f32x16 acc[NA][4];
 #pragma unroll
-  for ( int rt = 0; rt < 2; rt++ ) {
+  for ( int rt = 0; rt < NA; rt++ ) {
 #pragma unroll
     for ( int t = 0; t < 4; t++ ) {
 #pragma unroll
@@ -126,21 +133,25 @@ __global__ __launch_bounds__( T256_THREADS, 1 ) void gemm_tile256_kernel( __half
   }
   const uint32_t n_steps = s / TKS;
   const uint32_t fr = lane & 31, g2 = lane >> 5;
-  auto fetch = [&]( uint4* wt, uint4* xt, uint32_t kb ) { // global -> LDS stage, 8 x 1 KiB per wave
+  auto fetch = [&]( uint4* wt, uint4* xt, uint32_t kb ) { // global -> LDS stage, 1 KiB per wave and instruction
 #pragma unroll
-    for ( int i = 0; i < 4; i++ ) {
+    for ( int i = 0; i < 2 * NA; i++ ) {
       __builtin_amdgcn_raw_ptr_buffer_load_lds( w_rsrc, (lds_ptr)( wt + wave_slot0 + 64 * i * 8 ), 16, voff, 64 * i * ld_bytes + kb, 0, 0 );
-      __builtin_amdgcn_raw_ptr_buffer_load_lds( x_rsrc, (lds_ptr)( xt + wave_slot0 + 64 * i * 8 ), 16, voff, 64 * i * ld_bytes + kb, 0, 0 );
+      if ( i < 4 ) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds( x_rsrc, (lds_ptr)( xt + wave_slot0 + 64 * i * 8 ), 16, voff, 64 * i * ld_bytes + kb, 0, 0 );
+      }
     }
   };
   struct Frags
   {
-    f16x8 a[2], bb[4];
+    f16x8 a[NA], bb[4];
   };
   auto read_k16 = [&]( Frags& f, const uint4* wt, const uint4* xt, int kk ) {
     const uint32_t ch = 2 * kk + g2;
-    f.a[0] = __builtin_bit_cast( f16x8, wt[swz( 64 * wr + fr, ch )] );
-    f.a[1] = __builtin_bit_cast( f16x8, wt[swz( 64 * wr + 32 + fr, ch )] );
+#pragma unroll
+    for ( int rt = 0; rt < NA; rt++ ) {
+      f.a[rt] = __builtin_bit_cast( f16x8, wt[swz( 32 * NA * wr + 32 * rt + fr, ch )] );
+    }
 #pragma unroll
     for ( int t = 0; t < 4; t++ ) {
       f.bb[t] = __builtin_bit_cast( f16x8, xt[swz( 128 * wc + 32 * t + fr, ch )] );
@@ -149,8 +160,10 @@ __global__ __launch_bounds__( T256_THREADS, 1 ) void gemm_tile256_kernel( __half
   auto mfma_k16 = [&]( const Frags& f ) {
 #pragma unroll
     for ( int t = 0; t < 4; t++ ) {
-      acc[0][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16( f.a[0], f.bb[t], acc[0][t], 0, 0, 0 );
-      acc[1][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16( f.a[1], f.bb[t], acc[1][t], 0, 0, 0 );
+#pragma unroll
+      for ( int rt = 0; rt < NA; rt++ ) {
+        acc[rt][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16( f.a[rt], f.bb[t], acc[rt][t], 0, 0, 0 );
+      }
     }
   };
   // Step j multiplies out of stage j % 2 while the memory unit writes step j + 1 straight into the
@@ -158,22 +171,37 @@ __global__ __launch_bounds__( T256_THREADS, 1 ) void gemm_tile256_kernel( __half
   // waits for those loads.  The loads behind the last step read the start of the next rows (bounded
   // by the descriptors); what they bring is never multiplied.
   auto step = [&]( const uint4* wt, const uint4* xt, uint4* wn, uint4* xn, uint32_t j ) {
-    Frags f0, f1;
-    read_k16( f0, wt, xt, 0 );
-    fetch( wn, xn, ( j + 1 ) * TKS * 2 );
-    read_k16( f1, wt, xt, 1 );
-    __builtin_amdgcn_s_setprio( 1 );
-    mfma_k16( f0 );
-    __builtin_amdgcn_s_setprio( 0 );
-    read_k16( f0, wt, xt, 2 );
-    __builtin_amdgcn_s_setprio( 1 );
-    mfma_k16( f1 );
-    __builtin_amdgcn_s_setprio( 0 );
-    read_k16( f1, wt, xt, 3 );
-    __builtin_amdgcn_s_setprio( 1 );
-    mfma_k16( f0 );
-    mfma_k16( f1 );
-    __builtin_amdgcn_s_setprio( 0 );
+    if constexpr ( NA == 2 ) { // two fragment sets: the reads of the next 16 k go out before the MFMAs of these
+      Frags f0, f1;
+      read_k16( f0, wt, xt, 0 );
+      fetch( wn, xn, ( j + 1 ) * TKS * 2 );
+      read_k16( f1, wt, xt, 1 );
+      __builtin_amdgcn_s_setprio( 1 );
+      mfma_k16( f0 );
+      __builtin_amdgcn_s_setprio( 0 );
+      read_k16( f0, wt, xt, 2 );
+      __builtin_amdgcn_s_setprio( 1 );
+      mfma_k16( f1 );
+      __builtin_amdgcn_s_setprio( 0 );
+      read_k16( f1, wt, xt, 3 );
+      __builtin_amdgcn_s_setprio( 1 );
+      mfma_k16( f0 );
+      mfma_k16( f1 );
+      __builtin_amdgcn_s_setprio( 0 );
+    } else { // 192 accumulator registers leave room for one set
+      Frags f;
+      read_k16( f, wt, xt, 0 );
+      fetch( wn, xn, ( j + 1 ) * TKS * 2 );
+#pragma unroll
+      for ( int kk = 0; kk < 4; kk++ ) {
+        __builtin_amdgcn_s_setprio( 1 );
+        mfma_k16( f );
+        __builtin_amdgcn_s_setprio( 0 );
+        if ( kk < 3 ) {
+          read_k16( f, wt, xt, kk + 1 );
+        }
+      }
+    }
     __syncthreads();
   };
   fetch( s_w0, s_x0, 0 );
@@ -188,7 +216,7 @@ __global__ __launch_bounds__( T256_THREADS, 1 ) void gemm_tile256_kernel( __half
       break;
     }
   }
-  // acc[rt][t][v]: row = tile_row0 + 64*wr + 32*rt + 8*(v/4) + 4*(lane/32) + v%4, token = tile_col0 + 128*wc + 32*t + lane%32
+  // acc[rt][t][v]: row = tile_row0 + 32*NA*wr + 32*rt + 8*(v/4) + 4*(lane/32) + v%4, token = tile_col0 + 128*wc + 32*t + lane%32
 #pragma unroll
   for ( int t = 0; t < 4; t++ ) {
     const uint32_t col = tile_col0 + 128 * wc + 32 * t + fr;
@@ -196,10 +224,10 @@ __global__ __launch_bounds__( T256_THREADS, 1 ) void gemm_tile256_kernel( __half
       continue;
     }
 #pragma unroll
-    for ( int rt = 0; rt < 2; rt++ ) {
+    for ( int rt = 0; rt < NA; rt++ ) {
 #pragma unroll
       for ( int q4 = 0; q4 < 4; q4++ ) {
-        const uint32_t row = tile_row0 + 64 * wr + 32 * rt + 8 * q4 + 4 * g2;
+        const uint32_t row = tile_row0 + 32 * NA * wr + 32 * rt + 8 * q4 + 4 * g2;
         const bool whole = row + 3 < r && ( r & 3 ) == 0;
         if ( PARTIAL ) {
           float* dst = partial + (uint64_t)col * r + row;
@@ -238,7 +266,32 @@ __global__ __launch_bounds__( T256_THREADS, 1 ) void gemm_tile256_kernel( __half
   }
 }
 
+int g_tile_rows = 0; // 0: by tile256_rows(); 256 or 384: forced
+
+// Rounds of one work-group per CU that an XCD (32 CUs) runs for its share of the tiles.
+uint64_t rounds_per_xcd( uint64_t r, uint64_t b, uint64_t tile_rows )
+{
+  const uint64_t row_tiles = ( r + tile_rows - 1 ) / tile_rows, token_tiles = ( b + TN2 - 1 ) / TN2;
+  const uint64_t tiles = ( row_tiles / 8 ) * token_tiles + ( ( row_tiles % 8 ) * token_tiles + 7 ) / 8;
+  return ( tiles + 31 ) / 32;
+}
+
+// 384 rows per work-group when that takes less time: rounds x the time of a round.  Measured at
+// 16384 tokens x 12288 rows (12 rounds of 256-row tiles, 8 of 384-row tiles), a round of 384-row
+// tiles takes 1.44-1.49 x a round of 256-row tiles for K >= 7168 and 1.32-1.45 x for shorter K (the
+// cost of starting and storing a tile is paid for 1.5 x the flops), against 1.5 x the flops.
+uint32_t tile256_rows( uint64_t s, uint64_t r, uint64_t b )
+{
+  if ( g_tile_rows == 256 || g_tile_rows == 384 ) {
+    return (uint32_t)g_tile_rows;
+  }
+  const uint64_t round_cost_pct = s >= 7168 ? 147 : 138;
+  return round_cost_pct * rounds_per_xcd( r, b, 384 ) < 97 * rounds_per_xcd( r, b, 256 ) ? 384 : 256; // 3 % in hand for 256
+}
+
 } // namespace
+
+void gemm_tile256_tuning( int rows ) { g_tile_rows = rows; }
 
 // Worth it when the 256 x 256 tiles alone fill the chip (no K split here) and the last round of them
 // is not mostly empty (measured against the 128 x 128 kernel: 15-40 % faster from 192 tiles up, except
@@ -258,7 +311,8 @@ bool gemm_tile256_applicable( uint64_t s, uint64_t r, uint64_t b, const void* x,
 int gemm_tile256_launch( __half* xout, float* partial, const __half* x, const __half* w, uint64_t s, uint64_t r, uint64_t b, hipStream_t st )
 {
   TileOrder ord;
-  ord.row_tiles = (uint32_t)( ( r + TM2 - 1 ) / TM2 );
+  const uint32_t tile_rows = tile256_rows( s, r, b );
+  ord.row_tiles = (uint32_t)( ( r + tile_rows - 1 ) / tile_rows );
   ord.token_tiles = (uint32_t)( ( b + TN2 - 1 ) / TN2 );
   ord.gn = std::min<uint32_t>( ord.token_tiles, 8 );
   ord.rows_per_xcd = ord.row_tiles / 8;
@@ -272,10 +326,20 @@ int gemm_tile256_launch( __half* xout, float* partial, const __half* x, const __
   GH_REQUIRE( gx < ( 1ull << 31 ), "gh_matmul: grid too large" );
   ord.main_per_xcd = (uint32_t)main_per_xcd;
   ord.rest_share = (uint32_t)rest_share;
-  if ( partial != nullptr ) {
-    gemm_tile256_kernel<true><<<(unsigned)gx, T256_THREADS, 0, st>>>( xout, partial, x, w, (uint32_t)s, (uint32_t)r, (uint32_t)b, ord );
+  const dim3 grid( (unsigned)gx ), block( T256_THREADS );
+  const uint32_t s32 = (uint32_t)s, r32 = (uint32_t)r, b32 = (uint32_t)b;
+  if ( tile_rows == 384 ) {
+    if ( partial != nullptr ) {
+      gemm_tile256_kernel<true, 3><<<grid, block, 0, st>>>( xout, partial, x, w, s32, r32, b32, ord );
+    } else {
+      gemm_tile256_kernel<false, 3><<<grid, block, 0, st>>>( xout, partial, x, w, s32, r32, b32, ord );
+    }
   } else {
-    gemm_tile256_kernel<false><<<(unsigned)gx, T256_THREADS, 0, st>>>( xout, partial, x, w, (uint32_t)s, (uint32_t)r, (uint32_t)b, ord );
+    if ( partial != nullptr ) {
+      gemm_tile256_kernel<true, 2><<<grid, block, 0, st>>>( xout, partial, x, w, s32, r32, b32, ord );
+    } else {
+      gemm_tile256_kernel<false, 2><<<grid, block, 0, st>>>( xout, partial, x, w, s32, r32, b32, ord );
+    }
   }
   GH_LAUNCH_CHECK();
   return GH_OK;

@@ -130,9 +130,10 @@ int gh_silu( void* hb, const void* hb2, uint64_t hidden_dim, uint64_t batch, gh_
 int gh_argmax( uint32_t* out_host, uint32_t* out_dev, const void* v, uint64_t n, uint64_t batch, gh_dtype dt, gh_stream stream );
 /* Operations::matmul<s,r> / untemplated_matmul  arch/amd64/common/ops.hh:74-93,212-271 :
  * xout(b, r) = sum_p w(r, p) * x(b, p); w row-major (r, s); fp32 accumulate */
-/* tuning hook: kernel 0 auto / 1 small tiled / 2 streaming (decode) / 3 128x128 tile / 4 256x256 tile (many rows); the number of compute units the
- * streaming kernel's K split is balanced for (<= 0 keeps the current value; the default is the device's own count); the third argument is ignored */
-int gh_gemm_set_tuning( int kernel, int target_workgroups, int depth );
+/* tuning hook: kernel 0 auto / 1 small tiled / 2 streaming (decode) / 3 128x128 tile / 4 256-token tile (many rows); the number of compute units the
+ * streaming kernel's K split is balanced for (<= 0 keeps the current value; the default is the device's own count); weight rows per work-group of the
+ * 256-token tile kernel: 256, 384, or 0 for the library's choice */
+int gh_gemm_set_tuning( int kernel, int target_workgroups, int tile_rows );
 /* host-only query: how the weight-streaming kernel would cut an (r x s) . (b x s)^T product for the initialised device (256 compute
  * units before initialisation): number of K ranges, k per range (a multiple of 256), weight rows per work-group */
 int gh_gemm_stream_plan( uint64_t s, uint64_t r, uint64_t b, uint32_t* splits, uint32_t* k_per_split, uint32_t* rows_per_workgroup );

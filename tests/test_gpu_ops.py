@@ -168,15 +168,17 @@ def test_matmul_many_rows(dt, b, s, r):
     assert_close(got, want, what=f"matmul {dt} {b}x{s}x{r}")
 
 
-# enough 256 x 256 tiles for the second tile kernel (forced, and whatever the dispatcher picks), ragged edges
-@pytest.mark.parametrize("force", [4, 0])
+# enough 256-token tiles for the second tile kernel (forced with 256 and with 384 rows per work-group, and
+# whatever the dispatcher picks), ragged edges; the row counts leave 4, 0 and 6 (256) / 3, 6 and 7 (384)
+# row tiles beyond a multiple of 8, the part of the tile order that is cut into equal runs per XCD
+@pytest.mark.parametrize("force,rows", [(4, 256), (4, 384), (4, 0), (0, 0)])
 @pytest.mark.parametrize("b,s,r", [(3000, 8192, 4100), (8200, 128, 8190), (700, 8256, 18000)])
-def test_matmul_256_tiles(force, b, s, r):
+def test_matmul_256_tiles(force, rows, b, s, r):
     from glinthawk_amd import _lib
     rng = np.random.default_rng(26)
     x = rng.standard_normal((b, s)).astype(np.float16)
     w = (rng.standard_normal((r, s)) / np.sqrt(s)).astype(np.float16)
-    _lib.lib().gh_gemm_set_tuning(force, 0, 0)
+    _lib.lib().gh_gemm_set_tuning(force, 0, rows)
     try:
         got = ops.matmul(torch.from_numpy(x).cuda(), torch.from_numpy(w).cuda())
     finally:
@@ -189,14 +191,18 @@ def test_matmul_256_tiles(force, b, s, r):
     assert_close(got[:8].cpu().numpy(), want_cpu, what=f"matmul 256-tile {b}x{s}x{r}")
 
 
-def test_matmul_256_tile_one_hot_layout():
+@pytest.mark.parametrize("rows", [256, 384])
+@pytest.mark.parametrize("s,r,b", [(8192, 12544, 1030),    # 49 / 33 row tiles x 5: one left-over row tile
+                                   (1024, 5000, 16390),    # 20 / 14 row tiles x 65: 4 / 6 left over, ragged last token tile
+                                   (256, 1700, 9000)])     # 7 / 5 row tiles: left-over tiles only
+def test_matmul_256_tile_one_hot_layout(rows, s, r, b):
+    """One-hot activations: every output is one weight, so each tile of the order must land bit for bit."""
     from glinthawk_amd import _lib
-    s, r, b = 8192, 12544, 1030            # 49 x 5 = 245 tiles, ragged in both directions
     w = torch.arange(r * s, dtype=torch.float32, device="cuda").reshape(r, s).remainder(1000).half()
     x = torch.zeros((b, s), dtype=torch.float16, device="cuda")
     cols = [(7919 * i + 3) % s for i in range(b)]
     x[torch.arange(b), torch.tensor(cols)] = 1
-    _lib.lib().gh_gemm_set_tuning(4, 0, 0)
+    _lib.lib().gh_gemm_set_tuning(4, 0, rows)
     try:
         got = ops.matmul(x, w)
     finally:
