@@ -133,13 +133,30 @@ __global__ __launch_bounds__( T256_THREADS, 1 ) void gemm_tile256_kernel( __half
   }
   const uint32_t n_steps = s / TKS;
   const uint32_t fr = lane & 31, g2 = lane >> 5;
-  auto fetch = [&]( uint4* wt, uint4* xt, uint32_t kb ) { // global -> LDS stage, 1 KiB per wave and instruction
+  // global -> LDS stage, 1 KiB per wave and instruction: loads [from, to) of the list W0 X0 W1 X1 W2 X2 W3 X3 (W4 W5)
+  constexpr int N_LOADS = 2 * NA + 4;
+  auto fetch = [&]( uint4* wt, uint4* xt, uint32_t kb, int from, int to ) {
 #pragma unroll
-    for ( int i = 0; i < 2 * NA; i++ ) {
-      __builtin_amdgcn_raw_ptr_buffer_load_lds( w_rsrc, (lds_ptr)( wt + wave_slot0 + 64 * i * 8 ), 16, voff, 64 * i * ld_bytes + kb, 0, 0 );
-      if ( i < 4 ) {
+    for ( int l = 0; l < N_LOADS; l++ ) {
+      if ( l < from || l >= to ) {
+        continue;
+      }
+      const bool is_w = l >= 8 || ( l & 1 ) == 0;
+      const int i = l >= 8 ? l - 4 : l >> 1;
+      if ( is_w ) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds( w_rsrc, (lds_ptr)( wt + wave_slot0 + 64 * i * 8 ), 16, voff, 64 * i * ld_bytes + kb, 0, 0 );
+      } else {
         __builtin_amdgcn_raw_ptr_buffer_load_lds( x_rsrc, (lds_ptr)( xt + wave_slot0 + 64 * i * 8 ), 16, voff, 64 * i * ld_bytes + kb, 0, 0 );
       }
+    }
+  };
+  // The loads of a step go out in front of the MFMAs of its first two (three, for 384 rows) groups of
+  // 16 k: all of them at the head of the step measured 0-4 % slower, spread over all four groups
+  // slower again for 256 rows (the last ones then have a quarter of a step to arrive).
+  auto fetch_at = [&]( uint4* wn, uint4* xn, uint32_t kb, int kk ) {
+    constexpr int parts = NA == 2 ? 2 : 3;
+    if ( kk < parts ) {
+      fetch( wn, xn, kb, ( N_LOADS * kk + parts - 1 ) / parts, ( N_LOADS * ( kk + 1 ) + parts - 1 ) / parts );
     }
   };
   struct Frags
@@ -171,29 +188,35 @@ __global__ __launch_bounds__( T256_THREADS, 1 ) void gemm_tile256_kernel( __half
   // waits for those loads.  The loads behind the last step read the start of the next rows (bounded
   // by the descriptors); what they bring is never multiplied.
   auto step = [&]( const uint4* wt, const uint4* xt, uint4* wn, uint4* xn, uint32_t j ) {
+    const uint32_t kb = ( j + 1 ) * TKS * 2;
     if constexpr ( NA == 2 ) { // two fragment sets: the reads of the next 16 k go out before the MFMAs of these
       Frags f0, f1;
       read_k16( f0, wt, xt, 0 );
-      fetch( wn, xn, ( j + 1 ) * TKS * 2 );
+      fetch_at( wn, xn, kb, 0 );
       read_k16( f1, wt, xt, 1 );
       __builtin_amdgcn_s_setprio( 1 );
       mfma_k16( f0 );
       __builtin_amdgcn_s_setprio( 0 );
+      fetch_at( wn, xn, kb, 1 );
       read_k16( f0, wt, xt, 2 );
       __builtin_amdgcn_s_setprio( 1 );
       mfma_k16( f1 );
       __builtin_amdgcn_s_setprio( 0 );
+      fetch_at( wn, xn, kb, 2 );
       read_k16( f1, wt, xt, 3 );
       __builtin_amdgcn_s_setprio( 1 );
       mfma_k16( f0 );
+      __builtin_amdgcn_s_setprio( 0 );
+      fetch_at( wn, xn, kb, 3 );
+      __builtin_amdgcn_s_setprio( 1 );
       mfma_k16( f1 );
       __builtin_amdgcn_s_setprio( 0 );
     } else { // 192 accumulator registers leave room for one set
       Frags f;
       read_k16( f, wt, xt, 0 );
-      fetch( wn, xn, ( j + 1 ) * TKS * 2 );
 #pragma unroll
       for ( int kk = 0; kk < 4; kk++ ) {
+        fetch_at( wn, xn, kb, kk );
         __builtin_amdgcn_s_setprio( 1 );
         mfma_k16( f );
         __builtin_amdgcn_s_setprio( 0 );
@@ -204,7 +227,7 @@ __global__ __launch_bounds__( T256_THREADS, 1 ) void gemm_tile256_kernel( __half
     }
     __syncthreads();
   };
-  fetch( s_w0, s_x0, 0 );
+  fetch( s_w0, s_x0, 0, 0, N_LOADS );
   __syncthreads();
   for ( uint32_t j = 0;; ) {
     step( s_w0, s_x0, s_w1, s_x1, j );
