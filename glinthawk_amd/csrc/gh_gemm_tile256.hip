@@ -25,9 +25,15 @@
 //                 one step ahead, ds_write in the middle of the MFMAs): 1.02 -> 1.15 PFLOP/s at
 //                 16384 x 8192 x 57344.
 //   what binds  with the loads taken out the loop runs at 1.8-2.1 PFLOP/s (2.1-2.3 without the
-//                 barrier as well); with every work-group reading the same L2-resident tile at
-//                 1.2: a step's 64 KiB arrive at about 16 bytes per clock and CU from L2, however
-//                 they are addressed, and that, not the matrix pipe or LDS, sets the step time.
+//                 barrier as well); with the loads issued but never waited for (all aimed at one
+//                 spare KiB of LDS) at 1.65; with every work-group reading the same L2-resident
+//                 tile at 1.2.  So neither the matrix pipe, nor LDS, nor the rate of the path from
+//                 L2 sets the step time, but how much can be in flight: a step's 64 KiB are asked
+//                 for at its head and must be there at its end, and two stages are all the LDS
+//                 holds beside the stage being read.  Tried and not kept: a third stage for the
+//                 activations alone (their loads two steps ahead, the weights' one: -6..+7 %), five
+//                 32-k stages as a ring with the loads three half-steps ahead (two barriers per
+//                 64 k, half lines per request: -5..-15 %), non-temporal loads (-10 %).
 //   tile order  as in the 128 x 128 kernel: each XCD owns every 8th row tile and walks patches of
 //                 tiles that are resident together.  The row tiles beyond a multiple of 8 are cut
 //                 into 8 equal runs of tiles instead, so that every XCD gets the same number of
