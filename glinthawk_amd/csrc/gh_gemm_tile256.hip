@@ -24,16 +24,17 @@
 //                 the one with matrix work goes first.  Against staging through registers (loads
 //                 one step ahead, ds_write in the middle of the MFMAs): 1.02 -> 1.15 PFLOP/s at
 //                 16384 x 8192 x 57344.
-//   what binds  with the loads taken out the loop runs at 1.8-2.1 PFLOP/s (2.1-2.3 without the
-//                 barrier as well); with the loads issued but never waited for (all aimed at one
-//                 spare KiB of LDS) at 1.65; with every work-group reading the same L2-resident
-//                 tile at 1.2.  So neither the matrix pipe, nor LDS, nor the rate of the path from
-//                 L2 sets the step time, but how much can be in flight: a step's 64 KiB are asked
-//                 for at its head and must be there at its end, and two stages are all the LDS
-//                 holds beside the stage being read.  Tried and not kept: a third stage for the
-//                 activations alone (their loads two steps ahead, the weights' one: -6..+7 %), five
-//                 32-k stages as a ring with the loads three half-steps ahead (two barriers per
-//                 64 k, half lines per request: -5..-15 %), non-temporal loads (-10 %).
+//   what binds  measured at 16384 tokens, 70B shapes, 256 rows (1.15-1.19 PFLOP/s as is; variants
+//                 that keep every LDS read: the compiler folds reads of a stage nothing writes):
+//                 loads taken out of the loop, both stages filled once, barrier kept: 1.33-1.45;
+//                 loads issued into one stage pair but never waited for, reads from the other:
+//                 1.16-1.22.  So waiting for the loads costs nothing to speak of, their traffic
+//                 through the CU about 15 %, and the rest is the loop of LDS reads, MFMAs and one
+//                 barrier per 64 k itself (MFMA pipes busy 55 %; a wave sits in s_waitcnt 15 % of
+//                 its time, LDS reads take 4 cycles per instruction without conflicts).  Tried and
+//                 not kept: a third stage for the activations (their loads two steps ahead, -6..+7 %),
+//                 that plus the weights two steps ahead through registers (-5..+3 %), five 32-k
+//                 stages as a ring (two barriers per 64 k: -5..-15 %), non-temporal loads (-10 %).
 //   tile order  as in the 128 x 128 kernel: each XCD owns every 8th row tile and walks patches of
 //                 tiles that are resident together.  The row tiles beyond a multiple of 8 are cut
 //                 into 8 equal runs of tiles instead, so that every XCD gets the same number of
