@@ -229,7 +229,8 @@ class Stage:
         if toks is not None:
             assert toks.size == batch * n_tokens
         dim = None if acts is None else acts.reshape(batch * n_tokens, -1).shape[1]
-        out = None
+        if not want_activations:
+            out = None
         if want_activations:
             if dim is None:
                 raise ValueError("pass dim via activations or call with want_activations=False")

@@ -190,7 +190,11 @@ def test_stage_prefill_middle_stage_and_chunks():
         outs[:, pos] = b.activations().reshape(batch, cfg.dim).astype(np.float32)
     first, second = 16, T - 16
     o1, _ = a.prefill([70, 71], [0, 0], first, 1, activations=x[:, :first].reshape(batch * first, cfg.dim))
-    o2, _ = a.prefill([70, 71], [first, first], second, 1, activations=x[:, first:].reshape(batch * second, cfg.dim))
+    # the second chunk lands in a buffer of the caller's (page-locked, as the benchmark passes it)
+    mine = ops.pinned_empty((batch * second, cfg.dim), x.dtype)
+    mine[:] = 0
+    o2, _ = a.prefill([70, 71], [first, first], second, 1, activations=x[:, first:].reshape(batch * second, cfg.dim), out=mine)
+    assert o2 is mine
     got = np.concatenate([o1.reshape(batch, first, cfg.dim), o2.reshape(batch, second, cfg.dim)], axis=1).astype(np.float32)
     np.testing.assert_allclose(got, outs, rtol=6e-3, atol=6e-3)
     a.close()
