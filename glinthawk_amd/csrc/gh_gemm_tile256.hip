@@ -11,8 +11,12 @@
 //                 0.82-0.97 PFLOP/s however the operands were fetched.
 //   384 rows    bring 80 KiB per 64 k for 1.5 x the flops of 256 rows (64 KiB) and fill the LDS
 //                 (2 x 80 KiB) and the registers (one set of MFMA operands instead of two); a round
-//                 of them takes 1.32-1.49 x as long, so they win where their rounds fit the shape
+//                 of them takes 1.24-1.44 x as long, so they win where their rounds fit the shape
 //                 at least as well (tile256_rows() below)
+//   output      through LDS, token-major, and from there as whole row segments (16 bytes per lane,
+//                 512 or 768 contiguous bytes per token): stored from the accumulator registers, an
+//                 instruction touches 32 lines with 16 bytes each, which cost 10-16 % of the kernel
+//                 at K 5120-8192
 //   operands    both go global -> LDS without passing through registers (`buffer_load ... lds`, 16
 //                 bytes per lane: a wave's instruction writes 1 KiB of LDS, lane l at + 16 l, so the
 //                 XOR swizzle that keeps the MFMA reads free of bank conflicts is applied to the
@@ -247,6 +251,75 @@ __global__ __launch_bounds__( T256_THREADS, 1 ) void gemm_tile256_kernel( __half
     }
   }
   // acc[rt][t][v]: row = tile_row0 + 32*NA*wr + 32*rt + 8*(v/4) + 4*(lane/32) + v%4, token = tile_col0 + 128*wc + 32*t + lane%32
+  if ( !PARTIAL && ( r & 7 ) == 0 ) {
+    // Output through LDS: a lane holds 4 rows (8 bytes) of 32 different tokens, and stored from the
+    // registers every instruction would touch 32 lines, 16 bytes each (that epilogue cost 10-16 % of
+    // the kernel at K 5120-8192).  The tile goes to LDS token-major instead, 64 tokens per stage array
+    // (16-byte chunks of 8 rows, chunk index XORed with the token so that neither side has bank
+    // conflicts), and from there to memory as whole row segments, 16 bytes per lane.
+    constexpr uint32_t CHUNKS = TM / 8;                    // 16-byte chunks per token: 32 or 48
+    constexpr uint32_t SWZ_MASK = NA == 2 ? 31 : 15;      // the XOR stays inside a power-of-two group of chunks
+    auto put = [&]( uint4* region, int t ) { // this wave's 32 tokens of block t -> tokens 32 (t % 2) + fr of the region
+      uint2* out = reinterpret_cast<uint2*>( region );
+      const uint32_t token = 32 * ( t & 1 ) + fr;
+#pragma unroll
+      for ( int rt = 0; rt < NA; rt++ ) {
+#pragma unroll
+        for ( int q4 = 0; q4 < 4; q4++ ) {
+          union
+          {
+            uint2 raw;
+            __half h[4];
+          } o;
+#pragma unroll
+          for ( int e = 0; e < 4; e++ ) {
+            o.h[e] = __float2half_rn( acc[rt][t][4 * q4 + e] );
+          }
+          const uint32_t chunk = 4 * NA * wr + 4 * rt + q4;
+          out[( token * CHUNKS + ( chunk ^ ( token & SWZ_MASK ) ) ) * 2 + g2] = o.raw;
+        }
+      }
+    };
+    auto copy_out = [&]( const uint4* region, uint32_t first_token, uint32_t j ) { // chunk j of a region of 64 tokens
+      const uint32_t token = j / CHUNKS, slot = j % CHUNKS;
+      const uint32_t chunk = slot ^ ( token & SWZ_MASK );
+      const uint32_t col = tile_col0 + first_token + token, row = tile_row0 + 8 * chunk;
+      if ( col < b && row < r ) {
+        *reinterpret_cast<uint4*>( xout + (uint64_t)col * r + row ) = region[j];
+      }
+    };
+    if constexpr ( NA == 2 ) { // four regions of 64 tokens x 256 rows = the four stage arrays
+#pragma unroll
+      for ( int t = 0; t < 4; t++ ) {
+        put( wc == 0 ? ( t < 2 ? s_x0 : s_x1 ) : ( t < 2 ? s_w0 : s_w1 ), t );
+      }
+      __syncthreads();
+#pragma unroll
+      for ( int it = 0; it < 16; it++ ) {
+        const uint4* region = it < 4 ? s_x0 : it < 8 ? s_x1 : it < 12 ? s_w0 : s_w1;
+        copy_out( region, 64 * ( it / 4 ), ( it % 4 ) * T256_THREADS + threadIdx.x );
+      }
+    } else { // 64 tokens x 384 rows fill a weight stage: the two token halves of the tile one after the other
+#pragma unroll
+      for ( int half = 0; half < 2; half++ ) {
+        if ( half == 1 ) {
+          __syncthreads();
+        }
+        if ( wc == (uint32_t)half ) {
+#pragma unroll
+          for ( int t = 0; t < 4; t++ ) {
+            put( t < 2 ? s_w0 : s_w1, t );
+          }
+        }
+        __syncthreads();
+#pragma unroll
+        for ( int it = 0; it < 12; it++ ) {
+          copy_out( it < 6 ? s_w0 : s_w1, 128 * half + 64 * ( it / 6 ), ( it % 6 ) * T256_THREADS + threadIdx.x );
+        }
+      }
+    }
+    return;
+  }
 #pragma unroll
   for ( int t = 0; t < 4; t++ ) {
     const uint32_t col = tile_col0 + 128 * wc + 32 * t + fr;
@@ -308,14 +381,14 @@ uint64_t rounds_per_xcd( uint64_t r, uint64_t b, uint64_t tile_rows )
 
 // 384 rows per work-group when that takes less time: rounds x the time of a round.  Measured at
 // 16384 tokens x 12288 rows (12 rounds of 256-row tiles, 8 of 384-row tiles), a round of 384-row
-// tiles takes 1.44-1.49 x a round of 256-row tiles for K >= 7168 and 1.32-1.45 x for shorter K (the
+// tiles takes 1.41-1.44 x a round of 256-row tiles for K 7168-13824 and 1.24-1.39 x for shorter K (the
 // cost of starting and storing a tile is paid for 1.5 x the flops), against 1.5 x the flops.
 uint32_t tile256_rows( uint64_t s, uint64_t r, uint64_t b )
 {
   if ( g_tile_rows == 256 || g_tile_rows == 384 ) {
     return (uint32_t)g_tile_rows;
   }
-  const uint64_t round_cost_pct = s >= 7168 ? 147 : 138;
+  const uint64_t round_cost_pct = s >= 7168 ? 143 : 136;
   return round_cost_pct * rounds_per_xcd( r, b, 384 ) < 97 * rounds_per_xcd( r, b, 256 ) ? 384 : 256; // 3 % in hand for 256
 }
 
