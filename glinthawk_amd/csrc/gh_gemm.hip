@@ -25,7 +25,7 @@ bool gemm_stream_gate_applicable( uint64_t s, uint64_t hidden, uint64_t b, const
 int gemm_stream_gate_launch( __half* hb, const __half* x, const __half* w13, uint64_t s, uint64_t hidden, uint64_t b, hipStream_t st );
 // 256 x 256 tile kernel for products with enough tiles (gh_gemm_tile256.hip)
 bool gemm_tile256_applicable( uint64_t s, uint64_t r, uint64_t b, const void* x, const void* w, const void* xout );
-int gemm_tile256_launch( __half* xout, float* partial, const __half* x, const __half* w, uint64_t s, uint64_t r, uint64_t b, hipStream_t st );
+int gemm_tile256_launch( __half* xout, float* partial, const __half* x, const __half* w, uint64_t s, uint64_t r, uint64_t b, int epilogue, hipStream_t st );
 void gemm_tile256_tuning( int rows );
 // large-batch (prefill) kernel (gh_gemm_tile.hip)
 bool gemm_tile_applicable( uint64_t s, uint64_t r, uint64_t b, const void* x, const void* w, const void* xout );
@@ -250,6 +250,25 @@ int gemm_gate_one_launch( void* hb, const void* x, const void* w13, uint64_t s, 
   return gemm_stream_gate_launch( static_cast<__half*>( hb ), static_cast<const __half*>( x ), static_cast<const __half*>( w13 ), s, hidden, b, st );
 }
 
+// Many rows: the large tile kernel with the op that follows the product in its epilogue, 1 = xout += product
+// (accum).  *done = false: nothing was launched (shape or alignment not for that kernel), the caller takes
+// its other route.
+bool gemm_tile_epilogue_applicable( uint64_t s, uint64_t r, uint64_t b, gh_dtype dt, const void* x, const void* w, const void* xout )
+{
+  return dt == GH_F16 && r % 8 == 0 && ( g_force_kernel == 0 || g_force_kernel == 4 ) && gemm_tile256_applicable( s, r, b, x, w, xout );
+}
+
+int gemm_tile_epilogue_launch( void* xout, const void* x, const void* w, uint64_t s, uint64_t r, uint64_t b, gh_dtype dt, int epilogue, hipStream_t st,
+                               bool* done )
+{
+  *done = false;
+  if ( !gemm_tile_epilogue_applicable( s, r, b, dt, x, w, xout ) ) {
+    return GH_OK;
+  }
+  *done = true;
+  return gemm_tile256_launch( static_cast<__half*>( xout ), nullptr, static_cast<const __half*>( x ), static_cast<const __half*>( w ), s, r, b, epilogue, st );
+}
+
 int gemm_partials( void* xout, const void* x, const void* w, uint64_t s, uint64_t r, uint64_t b, gh_dtype dt, hipStream_t st, bool want_partials,
                    float** partial_out, uint32_t* splits_out )
 {
@@ -281,7 +300,7 @@ int gemm_partials( void* xout, const void* x, const void* w, uint64_t s, uint64_
       *partial_out = ws;
       *splits_out = 1;
     }
-    return gemm_tile256_launch( static_cast<__half*>( xout ), ws, static_cast<const __half*>( x ), static_cast<const __half*>( w ), s, r, b, st );
+    return gemm_tile256_launch( static_cast<__half*>( xout ), ws, static_cast<const __half*>( x ), static_cast<const __half*>( w ), s, r, b, 0, st );
   }
   GH_REQUIRE( g_force_kernel != 4, "gh_matmul: the 256 x 256 tile kernel needs b >= 192, at least 192 tiles with a last round that is not mostly empty, s %% 64 == 0 and 16-byte aligned operands" );
   if ( ( g_force_kernel == 0 || g_force_kernel == 3 ) && gemm_tile_applicable( s, r, b, x, w, xout ? xout : x ) ) {
@@ -364,6 +383,12 @@ int gh_gemm_set_tuning( int kernel, int target_workgroups, int tile_rows )
   gemm_stream_tuning( target_workgroups, 0 );
   gemm_tile256_tuning( tile_rows );
   return GH_OK;
+}
+
+int gh_matmul_fuses_many_rows( uint64_t s, uint64_t r, uint64_t b, gh_dtype dt )
+{
+  static const char aligned[16] __attribute__( ( aligned( 16 ) ) ) = { 0 };
+  return gemm_tile_epilogue_applicable( s, r, b, dt, aligned, aligned, aligned ) ? 1 : 0;
 }
 
 int gh_gemm_stream_plan( uint64_t s, uint64_t r, uint64_t b, uint32_t* splits, uint32_t* k_per_split, uint32_t* rows_per_workgroup )

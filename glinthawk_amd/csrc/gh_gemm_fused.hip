@@ -11,6 +11,8 @@ namespace gh {
 int gemm_partials( void* xout, const void* x, const void* w, uint64_t s, uint64_t r, uint64_t b, gh_dtype dt, hipStream_t st, bool want_partials,
                    float** partial_out, uint32_t* splits_out );
 int gemm_gate_one_launch( void* hb, const void* x, const void* w13, uint64_t s, uint64_t hidden, uint64_t b, gh_dtype dt, hipStream_t st, bool* done );
+int gemm_tile_epilogue_launch( void* xout, const void* x, const void* w, uint64_t s, uint64_t r, uint64_t b, gh_dtype dt, int epilogue, hipStream_t st,
+                               bool* done );
 
 namespace {
 
@@ -302,6 +304,15 @@ int gh_matmul_accum( void* residual, const void* x, const void* w, uint64_t s, u
   GH_REQUIRE( residual != nullptr, "gh_matmul_accum: NULL residual" );
   GH_REQUIRE( ( norm_out == nullptr ) == ( norm_weight == nullptr ), "gh_matmul_accum: norm_out and norm_weight go together" );
   hipStream_t st = as_stream( stream );
+  // many rows (prompt tokens): the residual is added in the tile kernel's epilogue, no fp32 partials;
+  // the norm of the new residual, when asked for, is the plain row kernel
+  bool done = false;
+  if ( int rc = gemm_tile_epilogue_launch( residual, x, w, s, r, b, dt, 1, st, &done ) ) {
+    return rc;
+  }
+  if ( done ) {
+    return norm_out != nullptr ? gh_rmsnorm( norm_out, residual, norm_weight, r, b, dt, stream ) : GH_OK;
+  }
   float* partial = nullptr;
   uint32_t splits = 0;
   if ( int rc = gemm_partials( nullptr, x, w, s, r, b, dt, st, true, &partial, &splits ) ) {

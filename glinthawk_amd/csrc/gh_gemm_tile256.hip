@@ -74,9 +74,15 @@ struct TileOrder
 
 constexpr int T256_THREADS = 512;
 
-// grid: 8 x (padded tiles of one XCD).  s % 64 == 0, 16-byte aligned operands.  PARTIAL: fp32 (1, b, r) instead of xout.
+// What a work-group does with its sums: xout = DType(sum); the reference's next op on top of that,
+// xout = DType(float(xout) + float(DType(sum))) (accum; only with r % 8 == 0); or the fp32 sums, (1, b, r).
+// (The SiLU gate was tried here as well: with one work-group per CU nothing hides the epilogue's
+// divisions and exponentials, and the separate element-wise kernel is faster.)
+constexpr int EPI_STORE = 0, EPI_ACCUM = 1, EPI_PARTIAL = 3;
+
+// grid: 8 x (padded tiles of one XCD).  s % 64 == 0, 16-byte aligned operands.
 // NA: 32-row accumulator tiles per wave, 2 (256 weight rows per work-group) or 3 (384).
-template<bool PARTIAL, int NA>
+template<int EPI, int NA>
 __global__ __launch_bounds__( T256_THREADS, 1 ) void gemm_tile256_kernel( __half* __restrict__ xout,
                                                                         float* __restrict__ partial,
                                                                         const __half* __restrict__ x,
@@ -251,6 +257,7 @@ __global__ __launch_bounds__( T256_THREADS, 1 ) void gemm_tile256_kernel( __half
     }
   }
   // acc[rt][t][v]: row = tile_row0 + 32*NA*wr + 32*rt + 8*(v/4) + 4*(lane/32) + v%4, token = tile_col0 + 128*wc + 32*t + lane%32
+  constexpr bool PARTIAL = EPI == EPI_PARTIAL;
   if ( !PARTIAL && ( r & 7 ) == 0 ) {
     // Output through LDS: a lane holds 4 rows (8 bytes) of 32 different tokens, and stored from the
     // registers every instruction would touch 32 lines, 16 bytes each (that epilogue cost 10-16 % of
@@ -285,7 +292,21 @@ __global__ __launch_bounds__( T256_THREADS, 1 ) void gemm_tile256_kernel( __half
       const uint32_t chunk = slot ^ ( token & SWZ_MASK );
       const uint32_t col = tile_col0 + first_token + token, row = tile_row0 + 8 * chunk;
       if ( col < b && row < r ) {
-        *reinterpret_cast<uint4*>( xout + (uint64_t)col * r + row ) = region[j];
+        uint4* dst = reinterpret_cast<uint4*>( xout + (uint64_t)col * r + row );
+        union
+        {
+          uint4 raw;
+          __half h[8];
+        } y, old;
+        y.raw = region[j];
+        if ( EPI == EPI_ACCUM ) { // the op that follows the product, on the rounded product
+          old.raw = *dst;
+#pragma unroll
+          for ( int e = 0; e < 8; e++ ) {
+            y.h[e] = __float2half_rn( __half2float( old.h[e] ) + __half2float( y.h[e] ) );
+          }
+        }
+        *dst = y.raw;
       }
     };
     if constexpr ( NA == 2 ) { // four regions of 64 tokens x 256 rows = the four stage arrays
@@ -410,8 +431,8 @@ bool gemm_tile256_applicable( uint64_t s, uint64_t r, uint64_t b, const void* x,
          && ( ( reinterpret_cast<uintptr_t>( x ) | reinterpret_cast<uintptr_t>( w ) | reinterpret_cast<uintptr_t>( xout ) ) & 15u ) == 0;
 }
 
-// `partial` != nullptr: fp32 sums (1, b, r) instead of xout
-int gemm_tile256_launch( __half* xout, float* partial, const __half* x, const __half* w, uint64_t s, uint64_t r, uint64_t b, hipStream_t st )
+// `partial` != nullptr: fp32 sums (1, b, r) instead of xout; else `epilogue` 0 stores, 1 accumulates into xout (needs r % 8 == 0)
+int gemm_tile256_launch( __half* xout, float* partial, const __half* x, const __half* w, uint64_t s, uint64_t r, uint64_t b, int epilogue, hipStream_t st )
 {
   TileOrder ord;
   const uint32_t tile_rows = tile256_rows( s, r, b );
@@ -431,19 +452,18 @@ int gemm_tile256_launch( __half* xout, float* partial, const __half* x, const __
   ord.rest_share = (uint32_t)rest_share;
   const dim3 grid( (unsigned)gx ), block( T256_THREADS );
   const uint32_t s32 = (uint32_t)s, r32 = (uint32_t)r, b32 = (uint32_t)b;
-  if ( tile_rows == 384 ) {
-    if ( partial != nullptr ) {
-      gemm_tile256_kernel<true, 3><<<grid, block, 0, st>>>( xout, partial, x, w, s32, r32, b32, ord );
-    } else {
-      gemm_tile256_kernel<false, 3><<<grid, block, 0, st>>>( xout, partial, x, w, s32, r32, b32, ord );
-    }
-  } else {
-    if ( partial != nullptr ) {
-      gemm_tile256_kernel<true, 2><<<grid, block, 0, st>>>( xout, partial, x, w, s32, r32, b32, ord );
-    } else {
-      gemm_tile256_kernel<false, 2><<<grid, block, 0, st>>>( xout, partial, x, w, s32, r32, b32, ord );
-    }
+  const int epi = partial != nullptr ? EPI_PARTIAL : epilogue;
+  GH_REQUIRE( epi == EPI_STORE || epi == EPI_ACCUM || epi == EPI_PARTIAL, "gh_matmul: unknown tile epilogue %d", epi );
+  GH_REQUIRE( epi != EPI_ACCUM || r % 8 == 0, "gh_matmul: the accumulating tile epilogue needs r %% 8 == 0" );
+#define GH_TILE256_LAUNCH( E, N ) gemm_tile256_kernel<E, N><<<grid, block, 0, st>>>( xout, partial, x, w, s32, r32, b32, ord )
+#define GH_TILE256_ROWS( E ) ( tile_rows == 384 ? GH_TILE256_LAUNCH( E, 3 ) : GH_TILE256_LAUNCH( E, 2 ) )
+  switch ( epi ) {
+    case EPI_STORE: GH_TILE256_ROWS( EPI_STORE ); break;
+    case EPI_ACCUM: GH_TILE256_ROWS( EPI_ACCUM ); break;
+    default: GH_TILE256_ROWS( EPI_PARTIAL ); break;
   }
+#undef GH_TILE256_ROWS
+#undef GH_TILE256_LAUNCH
   GH_LAUNCH_CHECK();
   return GH_OK;
 }

@@ -386,6 +386,8 @@ public:
 
     const gh_shape shape = LlamaOperations::shape();
     const uint64_t row_bytes = 2ull * Config::kv_dim * sizeof( DType );
+    const bool fuse_wo = n <= 65535 && gh_matmul_fuses_many_rows( Config::dim, Config::dim, n, hip::gh_type<DType>() ) == 1;
+    const bool fuse_w2 = n <= 65535 && gh_matmul_fuses_many_rows( Config::hidden_dim, Config::dim, n, hip::gh_type<DType>() ) == 1;
     ops_.template rmsnorm<Config::dim>( pxb, px, reinterpret_cast<float32_t*>( temp_ ), layers_[run[0]].rms_att_weight, n );
     for ( size_t k = 0; k < run.size(); k++ ) {
       const auto& w = layers_[run[k]];
@@ -413,16 +415,27 @@ public:
                            hip::gh_type<DType>(), ops_.stream() ) );
         GLINT_GH( gh_attn_prefill( pq, layer_rows_dev( k ), pos_dev(), pxb, batch, n_tokens, max_start, &shape, hip::gh_type<DType>(), pf_attn_ws_.get(),
                                    pf_attn_ws_bytes_, GH_ATTN_AUTO, ops_.stream() ) );
-        ops_.template matmul<Config::dim, Config::dim>( pxb2, pxb, w.wo, n );
-        ops_.template accum<Config::dim>( px, pxb2, n );
-        ops_.template rmsnorm<Config::dim>( pxb, px, reinterpret_cast<float32_t*>( temp_ ), w.rms_ffn_weight, n );
+        // the residual add rides in the tile kernel's epilogue where the library does that for the shape
+        // (same roundings as the separate op); elsewhere the ops stay separate kernels
+        if ( fuse_wo ) {
+          ops_.template matmul_accum<Config::dim, Config::dim>( px, pxb, w.wo, n, pxb, w.rms_ffn_weight );
+        } else {
+          ops_.template matmul<Config::dim, Config::dim>( pxb2, pxb, w.wo, n );
+          ops_.template accum<Config::dim>( px, pxb2, n );
+          ops_.template rmsnorm<Config::dim>( pxb, px, reinterpret_cast<float32_t*>( temp_ ), w.rms_ffn_weight, n );
+        }
         ops_.template matmul<Config::dim, Config::hidden_dim>( phb, pxb, w.w1, n );
         ops_.template matmul<Config::dim, Config::hidden_dim>( phb2, pxb, w.w3, n );
         ops_.template silu<Config::hidden_dim>( phb, phb2, n );
-        ops_.template matmul<Config::hidden_dim, Config::dim>( pxb, phb, w.w2, n );
-        ops_.template accum<Config::dim>( px, pxb, n );
-        if ( k + 1 < run.size() ) {
-          ops_.template rmsnorm<Config::dim>( pxb, px, reinterpret_cast<float32_t*>( temp_ ), layers_[run[k + 1]].rms_att_weight, n );
+        const DType* next_norm = k + 1 < run.size() ? layers_[run[k + 1]].rms_att_weight : nullptr;
+        if ( fuse_w2 ) {
+          ops_.template matmul_accum<Config::hidden_dim, Config::dim>( px, phb, w.w2, n, next_norm ? pxb : nullptr, next_norm );
+        } else {
+          ops_.template matmul<Config::hidden_dim, Config::dim>( pxb, phb, w.w2, n );
+          ops_.template accum<Config::dim>( px, pxb, n );
+          if ( next_norm != nullptr ) {
+            ops_.template rmsnorm<Config::dim>( pxb, px, reinterpret_cast<float32_t*>( temp_ ), next_norm, n );
+          }
         }
       }
     }

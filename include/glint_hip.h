@@ -134,6 +134,9 @@ int gh_argmax( uint32_t* out_host, uint32_t* out_dev, const void* v, uint64_t n,
  * streaming kernel's K split is balanced for (<= 0 keeps the current value; the default is the device's own count); weight rows per work-group of the
  * 256-token tile kernel: 256, 384, or 0 for the library's choice */
 int gh_gemm_set_tuning( int kernel, int target_workgroups, int tile_rows );
+/* host-only query: 1 when gh_matmul_accum runs a product of this shape (16-byte aligned operands) in the large tile kernel with the residual added
+ * in its epilogue, i.e. without fp32 partial sums of (b, r): the caller's test for taking the fused call on many rows */
+int gh_matmul_fuses_many_rows( uint64_t s, uint64_t r, uint64_t b, gh_dtype dt );
 /* host-only query: how the weight-streaming kernel would cut an (r x s) . (b x s)^T product for the initialised device (256 compute
  * units before initialisation): number of K ranges, k per range (a multiple of 256), weight rows per work-group */
 int gh_gemm_stream_plan( uint64_t s, uint64_t r, uint64_t b, uint32_t* splits, uint32_t* k_per_split, uint32_t* rows_per_workgroup );

@@ -20,7 +20,10 @@ def _init():
 @pytest.mark.parametrize("dt", [torch.float16, torch.float32])
 @pytest.mark.parametrize("b,s,r", [(4, 288, 288), (64, 1024, 512), (5, 768, 1000), (3, 100, 36),
                                    # more rows than one streaming slab: the tile kernels write the partials
-                                   (100, 512, 260), (256, 1024, 512), (300, 4096, 1000), (768, 8192, 16384)])
+                                   (100, 512, 260), (256, 1024, 512), (300, 4096, 1000),
+                                   # enough 256-token tiles: the residual is added in the large tile kernel's epilogue (f16, r % 8 == 0)
+                                   (768, 8192, 16384), (2048, 512, 6152), (3000, 1024, 6144),
+                                   (2048, 512, 6150)])          # r % 8 != 0: fp32 partials and the row kernel
 def test_matmul_accum_and_norm(dt, b, s, r):
     g = torch.Generator(device="cuda").manual_seed(1)
     x = torch.randn((b, s), generator=g, device="cuda").to(dt)
