@@ -106,6 +106,7 @@ SIGNATURES = {
     "gh_attn_set_chunk": (_i, [_u32]),
     "gh_attn_set_auto_variant": (_i, [_i]),
     "gh_attn_decode_workspace": (_u64, [_u64, _u32, _shp]),
+    "gh_attn_decode_plan": (_i, [_u64, _u32, _shp, _i, _i, C.POINTER(_u32), C.POINTER(_u32), C.POINTER(_u64)]),
     "gh_attn_decode": (_i, [_vp, _vp, _vp, _vp, _u64, _u32, _shp, _i, _vp, _u64, _i, _vp]),
     "gh_attn_decode_host": (_i, [_vp, _vp, _vp, _vp, _u64, _shp, _i, _vp, _u64, _i, _vp]),
     "gh_prefill_tables": (_i, [_vp, _vp, _u64, _u32, _u64, _vp, _vp, _vp, _vp]),

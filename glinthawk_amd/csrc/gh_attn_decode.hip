@@ -68,7 +68,7 @@ __global__ __launch_bounds__( 64 ) void attn_decode_generic_kernel( const T* __r
   if ( base == nullptr ) {
     return;
   }
-  const uint32_t n_tok = pos[ctx] + 1;
+  const uint32_t n_tok = min( pos[ctx] + 1, max_splits * chunk ); // never beyond what the host sized the grid and the partials for
   const uint32_t t_begin = split * chunk;
   if ( t_begin >= n_tok ) {
     return;
@@ -163,7 +163,8 @@ __global__ __launch_bounds__( 256 ) void attn_merge_kernel( Partials part,
   if ( layer_rows[ctx] == nullptr ) {
     return;
   }
-  const uint32_t n_splits = ( pos[ctx] + chunk ) / chunk; // ceil((pos + 1) / chunk)
+  // ceil((pos + 1) / chunk); a position beyond the host's bound must not walk into the partials of the next head
+  const uint32_t n_splits = min( ( pos[ctx] + chunk ) / chunk, max_splits );
   const uint64_t slot0 = ( (uint64_t)ctx * n_heads + head ) * max_splits;
   float m = -INFINITY;
   for ( uint32_t s = 0; s < n_splits; s++ ) {
@@ -211,7 +212,7 @@ __device__ __forceinline__ WaveJob wave_job( const __half* const* layer_rows,
   j.ctx = bid / max_splits;
   j.h = hg * 4 + wave;
   j.base = layer_rows[j.ctx];
-  const uint32_t n_tok = pos[j.ctx] + 1;
+  const uint32_t n_tok = min( pos[j.ctx] + 1, max_splits * chunk ); // never beyond what the host sized the grid and the partials for
   j.t_begin = j.split * chunk;
   j.t_end = min( n_tok, j.t_begin + chunk );
   j.valid = j.h < n_kv_heads && j.base != nullptr && j.t_begin < n_tok;
@@ -761,11 +762,34 @@ uint64_t gh_attn_decode_workspace( uint64_t batch, uint32_t max_pos, const gh_sh
   if ( shape == nullptr || batch == 0 ) {
     return 0;
   }
-  // the generic kernel splits per query head and may use more splits than the fast ones; size for the larger
-  const Plan a = make_plan( batch, max_pos, shape, GH_F16, GH_ATTN_AUTO );
-  const Plan b = make_plan( batch, max_pos, shape, GH_F32, GH_ATTN_GENERIC );
-  const uint32_t splits = std::max( a.split_bound, b.split_bound );
-  return partial_floats( batch, shape, splits ) * sizeof( float ) + 256;
+  // A smaller batch gets more splits per context, and batch * splits does not grow with the batch:
+  // the buffer has to hold the largest need of any batch in [1, batch].  The generic kernel splits
+  // per query head and may use more splits than the fast ones; size for the larger of the two.
+  uint64_t floats = 0;
+  for ( uint64_t b = 1; b <= batch; b++ ) {
+    const Plan fast = make_plan( b, max_pos, shape, GH_F16, GH_ATTN_AUTO );
+    const Plan generic = make_plan( b, max_pos, shape, GH_F32, GH_ATTN_GENERIC );
+    floats = std::max( floats, partial_floats( b, shape, std::max( fast.split_bound, generic.split_bound ) ) );
+  }
+  return floats * sizeof( float ) + 256;
+}
+
+int gh_attn_decode_plan( uint64_t batch, uint32_t max_pos, const gh_shape* shape, gh_dtype dt, int variant, uint32_t* tokens_per_split, uint32_t* max_splits,
+                         uint64_t* partial_bytes )
+{
+  GH_REQUIRE( shape != nullptr && batch > 0, "gh_attn_decode_plan: bad arguments" );
+  GH_REQUIRE( variant >= GH_ATTN_AUTO && variant <= GH_ATTN_MFMA, "gh_attn_decode_plan: unknown variant %d", variant );
+  const Plan plan = make_plan( batch, max_pos, shape, dt, variant );
+  if ( tokens_per_split ) {
+    *tokens_per_split = plan.chunk;
+  }
+  if ( max_splits ) {
+    *max_splits = plan.max_splits;
+  }
+  if ( partial_bytes ) {
+    *partial_bytes = plan.max_splits > 1 ? partial_floats( batch, shape, plan.max_splits ) * sizeof( float ) : 0;
+  }
+  return GH_OK;
 }
 
 int gh_attn_decode( const void* q, const void* const* layer_rows_dev, const uint32_t* pos_dev, void* xb, uint64_t batch,

@@ -197,7 +197,8 @@ int gh_attn_pv_host( const void* att, const void* const* layer_rows_host, void* 
  * q must already be rotated (gh_rope) and the current row appended (gh_kv_append).
  *   layer_rows_dev[i]  base of context i's rows for this layer (NULL: skipped, xb row untouched)
  *   pos_dev[i]         position of the current token; keys [0, pos_i] are attended
- *   max_pos            host-side upper bound of pos (sizes the grid; seq_len - 1 if unknown)
+ *   max_pos            host-side upper bound of pos (sizes the grid; seq_len - 1 if unknown); a context whose position lies
+ *                      beyond it is attended over the keys the grid covers only, never outside the workspace
  *   workspace          device scratch of at least gh_attn_decode_workspace() bytes
  *   variant            GH_ATTN_AUTO, or force a kernel (tests / measurements) */
 typedef enum gh_attn_variant
@@ -212,7 +213,12 @@ typedef enum gh_attn_variant
 int gh_attn_set_chunk( uint32_t tokens_per_split );
 /* measurement hook: which kernel GH_ATTN_AUTO picks where the shape permits it (GH_ATTN_AUTO restores the library's choice) */
 int gh_attn_set_auto_variant( int variant );
+/* bytes that serve every call with at most `batch` rows and positions up to `max_pos` (a smaller batch is cut into more splits per context, so the
+ * largest need over all batch sizes in [1, batch] is returned) */
 uint64_t gh_attn_decode_workspace( uint64_t batch, uint32_t max_pos, const gh_shape* shape );
+/* host-only query: how gh_attn_decode would cut this call (tokens per split, splits of the longest context) and the workspace bytes it would use */
+int gh_attn_decode_plan( uint64_t batch, uint32_t max_pos, const gh_shape* shape, gh_dtype dt, int variant, uint32_t* tokens_per_split, uint32_t* max_splits,
+                         uint64_t* partial_bytes );
 int gh_attn_decode( const void* q, const void* const* layer_rows_dev, const uint32_t* pos_dev, void* xb, uint64_t batch,
                     uint32_t max_pos, const gh_shape* shape, gh_dtype dt, void* workspace, uint64_t workspace_bytes,
                     int variant, gh_stream stream );
