@@ -649,6 +649,17 @@ void glint_state_set_prompt( void* h, uint32_t i, const uint8_t prompt_id[32], u
 void glint_state_discard( void* h, uint32_t i ) { as_state( h )->discard( i ); }
 void glint_state_set_finished( void* h, uint32_t i ) { as_state( h )->set_finished( i ); }
 int glint_state_check_finished( void* h, uint32_t i ) { return as_state( h )->check_finished( i ) ? 1 : 0; }
+// host-only: the stage driver's position check (positions_fit) on this state, with a slot for every active row and the shared empty
+// context for the others, as the context manager hands them out
+int glint_state_positions_fit( void* h, uint64_t seq_len )
+{
+  const auto settings = StageSettings<configs::Test_Tiny>::slice( 0, 1, 1024, 1024 );
+  std::vector<std::shared_ptr<EchoContext>> contexts;
+  for ( size_t i = 0; i < as_state( h )->batch_size(); i++ ) {
+    contexts.push_back( std::make_shared<EchoContext>( settings, !as_state( h )->active( i ) ) );
+  }
+  return positions_fit( *as_state( h ), contexts, seq_len ) ? 1 : 0;
+}
 uint64_t glint_state_free_slots( void* h ) { return as_state( h )->free_slots(); }
 uint32_t glint_state_batch_size( void* h ) { return as_state( h )->batch_size(); }
 int glint_state_all_assigned( void* h ) { return as_state( h )->all_assigned_to_nodes() ? 1 : 0; }

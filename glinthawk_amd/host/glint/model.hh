@@ -64,6 +64,20 @@ struct WeightLayout
   }
 };
 
+// Positions arrive in a state that was parsed from the wire unvalidated.  A row of a non-empty context
+// at or beyond seq_len would address cache rows and RoPE table entries past their allocations, so every
+// entry point that turns positions into addresses checks this on the host before anything is launched.
+template<typename State, typename ContextVector>
+bool positions_fit( const State& states, const ContextVector& contexts, const uint64_t seq_len )
+{
+  for ( size_t i = 0; i < contexts.size() && i < states.batch_size(); i++ ) {
+    if ( !contexts[i]->empty() && states.token_pos( i ) >= seq_len ) {
+      return false;
+    }
+  }
+  return true;
+}
+
 // glint/loader.hh: copies the hosted tensors out of the reference's model directory
 template<typename Model>
 std::string load_model_dir( Model& model, const std::filesystem::path& model_dir );
@@ -183,6 +197,7 @@ public:
   void forward( StateType& states, const ContextVector& contexts )
   {
     check_batch( states, contexts.size(), InferenceStage::PreAttention );
+    GLINT_CHECK( positions_fit( states, contexts, Config::seq_len ) );
     batch_ = states.batch_size();
     const uint32_t first = states.next_layer();
 
@@ -263,6 +278,7 @@ public:
   void forward_attention( StateType& states, const ContextVector& contexts )
   {
     check_batch( states, contexts.size(), InferenceStage::Attention );
+    GLINT_CHECK( positions_fit( states, contexts, Config::seq_len ) );
     batch_ = states.batch_size();
     const uint32_t l = states.next_layer();
     for ( size_t i = 0; i < states.batch_size(); i++ ) {
@@ -665,6 +681,7 @@ private:
     for ( size_t i = 0; i < batch_; i++ ) {
       pos[i] = token_positions_[i];
       if ( !contexts[i]->empty() ) {
+        GLINT_CHECK( token_positions_[i] < Config::seq_len );
         max_pos_ = std::max( max_pos_, token_positions_[i] );
       }
     }

@@ -96,6 +96,7 @@ def _lib():
             "glint_state_discard": (None, [vp, u32]),
             "glint_state_set_finished": (None, [vp, u32]),
             "glint_state_check_finished": (i, [vp, u32]),
+            "glint_state_positions_fit": (i, [vp, u64]),
             "glint_state_free_slots": (u64, [vp]),
             "glint_state_batch_size": (u32, [vp]),
             "glint_state_all_assigned": (i, [vp]),
@@ -157,6 +158,10 @@ class HostState:
 
     def check_finished(self, i) -> bool:
         return bool(_lib().glint_state_check_finished(self._h, i))
+
+    def positions_fit(self, seq_len: int) -> bool:
+        """The stage driver's host-side check of the rows' positions against the context window."""
+        return bool(_lib().glint_state_positions_fit(self._h, seq_len))
 
     def free_slots(self) -> int:
         return _lib().glint_state_free_slots(self._h)

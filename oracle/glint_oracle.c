@@ -34,7 +34,7 @@
  *   go_ctx_* addressing                   brute force enumeration on small shapes; disjointness
  *   go_dynctx_prepare                     brute-force page model (set of committed blocks)
  *   go_ctxman_*                           random op sequences vs a dict + deque model
- *   go_check_finished, temperature codec  exhaustive truth table on small ranges
+ *   go_check_finished, temperature codec  hand-derived literal cases (incl. eot != eos); exhaustive codec table
  *
  * What stays unpinned bit-for-bit: the last-ulp effect of the reference's -ffast-math build
  * (compiler specific) and the exact fp16 rounding sequence inside softmax for DType = _Float16

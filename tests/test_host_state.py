@@ -133,6 +133,29 @@ def test_check_finished(token, pos, plen, mcl, want):
     assert s.check_finished(0) == want
 
 
+def test_positions_beyond_the_window_are_refused_before_any_launch():
+    """A position parsed from the wire is not trusted: the stage driver's forward entry points check
+    every row that owns a context slot against seq_len on the host (rows past the window would address
+    cache rows and RoPE table entries outside their allocations).  Inactive rows hold the shared empty
+    context, which every op skips, so their positions do not matter."""
+    seq = HostState.SEQ_LEN
+    s = HostState(3, "f16")
+    s.set_prompt(0, b"a" * 32, 1, 5, 0, 0.0, 1, 0, 0, 0)
+    s.set_prompt(1, b"b" * 32, 2, 5, seq - 1, 0.0, 1, 0, 0, 0)
+    assert s.positions_fit(seq)
+    s.set_prompt(2, b"c" * 32, 3, 5, seq, 0.0, 1, 0, 0, 0)
+    assert not s.positions_fit(seq)
+    assert s.positions_fit(seq + 1)
+    # the same through the wire: parse() accepts the bytes, the check refuses the state
+    back = HostState.parse(s.serialize())
+    assert not back.positions_fit(seq)
+    s.discard(2)                                   # an inactive row is never addressed
+    assert s.positions_fit(seq)
+    huge = HostState(1, "f16")
+    huge.set_prompt(0, b"d" * 32, 1, 5, 0xFFFFFFFF, 0.0, 1, 0, 0, 0)
+    assert not huge.positions_fit(seq)
+
+
 def fill(state: HostState, prompts: np.ndarray, rng, which=(0, 2)):
     for i, r in enumerate(prompts):
         if r["active"]:

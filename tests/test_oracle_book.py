@@ -145,11 +145,35 @@ def test_context_manager_documented_cases():
     assert m.release(7) and m.get_contexts([1], [5]) == [0]     # FIFO reuse of the released slot
 
 
-def test_check_finished_truth_table():
-    seq = 16
-    for token, pos, plen, mcl in itertools.product([0, 2, 3], range(0, 20), [0, 3], [0, 5]):
-        want = (mcl == 0 and token == 2) or pos >= seq or (mcl > 0 and pos >= mcl + plen)
-        assert O.check_finished(token, pos, plen, mcl, seq) == want
+# (token, token_pos, prompt_length, max_completion_length, seq_len, eos, eot) -> finished, each case worked out by hand from the
+# three clauses of models/common/state.hh:621-631: an end token only counts while no completion length is set; the position
+# bound is `>=`; the completion bound is `>= max_completion_length + prompt_length` and only exists when a length is set.
+CHECK_FINISHED_CASES = [
+    ((5, 3, 2, 0, 16, 2, 9), False),     # ordinary token, inside the window, no length limit
+    ((2, 3, 2, 0, 16, 2, 9), True),      # end of sentence, no length limit
+    ((9, 3, 2, 0, 16, 2, 9), True),      # end of turn (a different id than eos), no length limit
+    ((2, 3, 2, 7, 16, 2, 9), False),     # eos is ignored once a completion length is set ...
+    ((9, 3, 2, 7, 16, 2, 9), False),     # ... and so is eot
+    ((5, 15, 2, 0, 16, 2, 9), False),    # last position of the window
+    ((5, 16, 2, 0, 16, 2, 9), True),     # position == seq_len
+    ((5, 17, 2, 0, 16, 2, 9), True),     # beyond it
+    ((5, 8, 2, 7, 16, 2, 9), False),     # 8 < 7 + 2
+    ((5, 9, 2, 7, 16, 2, 9), True),      # 9 >= 7 + 2
+    ((5, 10, 2, 7, 16, 2, 9), True),
+    ((5, 6, 0, 7, 16, 2, 9), False),     # no prompt: the limit is the completion length alone
+    ((5, 7, 0, 7, 16, 2, 9), True),
+    ((5, 0, 0, 0, 16, 2, 9), False),     # a length of 0 means "no limit", not "finished at once"
+    ((2, 16, 2, 7, 16, 2, 9), True),     # out of the window wins although eos is ignored
+    ((5, 15, 10, 7, 16, 2, 9), False),   # 15 < 17 and 15 < 16
+    ((0, 0, 0, 0, 1, 2, 9), False),      # a window of one position: position 0 is inside
+    ((0, 1, 0, 0, 1, 2, 9), True),
+    ((9, 3, 2, 0, 16, 2, 2), False),     # token 9 is no end token when eot == eos == 2 (the Llama2 configs)
+]
+
+
+def test_check_finished_hand_derived_cases():
+    for (token, pos, plen, mcl, seq, eos, eot), want in CHECK_FINISHED_CASES:
+        assert O.check_finished(token, pos, plen, mcl, seq, token_eos=eos, token_eot=eot) == want, (token, pos, plen, mcl, seq, eos, eot)
 
 
 def test_temperature_codec():
