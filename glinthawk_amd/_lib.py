@@ -71,7 +71,7 @@ SIGNATURES = {
     "gh_memset_zero": (_i, [_vp, _u64, _vp]),
     "gh_fill_uniform": (_i, [_vp, _u64, _f, _f, _u64, _i, _vp]),
     "gh_fill_normal": (_i, [_vp, _u64, _f, _f, _u64, _i, _vp]),
-    "gh_convert_and_copy": (_i, [_vp, _i, _vp, _i, _u64, _i]),
+    "gh_convert_and_copy": (_i, [_vp, _i, _vp, _i, _u64, _i, _vp]),
     "gh_convert": (_i, [_vp, _i, _vp, _i, _u64, _vp]),
     "gh_vmm_granularity": (_i, [C.POINTER(_u64)]),
     "gh_vmm_reserve": (_i, [C.POINTER(_vp), _u64]),

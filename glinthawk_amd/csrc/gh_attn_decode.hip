@@ -914,6 +914,7 @@ int gh_attn_decode_host( const void* q, const void* const* layer_rows_host, cons
   }
   void* d_rows = nullptr;
   void* d_pos = nullptr;
+  StageScope scope( as_stream( stream ) );
   if ( int rc = stage_table( layer_rows_host, batch * sizeof( void* ), as_stream( stream ), &d_rows ) ) {
     return rc;
   }
@@ -924,7 +925,7 @@ int gh_attn_decode_host( const void* q, const void* const* layer_rows_host, cons
                                 workspace, workspace_bytes, variant, stream ) ) {
     return rc;
   }
-  return stage_fence( as_stream( stream ) );
+  return scope.finish();
 }
 
 } // extern "C"

@@ -313,13 +313,14 @@ int gh_attn_scores_host( const void* q, const void* const* layer_rows_host, void
   GH_REQUIRE( layer_rows_host && pos_host, "gh_attn_scores_host: NULL table" );
   const void* const* d_rows = nullptr;
   const uint32_t* d_pos = nullptr;
+  StageScope scope( as_stream( stream ) );
   if ( int rc = stage_rows_and_pos( layer_rows_host, pos_host, batch, as_stream( stream ), &d_rows, &d_pos, "gh_attn_scores_host" ) ) {
     return rc;
   }
   if ( int rc = gh_attn_scores( q, d_rows, att, batch, d_pos, shape, dt, stream ) ) {
     return rc;
   }
-  return stage_fence( as_stream( stream ) );
+  return scope.finish();
 }
 
 int gh_attn_softmax_host( void* att, const uint32_t* pos_host, uint64_t batch, const gh_shape* shape, gh_dtype dt, gh_stream stream )
@@ -333,13 +334,14 @@ int gh_attn_softmax_host( void* att, const uint32_t* pos_host, uint64_t batch, c
   GH_REQUIRE( pos_host, "gh_attn_softmax_host: NULL table" );
   const void* const* d_rows = nullptr;
   const uint32_t* d_pos = nullptr;
+  StageScope scope( as_stream( stream ) );
   if ( int rc = stage_rows_and_pos( nullptr, pos_host, batch, as_stream( stream ), &d_rows, &d_pos, "gh_attn_softmax_host" ) ) {
     return rc;
   }
   if ( int rc = gh_attn_softmax( att, d_pos, batch, shape, dt, stream ) ) {
     return rc;
   }
-  return stage_fence( as_stream( stream ) );
+  return scope.finish();
 }
 
 int gh_attn_pv_host( const void* att, const void* const* layer_rows_host, void* xb, uint64_t batch, const uint32_t* pos_host,
@@ -354,13 +356,14 @@ int gh_attn_pv_host( const void* att, const void* const* layer_rows_host, void* 
   GH_REQUIRE( layer_rows_host && pos_host, "gh_attn_pv_host: NULL table" );
   const void* const* d_rows = nullptr;
   const uint32_t* d_pos = nullptr;
+  StageScope scope( as_stream( stream ) );
   if ( int rc = stage_rows_and_pos( layer_rows_host, pos_host, batch, as_stream( stream ), &d_rows, &d_pos, "gh_attn_pv_host" ) ) {
     return rc;
   }
   if ( int rc = gh_attn_pv( att, d_rows, xb, batch, d_pos, shape, dt, stream ) ) {
     return rc;
   }
-  return stage_fence( as_stream( stream ) );
+  return scope.finish();
 }
 
 } // extern "C"

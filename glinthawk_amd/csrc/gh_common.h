@@ -49,11 +49,43 @@ inline size_t dtype_size( gh_dtype dt ) { return dt == GH_F32 ? 4 : 2; }
 
 // ---- staging of host-side pointer / position tables ------------------------------------------
 // Copies `bytes` from a host array into a slot of a device-side ring (via pinned memory) on
-// `stream` and returns the device address.  A slot is reused only after the work that was queued
-// behind its previous use has finished.
+// `stream` and returns the device address; a table identical to one staged a moment ago on the same
+// stream gets that slot again without a copy.  A slot is rewritten only after the work that was
+// queued behind its last use has finished, and never between being handed out and the fence.
 int stage_table( const void* host_src, size_t bytes, hipStream_t stream, void** dev_out );
-// Marks the end of the work that reads the most recently staged slots on this stream.
+// Marks the end of the work that reads the slots handed out on this stream since its last fence.
 int stage_fence( hipStream_t stream );
+// Fences on every way out of an entry point that staged tables, also when the op in between failed.
+class StageScope
+{
+  hipStream_t stream_;
+  bool done_ = false;
+
+public:
+  explicit StageScope( hipStream_t stream )
+    : stream_( stream )
+  {
+  }
+  StageScope( const StageScope& ) = delete;
+  StageScope& operator=( const StageScope& ) = delete;
+  ~StageScope()
+  {
+    if ( !done_ ) {
+      (void)stage_fence( stream_ );
+    }
+  }
+  int finish()
+  {
+    done_ = true;
+    return stage_fence( stream_ );
+  }
+};
+
+// ---- library-owned device scratch ---------------------------------------------------------------
+// Grow-only buffer for purpose `which`, private to `stream`: work queued on different streams never
+// shares one.  Growing waits for that stream only.  `min_bytes` is the size of the first allocation.
+enum { SCRATCH_GEMM_PARTIALS = 0, SCRATCH_CONVERT = 1 };
+int stream_scratch( hipStream_t stream, int which, uint64_t bytes, uint64_t min_bytes, void** out );
 
 // Three events per sampled attention call when the benchmark's timer is enabled (slot == -1: off):
 // before the split-K kernel, between it and the merge kernel, after the merge kernel.

@@ -409,6 +409,7 @@ int gh_soft_sample( void* v, const float* temperatures, uint64_t vocab, uint64_t
     return GH_OK; // greedy rows are untouched, as in the reference
   }
   void* d_temps = nullptr;
+  StageScope scope( as_stream( stream ) );
   if ( int rc = stage_table( temperatures, batch * sizeof( float ), as_stream( stream ), &d_temps ) ) {
     return rc;
   }
@@ -416,7 +417,7 @@ int gh_soft_sample( void* v, const float* temperatures, uint64_t vocab, uint64_t
   GH_DISPATCH_DT( dt, gumbel_kernel<T><<<grid, EW_THREADS, 0, as_stream( stream )>>>(
                         static_cast<T*>( v ), static_cast<const float*>( d_temps ), (uint32_t)vocab, seed ) );
   GH_LAUNCH_CHECK();
-  return stage_fence( as_stream( stream ) );
+  return scope.finish();
 }
 
 int gh_fill_uniform( void* dst, uint64_t n, float lo, float hi, uint64_t seed, gh_dtype dt, gh_stream stream )
@@ -493,8 +494,9 @@ int gh_convert( void* dst, gh_dtype dst_dt, const void* src, gh_dtype src_dt, ui
 }
 
 // LlamaOperations::convert_and_copy: the conversion runs on the side that is the device; the host
-// side only sees a byte copy of its own dtype.
-int gh_convert_and_copy( void* dst, gh_dtype dst_dt, const void* src, gh_dtype src_dt, uint64_t n, gh_copy_kind kind )
+// side only sees a byte copy of its own dtype.  Everything is queued on the caller's stream, which
+// is waited for before the call returns (the reference's conversion is synchronous).
+int gh_convert_and_copy( void* dst, gh_dtype dst_dt, const void* src, gh_dtype src_dt, uint64_t n, gh_copy_kind kind, gh_stream stream )
 {
   if ( int rc = ensure_init() ) {
     return rc;
@@ -504,35 +506,40 @@ int gh_convert_and_copy( void* dst, gh_dtype dst_dt, const void* src, gh_dtype s
   }
   GH_REQUIRE( dst && src, "gh_convert_and_copy: NULL pointer" );
   GH_REQUIRE( ( dst_dt == GH_F16 || dst_dt == GH_F32 ) && ( src_dt == GH_F16 || src_dt == GH_F32 ), "gh_convert_and_copy: unsupported dtype" );
+  GH_REQUIRE( kind == GH_HOST_TO_DEVICE || kind == GH_DEVICE_TO_HOST || kind == GH_DEVICE_TO_DEVICE || kind == GH_HOST_TO_HOST,
+              "gh_convert_and_copy: bad copy kind %d", (int)kind );
   if ( dst_dt == src_dt ) {
-    return gh_memcpy( dst, src, n * dtype_size( dst_dt ), kind, 0, nullptr );
+    return gh_memcpy( dst, src, n * dtype_size( dst_dt ), kind, 0, stream );
   }
+  hipStream_t st = as_stream( stream );
   if ( kind == GH_DEVICE_TO_DEVICE ) {
-    if ( int rc = gh_convert( dst, dst_dt, src, src_dt, n, nullptr ) ) {
+    if ( int rc = gh_convert( dst, dst_dt, src, src_dt, n, stream ) ) {
       return rc;
     }
-    GH_HIP( hipStreamSynchronize( nullptr ) );
+    GH_HIP( hipStreamSynchronize( st ) );
     return GH_OK;
   }
-  GH_REQUIRE( kind == GH_HOST_TO_DEVICE || kind == GH_DEVICE_TO_HOST, "gh_convert_and_copy: bad copy kind for a converting copy" );
+  // a device target never converts host memory into host memory (LOG(FATAL) "Invalid copy type" in arch/cuda/llama2/ops.cuh:490)
+  GH_REQUIRE( kind != GH_HOST_TO_HOST, "gh_convert_and_copy: a converting copy needs a device side" );
   void* tmp = nullptr;
-  if ( kind == GH_HOST_TO_DEVICE ) {
-    GH_HIP( hipMalloc( &tmp, n * dtype_size( src_dt ) ) );
-    int rc = gh_memcpy( tmp, src, n * dtype_size( src_dt ), GH_HOST_TO_DEVICE, 0, nullptr );
-    if ( rc == GH_OK ) {
-      rc = gh_convert( dst, dst_dt, tmp, src_dt, n, nullptr );
-    }
-    (void)hipStreamSynchronize( nullptr );
-    (void)hipFree( tmp );
+  const gh_dtype tmp_dt = kind == GH_HOST_TO_DEVICE ? src_dt : dst_dt;
+  if ( int rc = stream_scratch( st, SCRATCH_CONVERT, n * dtype_size( tmp_dt ), 4ull << 20, &tmp ) ) {
     return rc;
   }
-  GH_HIP( hipMalloc( &tmp, n * dtype_size( dst_dt ) ) );
-  int rc = gh_convert( tmp, dst_dt, src, src_dt, n, nullptr );
-  if ( rc == GH_OK ) {
-    rc = gh_memcpy( dst, tmp, n * dtype_size( dst_dt ), GH_DEVICE_TO_HOST, 0, nullptr );
+  if ( kind == GH_HOST_TO_DEVICE ) {
+    GH_HIP( hipMemcpyAsync( tmp, src, n * dtype_size( src_dt ), hipMemcpyHostToDevice, st ) );
+    if ( int rc = gh_convert( dst, dst_dt, tmp, src_dt, n, stream ) ) {
+      (void)hipStreamSynchronize( st );
+      return rc;
+    }
+  } else {
+    if ( int rc = gh_convert( tmp, dst_dt, src, src_dt, n, stream ) ) {
+      return rc;
+    }
+    GH_HIP( hipMemcpyAsync( dst, tmp, n * dtype_size( dst_dt ), hipMemcpyDeviceToHost, st ) );
   }
-  (void)hipFree( tmp );
-  return rc;
+  GH_HIP( hipStreamSynchronize( st ) );
+  return GH_OK;
 }
 
 } // extern "C"

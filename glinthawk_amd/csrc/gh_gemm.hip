@@ -44,25 +44,14 @@ constexpr int BM = 64;  // weight rows per work-group
 constexpr int BN = 64;  // batch columns per work-group
 constexpr int BK = 128; // k per stage (16 chunks of 8 halves)
 
-std::mutex g_ws_mutex;
-float* g_ws = nullptr; // split-K partials, grow-only
-uint64_t g_ws_bytes = 0;
-
-int ensure_workspace( uint64_t bytes, float** out )
+// split-K partials: a grow-only buffer per stream, so that products queued on different streams never share one
+int ensure_workspace( uint64_t bytes, float** out, hipStream_t st )
 {
-  std::lock_guard<std::mutex> lock( g_ws_mutex );
-  if ( bytes > g_ws_bytes ) {
-    if ( g_ws ) {
-      GH_HIP( hipDeviceSynchronize() );
-      GH_HIP( hipFree( g_ws ) );
-      g_ws = nullptr;
-      g_ws_bytes = 0;
-    }
-    const uint64_t want = std::max<uint64_t>( bytes, 64ull << 20 );
-    GH_HIP( hipMalloc( reinterpret_cast<void**>( &g_ws ), want ) );
-    g_ws_bytes = want;
+  void* p = nullptr;
+  if ( int rc = stream_scratch( st, SCRATCH_GEMM_PARTIALS, bytes, 64ull << 20, &p ) ) {
+    return rc;
   }
-  *out = g_ws;
+  *out = static_cast<float*>( p );
   return GH_OK;
 }
 
@@ -277,7 +266,7 @@ int gemm_partials( void* xout, const void* x, const void* w, uint64_t s, uint64_
   if ( dt == GH_F32 ) {
     float* dst = static_cast<float*>( xout );
     if ( want_partials ) {
-      if ( int rc = ensure_workspace( b * r * sizeof( float ), &dst ) ) {
+      if ( int rc = ensure_workspace( b * r * sizeof( float ), &dst, st ) ) {
         return rc;
       }
       *partial_out = dst;
@@ -294,7 +283,7 @@ int gemm_partials( void* xout, const void* x, const void* w, uint64_t s, uint64_
   if ( ( g_force_kernel == 0 || g_force_kernel == 4 ) && gemm_tile256_applicable( s, r, b, x, w, xout ? xout : x ) ) {
     float* ws = nullptr;
     if ( want_partials ) {
-      if ( int rc = ensure_workspace( b * r * sizeof( float ), &ws ) ) {
+      if ( int rc = ensure_workspace( b * r * sizeof( float ), &ws, st ) ) {
         return rc;
       }
       *partial_out = ws;
@@ -308,7 +297,7 @@ int gemm_partials( void* xout, const void* x, const void* w, uint64_t s, uint64_
     gemm_tile_plan( s, r, b, &splits, &k_per_split );
     float* ws = nullptr;
     if ( want_partials || splits > 1 ) {
-      if ( int rc = ensure_workspace( (uint64_t)splits * b * r * sizeof( float ), &ws ) ) {
+      if ( int rc = ensure_workspace( (uint64_t)splits * b * r * sizeof( float ), &ws, st ) ) {
         return rc;
       }
       *partial_out = ws;
@@ -324,7 +313,7 @@ int gemm_partials( void* xout, const void* x, const void* w, uint64_t s, uint64_
     float* ws = nullptr;
     const bool partial = want_partials || splits > 1;
     if ( partial ) {
-      if ( int rc = ensure_workspace( (uint64_t)splits * b * r * sizeof( float ), &ws ) ) {
+      if ( int rc = ensure_workspace( (uint64_t)splits * b * r * sizeof( float ), &ws, st ) ) {
         return rc;
       }
       *partial_out = ws;
@@ -360,7 +349,7 @@ int gemm_partials( void* xout, const void* x, const void* w, uint64_t s, uint64_
     return GH_OK;
   }
   float* ws = nullptr;
-  if ( int rc = ensure_workspace( (uint64_t)splits * b * r * sizeof( float ), &ws ) ) {
+  if ( int rc = ensure_workspace( (uint64_t)splits * b * r * sizeof( float ), &ws, st ) ) {
     return rc;
   }
   gemm_f16_kernel<true><<<grid, 256, 0, st>>>( nullptr, ws, static_cast<const __half*>( x ), static_cast<const __half*>( w ), (uint32_t)s, (uint32_t)r,

@@ -190,13 +190,14 @@ int gh_kv_append_host( void* const* token_rows_host, const void* state_kv, uint6
   GH_REQUIRE( token_rows_host, "gh_kv_append_host: NULL table" );
   GH_REQUIRE( batch <= MAX_BATCH, "gh_kv_append_host: batch %llu > %llu", (unsigned long long)batch, (unsigned long long)MAX_BATCH );
   void* d_rows = nullptr;
+  StageScope scope( as_stream( stream ) );
   if ( int rc = stage_table( token_rows_host, batch * sizeof( void* ), as_stream( stream ), &d_rows ) ) {
     return rc;
   }
   if ( int rc = gh_kv_append( static_cast<void* const*>( d_rows ), state_kv, batch, kv_dim, dt, stream ) ) {
     return rc;
   }
-  return stage_fence( as_stream( stream ) );
+  return scope.finish();
 }
 
 int gh_rope( uint64_t batch, const uint32_t* pos_dev, const void* freq_real, const void* freq_imag, void* q,
@@ -245,6 +246,7 @@ int gh_rope_host( uint64_t batch, const uint32_t* pos_host, const void* freq_rea
   GH_REQUIRE( batch <= MAX_BATCH, "gh_rope_host: batch %llu > %llu", (unsigned long long)batch, (unsigned long long)MAX_BATCH );
   void* d_rows = nullptr;
   void* d_pos = nullptr;
+  StageScope scope( as_stream( stream ) );
   if ( int rc = stage_table( token_rows_host, batch * sizeof( void* ), as_stream( stream ), &d_rows ) ) {
     return rc;
   }
@@ -255,7 +257,7 @@ int gh_rope_host( uint64_t batch, const uint32_t* pos_host, const void* freq_rea
                          n_kv_heads, gqa_size, head_size, dt, stream ) ) {
     return rc;
   }
-  return stage_fence( as_stream( stream ) );
+  return scope.finish();
 }
 
 } // extern "C"

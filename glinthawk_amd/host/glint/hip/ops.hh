@@ -300,7 +300,7 @@ public:
   template<typename DTypeDst, typename DTypeSrc>
   void convert_and_copy( DTypeDst* dst, const DTypeSrc* src, const uint64_t size, const CopyType type ) const
   {
-    GLINT_GH( gh_convert_and_copy( dst, gh_type<DTypeDst>(), src, gh_type<DTypeSrc>(), size, gh_kind( type ) ) );
+    GLINT_GH( gh_convert_and_copy( dst, gh_type<DTypeDst>(), src, gh_type<DTypeSrc>(), size, gh_kind( type ), this->stream_ ) );
   }
 
   // Extension used by the stage driver: attention_0_gemm + attention_softmax + attention_2_gemm in

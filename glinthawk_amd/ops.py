@@ -275,5 +275,33 @@ def pinned_empty(shape, dtype):
     return arr
 
 
+def _addr(buf) -> int:
+    """Address of a torch tensor (device or host) or of a numpy array."""
+    if isinstance(buf, torch.Tensor):
+        assert buf.is_contiguous()
+        return buf.data_ptr()
+    assert buf.flags["C_CONTIGUOUS"]
+    return buf.ctypes.data
+
+
+def _dt_any(buf) -> int:
+    name = str(buf.dtype).replace("torch.", "")
+    if name == "float16":
+        return GH_F16
+    if name == "float32":
+        return GH_F32
+    raise TypeError(f"unsupported dtype {buf.dtype}")
+
+
+def convert_and_copy(dst, src, n: int, kind: int) -> None:
+    """LlamaOperations::convert_and_copy: `n` elements from `src` to `dst` (torch device tensors or numpy host
+    arrays, as `kind` says), converted element by element when the two types differ."""
+    check(lib().gh_convert_and_copy(_addr(dst), _dt_any(dst), _addr(src), _dt_any(src), n, kind, _stream()), "gh_convert_and_copy")
+
+
+def convert(dst: torch.Tensor, src: torch.Tensor, n: int) -> None:
+    check(lib().gh_convert(_p(dst), _dt(dst), _p(src), _dt(src), n, _stream()), "gh_convert")
+
+
 def sync() -> None:
     check(lib().gh_sync(None), "gh_sync")

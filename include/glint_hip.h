@@ -99,9 +99,11 @@ int gh_fill_uniform( void* dst, uint64_t n, float lo, float hi, uint64_t seed, g
 /* synthetic inputs of the benchmark configs: N(mean, std) */
 int gh_fill_normal( void* dst, uint64_t n, float mean, float std, uint64_t seed, gh_dtype dt, gh_stream stream );
 
-/* LlamaOperations::convert_and_copy (arch/cuda/llama2/ops.cuh:455-492): n elements, static_cast per
- * element; dst/src may each be host or device as `kind` says.  Synchronous (the reference's is). */
-int gh_convert_and_copy( void* dst, gh_dtype dst_dt, const void* src, gh_dtype src_dt, uint64_t n, gh_copy_kind kind );
+/* LlamaOperations::convert_and_copy (arch/cuda/llama2/ops.cuh:455-492, arch/amd64/llama2/ops.hh:354-368): n elements,
+ * static_cast per element (f32 -> f16 rounds to nearest even, f16 -> f32 is exact); dst/src may each be host or device
+ * as `kind` says.  Queued on `stream` and waited for before returning (the reference's is synchronous).  A converting
+ * host-to-host copy is refused, as on the reference's device target. */
+int gh_convert_and_copy( void* dst, gh_dtype dst_dt, const void* src, gh_dtype src_dt, uint64_t n, gh_copy_kind kind, gh_stream stream );
 /* same conversion, device to device, asynchronous */
 int gh_convert( void* dst, gh_dtype dst_dt, const void* src, gh_dtype src_dt, uint64_t n, gh_stream stream );
 

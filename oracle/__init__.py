@@ -104,8 +104,9 @@ def _declare(L: C.CDLL) -> None:
         getattr(L, f"go_softmax_row_{sfx}").argtypes = [vp, u64]
         getattr(L, f"go_attention_ops_{sfx}").argtypes = [cfgp, u64, vp, vp, vp, vp, vp, vp, vp]
     L.go_rope_tables_f32.argtypes = [vp, vp, u64, u64, f]
-    L.go_layer_forward_f32.argtypes = [cfgp, vp, vp, vp, vp, vp, vp, u64]
-    L.go_classify_f32.argtypes = [cfgp, vp, vp, vp, vp, u64]
+    for sfx in ("f32", "f16"):
+        getattr(L, f"go_layer_forward_{sfx}").argtypes = [cfgp, vp, vp, vp, vp, vp, vp, u64]
+        getattr(L, f"go_classify_{sfx}").argtypes = [cfgp, vp, vp, vp, vp, u64]
     for name in ("go_ctx_layer_offset", "go_ctx_token_offset", "go_ctx_key_head_offset",
                  "go_ctx_value_head_offset", "go_ctx_max_size_bytes", "go_dynctx_prepare",
                  "go_ctxman_free", "go_ctxman_allocated"):
@@ -176,6 +177,23 @@ def num_threads() -> int:
 # --------------------------------------------------------------------------------------------
 # common ops (arch/amd64/common/ops.hh)
 # --------------------------------------------------------------------------------------------
+def convert(src: np.ndarray, dst_dtype) -> np.ndarray:
+    """convert_and_copy (arch/amd64/llama2/ops.hh:354-368): element-wise static_cast between float32 and float16
+    storage; the same type is a plain copy."""
+    src = np.ascontiguousarray(src)
+    dst_dtype = np.dtype(dst_dtype)
+    if src.dtype == dst_dtype:
+        return src.copy()
+    out = np.empty(src.shape, dtype=dst_dtype)
+    if src.dtype == np.float16 and dst_dtype == np.float32:
+        lib().go_convert_f16_to_f32(out.ctypes.data, src.ctypes.data, src.size)
+    elif src.dtype == np.float32 and dst_dtype == np.float16:
+        lib().go_convert_f32_to_f16(out.ctypes.data, src.ctypes.data, src.size)
+    else:
+        raise TypeError(f"oracle converts between float32 and float16, got {src.dtype} -> {dst_dtype}")
+    return out
+
+
 def accum(a: np.ndarray, b: np.ndarray) -> None:
     """In place ``a += b`` over a (batch, size) array."""
     batch, size = a.shape
@@ -301,34 +319,41 @@ class _Scratch(C.Structure):
 def layer_forward(cfg: Config, weights: dict, freq_real: np.ndarray, freq_imag: np.ndarray,
                   x: np.ndarray, layers: Sequence[Optional[np.ndarray]], token_positions,
                   scratch: Optional[dict] = None) -> dict:
-    """One full layer (pre-attention + attention + post-attention), fp32.  ``x`` (batch, dim) is
-    updated in place; returns the scratch arrays (q, kv, xb, ...) for inspection."""
-    assert x.dtype == np.float32
+    """One full layer (pre-attention + attention + post-attention) in the storage type of ``x``: float32, or
+    float16 with every op's result rounded to binary16 where the reference's DType = _Float16 build rounds it
+    (weights, tables and cache rows must have the same type).  ``x`` (batch, dim) is updated in place;
+    returns the scratch arrays (q, kv, xb, ...) for inspection."""
+    dt = x.dtype
+    assert dt in (np.float32, np.float16)
+    names = ("rms_att_weight", "wq", "wkv", "wo", "rms_ffn_weight", "w1", "w2", "w3")
+    assert all(weights[n].dtype == dt for n in names) and freq_real.dtype == dt and freq_imag.dtype == dt
+    assert all(l is None or l.dtype == dt for l in layers)
     batch = x.shape[0]
     s = scratch or {}
-    s.setdefault("xb", np.zeros((batch, cfg.dim), np.float32))
-    s.setdefault("xb2", np.zeros((batch, cfg.dim), np.float32))
-    s.setdefault("q", np.zeros((batch, cfg.dim), np.float32))
-    s.setdefault("kv", np.zeros((batch, 2 * cfg.kv_dim), np.float32))
-    s.setdefault("hb", np.zeros((batch, cfg.hidden_dim), np.float32))
-    s.setdefault("hb2", np.zeros((batch, cfg.hidden_dim), np.float32))
-    s.setdefault("att", np.zeros((batch, cfg.n_heads, cfg.seq_len), np.float32))
+    s.setdefault("xb", np.zeros((batch, cfg.dim), dt))
+    s.setdefault("xb2", np.zeros((batch, cfg.dim), dt))
+    s.setdefault("q", np.zeros((batch, cfg.dim), dt))
+    s.setdefault("kv", np.zeros((batch, 2 * cfg.kv_dim), dt))
+    s.setdefault("hb", np.zeros((batch, cfg.hidden_dim), dt))
+    s.setdefault("hb2", np.zeros((batch, cfg.hidden_dim), dt))
+    s.setdefault("att", np.zeros((batch, cfg.n_heads, cfg.seq_len), dt))
     s["x"] = x
-    lw = _LayerW(*[_p(weights[n]) for n in ("rms_att_weight", "wq", "wkv", "wo", "rms_ffn_weight",
-                                            "w1", "w2", "w3")])
+    lw = _LayerW(*[_p(weights[n]) for n in names])
     sc = _Scratch(*[_p(s[n]) for n in ("x", "xb", "xb2", "q", "kv", "hb", "hb2", "att")])
     c = cfg.c()
     pos = _pos(token_positions)
-    lib().go_layer_forward_f32(C.byref(c), C.byref(lw), _p(freq_real), _p(freq_imag), C.byref(sc),
+    _fn("go_layer_forward", x)(C.byref(c), C.byref(lw), _p(freq_real), _p(freq_imag), C.byref(sc),
                                _ptr_table(layers), _p(pos), batch)
     return s
 
 
 def classify(cfg: Config, rms_final: np.ndarray, wcls: np.ndarray, x: np.ndarray) -> np.ndarray:
+    """Final rmsnorm (in place on ``x``) and the logits, in the storage type of ``x``."""
+    assert rms_final.dtype == x.dtype and wcls.dtype == x.dtype
     batch = x.shape[0]
-    logits = np.empty((batch, cfg.vocab_size), np.float32)
+    logits = np.empty((batch, cfg.vocab_size), x.dtype)
     c = cfg.c()
-    lib().go_classify_f32(C.byref(c), _p(rms_final), _p(wcls), _p(x), _p(logits), batch)
+    _fn("go_classify", x)(C.byref(c), _p(rms_final), _p(wcls), _p(x), _p(logits), batch)
     return logits
 
 

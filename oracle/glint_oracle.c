@@ -30,6 +30,9 @@
  *   go_attention_2_gemm                   numpy einsum float64; uniform weights -> mean of V
  *   go_attention_ops                      composition vs float64 end-to-end attention; pos 0 -> V row 0
  *   go_layer_forward_f32, go_classify_f32 float64 numpy transformer block (independent einsum code)
+ *   go_layer_forward_f16, go_classify_f16 bit-equal to the chain of the binary16 ops above in the reference's
+ *                                         order; within half precision of the float64 block
+ *   go_convert_f16_to_f32 / _f32_to_f16   the two conversions above over whole arrays
  *   go_rope_tables_f32                    closed form vs numpy float64
  *   go_ctx_* addressing                   brute force enumeration on small shapes; disjointness
  *   go_dynctx_prepare                     brute-force page model (set of committed blocks)
@@ -186,60 +189,6 @@ void go_rope_tables_f32( float* real, float* imag, uint64_t seq_len, uint64_t he
       imag[p * half + k] = sinf( angle );
     }
   }
-}
-
-/* models/llama2/model.hh:326-427 -- one full layer in the order the reference issues the ops:
- * rmsnorm, wq, wkv, kv append | rope, scores, softmax, weighted sum | wo, accum, rmsnorm, w1, w3,
- * silu, w2, accum. */
-void go_layer_forward_f32( const go_config* c,
-                           const go_layer_weights_f32* w,
-                           const float* freq_cis_real,
-                           const float* freq_cis_imag,
-                           go_scratch_f32* s,
-                           float* const* layer_ctx,
-                           const uint32_t* token_positions,
-                           uint64_t batch )
-{
-  float** token_ctx = (float**)malloc( sizeof( float* ) * ( batch ? batch : 1 ) );
-  for ( uint64_t i = 0; i < batch; i++ ) {
-    token_ctx[i] = layer_ctx[i] ? layer_ctx[i] + (uint64_t)token_positions[i] * 2 * c->kv_dim : NULL;
-  }
-
-  /* pre-attention: model.hh:326-351 */
-  go_rmsnorm_f32( s->xb, s->x, w->rms_att_weight, c->dim, batch );
-  go_matmul_f32( s->q, s->xb, w->wq, c->dim, c->dim, batch );
-  go_matmul_f32( s->kv, s->xb, w->wkv, c->dim, 2 * c->kv_dim, batch );
-  go_copy_kv_cache_f32( c, token_ctx, s->kv, batch );
-
-  /* attention: model.hh:354-387 */
-  go_apply_rope_f32( c, batch, token_positions, freq_cis_real, freq_cis_imag, s->q, token_ctx );
-  go_attention_0_gemm_f32( c, s->q, (const float* const*)layer_ctx, s->att, batch, token_positions );
-  go_attention_softmax_f32( c, s->att, token_positions, batch );
-  go_attention_2_gemm_f32( c, s->att, (const float* const*)layer_ctx, s->xb, batch, token_positions );
-
-  /* post-attention: model.hh:390-427 */
-  go_matmul_f32( s->xb2, s->xb, w->wo, c->dim, c->dim, batch );
-  go_accum_f32( s->x, s->xb2, c->dim, batch );
-  go_rmsnorm_f32( s->xb, s->x, w->rms_ffn_weight, c->dim, batch );
-  go_matmul_f32( s->hb, s->xb, w->w1, c->dim, c->hidden_dim, batch );
-  go_matmul_f32( s->hb2, s->xb, w->w3, c->dim, c->hidden_dim, batch );
-  go_silu_f32( s->hb, s->hb2, c->hidden_dim, batch );
-  go_matmul_f32( s->xb, s->hb, w->w2, c->hidden_dim, c->dim, batch );
-  go_accum_f32( s->x, s->xb, c->dim, batch );
-
-  free( token_ctx );
-}
-
-/* models/llama2/model.hh:430-442 */
-void go_classify_f32( const go_config* c,
-                      const float* rms_final_weight,
-                      const float* wcls,
-                      float* x,
-                      float* logits,
-                      uint64_t batch )
-{
-  go_rmsnorm_f32( x, x, rms_final_weight, c->dim, batch );
-  go_matmul_f32( logits, x, wcls, c->dim, c->vocab_size, batch );
 }
 
 /* ---------------------------------------------------------------------------------------------

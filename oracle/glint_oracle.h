@@ -109,48 +109,38 @@ GO_DECLARE_ATTN_OPS( f16, go_half )
 void go_rope_tables_f32( float* real, float* imag, uint64_t seq_len, uint64_t head_size, float theta );
 
 /* ---- one layer / one stage of the model driver: models/llama2/model.hh:326-442,534-571 ---- */
-typedef struct go_layer_weights_f32
-{
-  const float* rms_att_weight; /* (dim) */
-  const float* wq;             /* (dim, dim) row-major, row = output feature */
-  const float* wkv;            /* (2*kv_dim, dim): wk rows then wv rows */
-  const float* wo;             /* (dim, dim) */
-  const float* rms_ffn_weight; /* (dim) */
-  const float* w1;             /* (hidden_dim, dim) */
-  const float* w2;             /* (dim, hidden_dim) */
-  const float* w3;             /* (hidden_dim, dim) */
-} go_layer_weights_f32;
+#define GO_DECLARE_LAYER( T, SFX )                                                                                     \
+  typedef struct go_layer_weights_##SFX                                                                                \
+  {                                                                                                                    \
+    const T* rms_att_weight; /* (dim) */                                                                               \
+    const T* wq;             /* (dim, dim) row-major, row = output feature */                                          \
+    const T* wkv;            /* (2*kv_dim, dim): wk rows then wv rows */                                               \
+    const T* wo;             /* (dim, dim) */                                                                          \
+    const T* rms_ffn_weight; /* (dim) */                                                                               \
+    const T* w1;             /* (hidden_dim, dim) */                                                                   \
+    const T* w2;             /* (dim, hidden_dim) */                                                                   \
+    const T* w3;             /* (hidden_dim, dim) */                                                                   \
+  } go_layer_weights_##SFX;                                                                                            \
+  typedef struct go_scratch_##SFX                                                                                      \
+  {                                                                                                                    \
+    T* x;   /* (B, dim) residual stream, in/out */                                                                     \
+    T* xb;  /* (B, dim) */                                                                                             \
+    T* xb2; /* (B, dim) */                                                                                             \
+    T* q;   /* (B, dim) */                                                                                             \
+    T* kv;  /* (B, 2*kv_dim) */                                                                                        \
+    T* hb;  /* (B, hidden) */                                                                                          \
+    T* hb2; /* (B, hidden) */                                                                                          \
+    T* att; /* (B, n_heads, seq_len) */                                                                                \
+  } go_scratch_##SFX;                                                                                                  \
+  /* pre_attention_ops(update_kv_cache=true) + attention_ops() + post_attention_ops() for one layer.                   \
+   * layer_ctx[i] = base of this layer's rows for context i (NULL = empty). */                                         \
+  void go_layer_forward_##SFX( const go_config* c, const go_layer_weights_##SFX* w, const T* freq_cis_real, const T* freq_cis_imag,            \
+                               go_scratch_##SFX* s, T* const* layer_ctx, const uint32_t* token_positions, uint64_t batch );                  \
+  /* classify_ops(): final rmsnorm (in place on x) + logits = x . wcls^T ; model.hh:430-442 */                        \
+  void go_classify_##SFX( const go_config* c, const T* rms_final_weight, const T* wcls, T* x, T* logits, uint64_t batch );
 
-typedef struct go_scratch_f32
-{
-  float* x;   /* (B, dim) residual stream, in/out */
-  float* xb;  /* (B, dim) */
-  float* xb2; /* (B, dim) */
-  float* q;   /* (B, dim) */
-  float* kv;  /* (B, 2*kv_dim) */
-  float* hb;  /* (B, hidden) */
-  float* hb2; /* (B, hidden) */
-  float* att; /* (B, n_heads, seq_len) */
-} go_scratch_f32;
-
-/* pre_attention_ops(update_kv_cache=true) + attention_ops() + post_attention_ops() for one layer.
- * layer_ctx[i] = base of this layer's rows for context i (NULL = empty). */
-void go_layer_forward_f32( const go_config* c,
-                           const go_layer_weights_f32* w,
-                           const float* freq_cis_real,
-                           const float* freq_cis_imag,
-                           go_scratch_f32* s,
-                           float* const* layer_ctx,
-                           const uint32_t* token_positions,
-                           uint64_t batch );
-
-/* classify_ops(): final rmsnorm (in place on x) + logits = x . wcls^T ; model.hh:430-442 */
-void go_classify_f32( const go_config* c,
-                      const float* rms_final_weight,
-                      const float* wcls,
-                      float* x,
-                      float* logits,
-                      uint64_t batch );
+GO_DECLARE_LAYER( float, f32 )
+GO_DECLARE_LAYER( go_half, f16 ) /* every intermediate rounded to binary16 where the reference's DType = _Float16 build rounds it */
 
 /* ---- bookkeeping models (pure integer semantics) ------------------------------------------ */
 

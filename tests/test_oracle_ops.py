@@ -465,6 +465,68 @@ def test_layer_forward(cfg):
         np.testing.assert_allclose(layers[i], want_layers[i], rtol=2e-4, atol=2e-5)
 
 
+@pytest.mark.parametrize("cfg", [TINY, MHA])
+def test_layer_forward_half_storage(cfg):
+    """The binary16 layer: (a) it is the chain of the individually pinned binary16 ops in the reference's order
+    (models/llama2/model.hh:326-427), bit for bit -- a skipped op, a swapped buffer or a missing rounding between
+    two ops fails this; (b) it stays within half-precision distance of the independent float64 block."""
+    batch = 3
+    pos = [0, 4, cfg.seq_len - 1]
+    w = make_layer_weights(cfg, dtype=np.float16)
+    re32, im32 = O.rope_tables(cfg.seq_len, cfg.head_size)
+    re, im = re32.astype(np.float16), im32.astype(np.float16)
+    layers = [rng.standard_normal((cfg.seq_len, 2 * cfg.kv_dim)).astype(np.float16) for _ in range(batch)]
+    x = rng.standard_normal((batch, cfg.dim)).astype(np.float16)
+
+    # (a) op by op, every result stored as binary16
+    x_ops = x.copy()
+    l_ops = [l.copy() for l in layers]
+    xb = O.rmsnorm(x_ops, w["rms_att_weight"])
+    q = O.matmul(xb, w["wq"])
+    kv = O.matmul(xb, w["wkv"])
+    assert xb.dtype == q.dtype == kv.dtype == np.float16
+    O.copy_kv_cache(cfg, [l_ops[i][pos[i]] for i in range(batch)], kv)
+    att_out = O.attention_ops(cfg, pos, re, im, q, l_ops)
+    assert att_out.dtype == np.float16
+    O.accum(x_ops, O.matmul(att_out, w["wo"]))
+    xb = O.rmsnorm(x_ops, w["rms_ffn_weight"])
+    hb, hb2 = O.matmul(xb, w["w1"]), O.matmul(xb, w["w3"])
+    O.silu(hb, hb2)
+    O.accum(x_ops, O.matmul(hb, w["w2"]))
+
+    x_layer = x.copy()
+    l_layer = [l.copy() for l in layers]
+    O.layer_forward(cfg, w, re, im, x_layer, l_layer, pos)
+    assert x_layer.dtype == np.float16
+    assert np.array_equal(x_layer.view(np.uint16), x_ops.view(np.uint16))
+    for i in range(batch):
+        assert np.array_equal(l_layer[i].view(np.uint16), l_ops[i].view(np.uint16))
+
+    # (b) against float64 on the same (binary16-representable) inputs
+    w32 = {k: v.astype(np.float32) for k, v in w.items()}
+    want_x, want_layers = layer_ref64(cfg, w32, x.astype(np.float32), [l.astype(np.float32) for l in layers], pos)
+    err = np.abs(x_layer.astype(np.float64) - want_x)
+    assert err.max() <= 3e-2 and err.mean() / np.abs(want_x).mean() <= 2e-3
+    for i in range(batch):
+        np.testing.assert_allclose(l_layer[i].astype(np.float64), want_layers[i], rtol=2e-3, atol=2e-3)
+
+
+def test_classify_half_storage():
+    cfg = TINY
+    r = np.random.default_rng(3)
+    x = r.standard_normal((2, cfg.dim)).astype(np.float16)
+    g = (1 + 0.1 * r.standard_normal(cfg.dim)).astype(np.float16)
+    wcls = (0.2 * r.standard_normal((cfg.vocab_size, cfg.dim))).astype(np.float16)
+    x_ops = O.rmsnorm(x.copy(), g)
+    want = O.matmul(x_ops, wcls)
+    logits = O.classify(cfg, g, wcls, x)
+    assert logits.dtype == np.float16
+    assert np.array_equal(logits.view(np.uint16), want.view(np.uint16))
+    assert np.array_equal(x.view(np.uint16), x_ops.view(np.uint16))          # normalised in place
+    x64 = x_ops.astype(np.float64)
+    np.testing.assert_allclose(logits.astype(np.float64), x64 @ wcls.astype(np.float64).T, rtol=2e-3, atol=2e-3)
+
+
 def test_classify():
     cfg = TINY
     r = np.random.default_rng(3)
