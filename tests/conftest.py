@@ -27,3 +27,24 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+def pytest_sessionfinish(session, exitstatus):
+    """Keeps the measured fp16 distances of the stage tests (helpers.DRIFT) next to the other GPU run outputs."""
+    try:
+        import helpers
+    except Exception:
+        return
+    if not helpers.DRIFT:
+        return
+    out = os.path.join(ROOT, "gpurun_out")
+    os.makedirs(out, exist_ok=True)
+    with open(os.path.join(out, "fp16_drift.txt"), "w") as f:
+        f.write("mean-relative distances: HIP vs fp16 oracle | HIP vs fp32 oracle | fp16 oracle vs fp32 oracle\n")
+        worst = {}
+        for what, r16, r32, rs in helpers.DRIFT:
+            key = what.split(" step ")[0]
+            w = worst.setdefault(key, [0.0, 0.0, 0.0, 0])
+            w[0], w[1], w[2], w[3] = max(w[0], r16), max(w[1], r32), max(w[2], rs), w[3] + 1
+        for key, (r16, r32, rs, n) in worst.items():
+            f.write(f"{key}: max over {n} outputs  {r16:.3e} | {r32:.3e} | {rs:.3e}\n")

@@ -6,7 +6,7 @@ import torch
 
 import oracle as O
 from glinthawk_amd import Shape, ops, stage as S
-from helpers import Arena, assert_close, oracle_cfg
+from helpers import Arena, assert_close, assert_half_parity, oracle_cfg
 from test_gpu_stage import SHAPES, OracleModel, d2h, load_weights, make_weights
 
 pytestmark = pytest.mark.gpu
@@ -130,6 +130,7 @@ def test_stage_with_and_without_fused_projections(name, dtype):
     a = S.Stage(name, dtype, 0, cfg.n_layers, batch, batch, with_cls=True, fused_projections=True)
     b = S.Stage(name, dtype, 0, cfg.n_layers, batch, batch, with_cls=True, fused_projections=False)
     ref = OracleModel(cfg, layers, base)
+    ref16 = OracleModel(cfg, layers, base, np.float16) if dtype == "f16" else None
     for st in (a, b):
         load_weights(st, cfg, layers, base, wcls)
         st.new_state(batch)
@@ -145,7 +146,12 @@ def test_stage_with_and_without_fused_projections(name, dtype):
         # projection against the split of its parts (an fp16 rounding can flip and travel through the layers)
         tol = 8e-3 if dtype == "f16" else 2e-5
         np.testing.assert_allclose(la, lb, rtol=tol, atol=tol)
-        assert_close(la, want, mean_rel=2e-3 if dtype == "f16" else 1e-3, what=f"{name} fused-projection logits step {step}")
+        if dtype == "f16":
+            want16 = ref16.step(tokens, list(range(batch)), [step] * batch)
+            assert_half_parity(la, want16, want, what=f"{name} fused-projection logits step {step}")
+            assert_half_parity(lb, want16, want, what=f"{name} separate-projection logits step {step}")
+        else:
+            assert_close(la, want, mean_rel=1e-3, what=f"{name} fused-projection logits step {step}")
         tokens = [a.row(i)["token"] for i in range(batch)]
         for i in range(batch):                         # keep both stages on the same token stream
             b.set_prompt(i, i, tokens[i], step + 1)

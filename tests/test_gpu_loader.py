@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 
 from glinthawk_amd import modeldir, stage as S
-from helpers import assert_close
+from helpers import assert_close, assert_half_parity
 from test_gpu_stage import SHAPES, WCLS, OracleModel, d2h, load_weights, make_weights
 
 pytestmark = pytest.mark.gpu
@@ -42,8 +42,12 @@ def test_loaded_stage_equals_tensor_by_tensor(tmp_path, name, dtype):
         assert np.array_equal(x, y)
     ref = OracleModel(cfg, layers, base)
     want = ref.step(tokens.tolist(), [40 + i for i in range(batch)], [0] * batch)
-    assert_close(la[0].astype(np.float32), want, mean_rel=3e-3 if name == "test-tiny" else (2e-3 if dtype == "f16" else 1e-3),
-                 what=f"{name} logits from loaded weights")
+    if dtype == "f16":
+        want16 = OracleModel(cfg, layers, base, np.float16).step(tokens.tolist(), [40 + i for i in range(batch)], [0] * batch)
+        assert_half_parity(la[0].astype(np.float32), want16, want, what=f"{name} logits from loaded weights",
+                           mean_rel32=3e-3 if name == "test-tiny" else 2e-3)
+    else:
+        assert_close(la[0].astype(np.float32), want, mean_rel=1e-3, what=f"{name} logits from loaded weights")
     a.close()
     b.close()
 

@@ -8,7 +8,7 @@ import torch
 import oracle as O
 from glinthawk_amd import Shape, ops
 from glinthawk_amd._lib import GH_ATTN_AUTO, GH_ATTN_GENERIC, GH_ATTN_MFMA
-from helpers import Arena, assert_close, errors, oracle_cfg
+from helpers import Arena, assert_close, assert_half_parity, errors, oracle_cfg
 
 pytestmark = pytest.mark.gpu
 
@@ -116,6 +116,7 @@ def test_stage_prefill_equals_token_by_token(name, dtype, n_prompt):
     a = S.Stage(name, dtype, 0, cfg.n_layers, batch, batch, with_cls=True)      # batched prefill
     b = S.Stage(name, dtype, 0, cfg.n_layers, batch, batch, with_cls=True)      # the reference's way: one token per forward
     ref = OracleModel(cfg, layers, base)
+    ref16 = OracleModel(cfg, layers, base, np.float16) if dtype == "f16" else None
     for st in (a, b):
         load_weights(st, cfg, layers, base, wcls)
 
@@ -125,6 +126,7 @@ def test_stage_prefill_equals_token_by_token(name, dtype, n_prompt):
         b.set_prompt(i, 10 + i, int(prompts[i, 0]), 0, 0.0, n_prompt, 0)
     for pos in range(n_prompt):
         want = ref.step(prompts[:, pos].tolist(), [10 + i for i in range(batch)], [pos] * batch)
+        want16 = ref16.step(prompts[:, pos].tolist(), [10 + i for i in range(batch)], [pos] * batch) if ref16 else None
         assert b.forward()
         if pos + 1 < n_prompt:
             for i in range(batch):
@@ -140,7 +142,11 @@ def test_stage_prefill_equals_token_by_token(name, dtype, n_prompt):
     pre_logits = d2h(a.scratch_ptr("logits"), (batch, cfg.vocab_size), np_dt).astype(np.float32)
     tol = 6e-3 if dtype == "f16" else 5e-5
     np.testing.assert_allclose(pre_logits, seq_logits, rtol=tol, atol=tol)
-    assert_close(pre_logits, want, mean_rel=2e-3 if dtype == "f16" else 1e-3, what=f"{name} prefill logits vs oracle")
+    if dtype == "f16":
+        assert_half_parity(pre_logits, want16, want, what=f"{name} prefill logits, {n_prompt} tokens")
+        assert_half_parity(seq_logits, want16, want, what=f"{name} token-by-token logits, {n_prompt} tokens")
+    else:
+        assert_close(pre_logits, want, mean_rel=1e-3, what=f"{name} prefill logits vs oracle")
     for i in range(batch):
         if nxt[i] != seq_next[i]:
             assert abs(seq_logits[i, nxt[i]] - seq_logits[i, seq_next[i]]) < 1e-2      # near tie only
