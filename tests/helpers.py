@@ -28,23 +28,29 @@ def assert_close(got, want, max_abs=MAX_ABS_TOL, mean_rel=MEAN_REL_TOL, what="")
 # Measured distances of the fp16 stage outputs: (what, HIP vs fp16 oracle, HIP vs fp32 oracle, fp16 oracle vs fp32 oracle),
 # mean-relative; written to gpurun_out/fp16_drift.txt at the end of a test session (conftest.py).
 DRIFT = []
-HALF_TOL = 5e-4       # HIP fp16 stage output against the oracle's fp16-storage path, mean-relative
 
 
-def assert_half_parity(got, want16, want32, what="", tol16=HALF_TOL, max_abs=MAX_ABS_TOL, mean_rel32=2e-3):
-    """An fp16-storage stage output against both CPU paths.  Every op of the reference's DType = _Float16 build
-    rounds its output to fp16, which by itself moves multi-layer outputs 1-2e-3 (mean-relative) away from
-    the fp32 build.  So the kernels are held to the fp16 oracle at `tol16`; the distance to the fp32 oracle
-    is bounded by the north-star max-abs and by `mean_rel32`, and must not exceed the fp16 oracle's own
-    distance from fp32 by more than `tol16`: what separates the GPU from fp32 is the storage type."""
+def assert_half_parity(got, want16, want32, what="", tol16=None, max_abs=MAX_ABS_TOL, mean_rel32=2e-3):
+    """An fp16-storage stage output against the CPU path in both storage types.
+
+    Every op of the reference's DType = _Float16 build rounds its output to fp16, which by itself moves
+    multi-layer outputs around 1e-3 (mean-relative) away from the fp32 build.  The test therefore measures
+    that distance (fp16 oracle against fp32 oracle, on the same inputs) and requires the GPU's distance from
+    the fp32 oracle to stay within 15 % + 1e-4 of it: a kernel error worth 1e-3 on top of the storage rounding
+    fails.  `mean_rel32` and the north-star max-abs bound the distance absolutely.  `tol16` (where given) holds
+    the output to the fp16 oracle directly; that is only tight for paths that round where the reference rounds
+    (the fused attention keeps scores and weights in fp32, the reference's fp16 build rounds both to fp16,
+    which moves its attention outputs as much as all its other roundings together)."""
     want16 = np.asarray(want16, dtype=np.float32)
     a16, r16 = errors(got, want16)
     a32, r32 = errors(got, want32)
     _, r_storage = errors(want16, want32)
     DRIFT.append((what, r16, r32, r_storage))
-    assert a16 <= max_abs and r16 <= tol16, f"{what}: vs fp16 oracle max_abs {a16:.3e}, mean_rel {r16:.3e} (tol {tol16})"
-    assert a32 <= max_abs and r32 <= mean_rel32, f"{what}: vs fp32 oracle max_abs {a32:.3e}, mean_rel {r32:.3e}"
-    assert r32 <= r_storage + tol16, f"{what}: {r32:.3e} from fp32, of which fp16 storage explains {r_storage:.3e}"
+    assert a32 <= max_abs and r32 <= mean_rel32, f"{what}: vs fp32 oracle max_abs {a32:.3e}, mean_rel {r32:.3e} (tol {mean_rel32})"
+    assert r32 <= 1.15 * r_storage + 1e-4, f"{what}: {r32:.3e} from the fp32 oracle, fp16 storage alone gives {r_storage:.3e}"
+    assert a16 <= max_abs, f"{what}: vs fp16 oracle max_abs {a16:.3e}"
+    if tol16 is not None:
+        assert r16 <= tol16, f"{what}: vs fp16 oracle mean_rel {r16:.3e} (tol {tol16})"
 
 
 def oracle_cfg(shape) -> O.Config:

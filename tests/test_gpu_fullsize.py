@@ -148,7 +148,8 @@ def test_one_full_layer_of_the_stage_against_the_oracle(BATCH, limit):
     O.layer_forward(cfg, w32, re16.astype(np.float32), im16.astype(np.float32), x32, ctx_layers, [pos] * BATCH)
     O.layer_forward(cfg, w16, re16, im16, x16, half_layers, [pos] * BATCH)
     # residual stream after one layer against the CPU path in both storage types
-    assert_half_parity(got, x16, x32, what=f"70B layer, B={BATCH} of {limit}, position 4095")
+    # a single layer is shallow enough for the comparison with the fp16 oracle to be tight as well (measured 1.9e-4)
+    assert_half_parity(got, x16, x32, what=f"70B layer, B={BATCH} of {limit}, position 4095", tol16=3e-4)
     # the appended rows (K rotated, V raw) landed where the oracle put them
     row = np.empty(2 * SHAPE.kv_dim, np.float16)
     for i in (0, BATCH // 2, BATCH - 1):

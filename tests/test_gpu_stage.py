@@ -129,8 +129,10 @@ def test_full_model_decode_matches_oracle(name, dtype, fused):
         else:
             # fp16 storage: held to the CPU path with the same storage type; the distance to fp32 is the storage's
             want16 = ref16.step(tokens, [100 + i for i in range(batch)], pos)
+            # the smallest shape runs kernels that add in the oracle's order: there the unfused path, which rounds
+            # where the reference rounds, reproduces the fp16 oracle almost bit for bit (measured 2e-5)
             assert_half_parity(got, want16, want, what=f"{name} {'fused' if fused else 'unfused'} logits step {step}",
-                               mean_rel32=3e-3 if name == "test-tiny" else 2e-3)
+                               tol16=1e-4 if (name == "test-tiny" and not fused) else None)
         rows = [st.row(i) for i in range(batch)]
         for i in range(batch):
             assert rows[i]["token_pos"] == step + 1
