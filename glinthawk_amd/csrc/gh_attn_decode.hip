@@ -29,6 +29,14 @@ namespace {
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr int HS = 128; // head size of the fast kernels
 
+// Split-K partials of gh_attn_decode_static: one array per GPU the library runs on, held until the
+// process ends.  Host code never uses the array's name as an address: the device address is looked
+// up once per device at initialisation (attn_static_scratch_init) and kept in g_static_scratch.
+constexpr uint64_t STATIC_SCRATCH_BYTES = 16ull << 20;
+constexpr int MAX_DEVICES = 16;
+static __device__ __align__( 256 ) float scratch[STATIC_SCRATCH_BYTES / sizeof( float )];
+float* g_static_scratch[MAX_DEVICES] = {};
+
 uint32_t g_chunk_override = 0;
 int g_auto_variant = GH_ATTN_AUTO; // what GH_ATTN_AUTO resolves to when the shape allows it (gh_attn_set_auto_variant)
 
@@ -738,6 +746,19 @@ void launch_mfma( dim3 grid, hipStream_t st, const void* q, const void* const* r
 }
 
 } // namespace
+
+// Called by the library's initialisation with `device` current: the device address of this GPU's
+// `scratch` array.  Every GPU holds its own copy of the array at its own address.
+int attn_static_scratch_init( int device )
+{
+  GH_REQUIRE( device >= 0 && device < MAX_DEVICES, "device %d beyond the %d devices the static attention scratch is kept for", device, MAX_DEVICES );
+  float* ptr = nullptr;
+  GH_HIP( hipGetSymbolAddress( reinterpret_cast<void**>( &ptr ), HIP_SYMBOL( scratch ) ) );
+  GH_REQUIRE( ptr != nullptr && ( reinterpret_cast<uintptr_t>( ptr ) & 255u ) == 0, "static attention scratch has no aligned device address" );
+  g_static_scratch[device] = ptr;
+  return GH_OK;
+}
+
 } // namespace gh
 
 using namespace gh;
@@ -792,16 +813,12 @@ int gh_attn_decode_plan( uint64_t batch, uint32_t max_pos, const gh_shape* shape
   return GH_OK;
 }
 
-int gh_attn_decode( const void* q, const void* const* layer_rows_dev, const uint32_t* pos_dev, void* xb, uint64_t batch,
-                    uint32_t max_pos, const gh_shape* shape, gh_dtype dt, void* workspace, uint64_t workspace_bytes,
-                    int variant, gh_stream stream )
+// Shared by gh_attn_decode (partials in the caller's workspace, kernel timer on request) and
+// gh_attn_decode_static (partials in this GPU's `scratch` array; nothing here allocates when `timed` is false).
+static int attn_decode_run( const char* who, const void* q, const void* const* layer_rows_dev, const uint32_t* pos_dev, void* xb, uint64_t batch,
+                            uint32_t max_pos, const gh_shape* shape, gh_dtype dt, void* workspace, uint64_t workspace_bytes, int variant,
+                            gh_stream stream, bool timed )
 {
-  if ( int rc = ensure_init() ) {
-    return rc;
-  }
-  if ( batch == 0 ) {
-    return GH_OK;
-  }
   GH_REQUIRE( shape != nullptr, "gh_attn_decode: NULL shape" );
   GH_REQUIRE( q && layer_rows_dev && pos_dev && xb, "gh_attn_decode: NULL pointer" );
   GH_REQUIRE( dt == GH_F16 || dt == GH_F32, "gh_attn_decode: unsupported dtype %d", (int)dt );
@@ -827,10 +844,10 @@ int gh_attn_decode( const void* q, const void* const* layer_rows_dev, const uint
   Partials part { nullptr, nullptr };
   if ( plan.max_splits > 1 ) {
     const uint64_t need = partial_floats( batch, shape, plan.max_splits ) * sizeof( float );
-    GH_REQUIRE( workspace != nullptr, "gh_attn_decode: workspace required (%llu bytes)", (unsigned long long)need );
+    GH_REQUIRE( workspace != nullptr, "%s: workspace required (%llu bytes)", who, (unsigned long long)need );
     if ( workspace_bytes < need ) {
-      return fail( GH_ERR_WORKSPACE, "gh_attn_decode: workspace of %llu bytes, %llu needed", (unsigned long long)workspace_bytes,
-                   (unsigned long long)need );
+      return fail( GH_ERR_WORKSPACE, "%s: %llu bytes of split partials needed, %llu available", who, (unsigned long long)need,
+                   (unsigned long long)workspace_bytes );
     }
     GH_REQUIRE( ( reinterpret_cast<uintptr_t>( workspace ) & 15u ) == 0, "gh_attn_decode: workspace must be 16-byte aligned" );
     part.out = static_cast<float*>( workspace );
@@ -840,8 +857,10 @@ int gh_attn_decode( const void* q, const void* const* layer_rows_dev, const uint
   hipStream_t st = as_stream( stream );
   const float scale = LOG2E / sqrtf( (float)shape->head_size );
   int timer = -1;
-  if ( int rc = timer_mark( st, &timer, 0 ) ) {
-    return rc;
+  if ( timed ) {
+    if ( int rc = timer_mark( st, &timer, 0 ) ) {
+      return rc;
+    }
   }
 
   if ( plan.variant == GH_ATTN_GENERIC ) {
@@ -876,8 +895,10 @@ int gh_attn_decode( const void* q, const void* const* layer_rows_dev, const uint
     }
   }
   GH_LAUNCH_CHECK();
-  if ( int rc = timer_mark( st, &timer, 1 ) ) {
-    return rc;
+  if ( timed ) {
+    if ( int rc = timer_mark( st, &timer, 1 ) ) {
+      return rc;
+    }
   }
 
   if ( plan.max_splits > 1 ) {
@@ -892,7 +913,37 @@ int gh_attn_decode( const void* q, const void* const* layer_rows_dev, const uint
     }
     GH_LAUNCH_CHECK();
   }
-  return timer_mark( st, &timer, 2 );
+  return timed ? timer_mark( st, &timer, 2 ) : GH_OK;
+}
+
+int gh_attn_decode( const void* q, const void* const* layer_rows_dev, const uint32_t* pos_dev, void* xb, uint64_t batch,
+                    uint32_t max_pos, const gh_shape* shape, gh_dtype dt, void* workspace, uint64_t workspace_bytes,
+                    int variant, gh_stream stream )
+{
+  if ( int rc = ensure_init() ) {
+    return rc;
+  }
+  if ( batch == 0 ) {
+    return GH_OK;
+  }
+  return attn_decode_run( "gh_attn_decode", q, layer_rows_dev, pos_dev, xb, batch, max_pos, shape, dt, workspace, workspace_bytes, variant, stream, true );
+}
+
+uint64_t gh_attn_decode_static_limit( void ) { return STATIC_SCRATCH_BYTES; }
+
+int gh_attn_decode_static( const void* q, const void* const* layer_rows_dev, const uint32_t* pos_dev, void* xb, uint64_t batch, uint32_t max_pos,
+                           const gh_shape* shape, gh_dtype dt, int variant, gh_stream stream )
+{
+  // no ensure_init() here: initialisation allocates (staging ring), so it has to have happened in gh_init()
+  const int device = initialised_device();
+  GH_REQUIRE( device >= 0, "gh_attn_decode_static: the library is not initialised; call gh_init() first (this entry point allocates nothing)" );
+  GH_REQUIRE( device < MAX_DEVICES && g_static_scratch[device] != nullptr, "gh_attn_decode_static: no scratch array on device %d", device );
+  if ( batch == 0 ) {
+    return GH_OK;
+  }
+  // a plan that needs more partials than the array holds is refused by the size check of the shared path (GH_ERR_WORKSPACE)
+  return attn_decode_run( "gh_attn_decode_static", q, layer_rows_dev, pos_dev, xb, batch, max_pos, shape, dt, g_static_scratch[device],
+                          STATIC_SCRATCH_BYTES, variant, stream, false );
 }
 
 int gh_attn_decode_host( const void* q, const void* const* layer_rows_host, const uint32_t* pos_host, void* xb, uint64_t batch,

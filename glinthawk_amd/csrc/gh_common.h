@@ -40,6 +40,10 @@ int fail( int status, const char* fmt, ... ) __attribute__( ( format( printf, 2,
 #define GH_LAUNCH_CHECK() GH_HIP( hipGetLastError() )
 
 int ensure_init();
+// device the library was initialised on, -1 before initialisation (never initialises)
+int initialised_device();
+// gh_attn_decode.hip: looks up the address of this device's static split-partial array; called once by the initialisation, with `device` current
+int attn_static_scratch_init( int device );
 // compute units of the device the library was initialised on (256 before initialisation)
 int cu_count();
 

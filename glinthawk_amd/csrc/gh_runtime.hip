@@ -123,6 +123,9 @@ static int init_locked( int device )
   if ( int rc = check_buffer_bounds() ) {
     return rc;
   }
+  if ( int rc = attn_static_scratch_init( device ) ) {
+    return rc;
+  }
   for ( int i = 0; i < STAGE_SLOTS; i++ ) {
     GH_HIP( hipHostMalloc( reinterpret_cast<void**>( &g_slots[i].pinned ), STAGE_SLOT_BYTES, hipHostMallocDefault ) );
     GH_HIP( hipMalloc( reinterpret_cast<void**>( &g_slots[i].device ), STAGE_SLOT_BYTES ) );
@@ -135,6 +138,12 @@ static int init_locked( int device )
 }
 
 int cu_count() { return g_cu_count; }
+
+int initialised_device()
+{
+  std::lock_guard<std::mutex> lock( g_mutex );
+  return g_ready ? g_device : -1;
+}
 
 int ensure_init()
 {

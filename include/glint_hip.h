@@ -224,6 +224,17 @@ int gh_attn_decode_plan( uint64_t batch, uint32_t max_pos, const gh_shape* shape
 int gh_attn_decode( const void* q, const void* const* layer_rows_dev, const uint32_t* pos_dev, void* xb, uint64_t batch,
                     uint32_t max_pos, const gh_shape* shape, gh_dtype dt, void* workspace, uint64_t workspace_bytes,
                     int variant, gh_stream stream );
+/* gh_attn_decode without a workspace argument and without any allocation.  It has no counterpart in the reference; it is
+ * for callers that cannot allocate device memory: code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc.  The split partials go to a fixed array in the library's device image instead
+ * (gh_attn_decode_static_limit() bytes, 16 MiB, per GPU, held until the process ends); a call whose plan needs more
+ * (see gh_attn_decode_plan) fails with GH_ERR_WORKSPACE.  Same kernels, same plan, same result as gh_attn_decode.
+ * gh_init() must have been called before: this entry point never initialises the library, because that allocates.
+ * All calls on one GPU share the one array: calls that overlap in time on one GPU (two streams, two threads) race.
+ * Nothing in the array needs clearing between calls: every partial that the merge reads was written by the same call. */
+uint64_t gh_attn_decode_static_limit( void );
+int gh_attn_decode_static( const void* q, const void* const* layer_rows_dev, const uint32_t* pos_dev, void* xb, uint64_t batch, uint32_t max_pos,
+                           const gh_shape* shape, gh_dtype dt, int variant, gh_stream stream );
 int gh_attn_decode_host( const void* q, const void* const* layer_rows_host, const uint32_t* pos_host, void* xb, uint64_t batch,
                          const gh_shape* shape, gh_dtype dt, void* workspace, uint64_t workspace_bytes, int variant, gh_stream stream );
 
