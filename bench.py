@@ -1,11 +1,11 @@
 #!/usr/bin/env python3
 """Benchmark of the per-stage Llama2 KV-cache path on one MI355X.
 
-One "step" is one pass of the hot path over one batch: the C++ stage driver's forward() for a
-pipeline stage of 10 layers of the Llama2-70B GQA shape (pre-attention, KV append, RoPE, fused
-decode attention, post-attention for every layer) with decode batch 64 and every context
-pre-filled so that the current token attends 4096 keys.  Inputs are synthetic (weights N(0,0.02),
-K/V rows N(0,1), activations N(0,1), all seeded) and resident in HBM before the timed region.
+One "step" is one pass of the hot path over one batch.  The headline workload is the C++ stage
+driver's forward() for a pipeline stage of 10 layers of the Llama2-70B GQA shape (pre-attention, KV
+append, RoPE, fused decode attention, post-attention for every layer) with decode batch 64 and every
+context pre-filled so that the current token attends 4096 keys.  Inputs are synthetic (weights
+N(0,0.02), K/V rows N(0,1), activations N(0,1), all seeded) and resident in HBM before the timed region.
 
 Prints ONE JSON line:
   value        decode-attention algorithmic bytes / time of the attention op (split-K kernel + merge)
@@ -14,14 +14,21 @@ Prints ONE JSON line:
   stage_*      whole stage step: tokens/s and the fraction of the bandwidth roofline, timed over K
                steps with no event between the kernels (ms_per_step); the K steps that carry the
                events run right after them and are reported as ms_per_step_with_attn_events
-  cpu_baseline the CPU oracle (a port of the reference's fp32 OpenMP path) timed on a bounded sample
+  cpu_baseline the CPU oracle (a port of the reference's fp32 OpenMP path) timed on a bounded sample:
+               one hosted layer on the very weights, cache rows and activations the GPU stage ran on
+  concept_path the same stage driven through the reference's own op sequence only (unfused attention
+               ops with a score buffer, separate projections, host-side tables staged per op)
+  other        short runs of the other decode / prefill / churn configurations, each with its own
+               roofline and CPU sample (leave out with --skip-others)
 """
 from __future__ import annotations
 
 import argparse
 import ctypes as C
+import hashlib
 import json
 import os
+import re
 import sys
 import time
 
@@ -29,11 +36,15 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+MFMA_PEAK_TFLOPS = 2500.0
 
-# HBM bytes per launch of the dominant kernel, from the FETCH_SIZE / WRITE_SIZE counter passes
-# summarised in profiles/attn_decode_mfma_llama2-70b-gqa-b64-ctx4096_hbm_counters.md (each counter
-# scaled by what it reads for a 1 GiB copy).  Only valid for the workload it was measured on.
-MEASURED_TRAFFIC = {"llama2-70b-gqa-b64-ctx4096": 1086915785}
+# HBM bytes per launch of the dominant kernel come from hardware counters (FETCH_SIZE / WRITE_SIZE under
+# rocprofv3, each scaled by what it reads for a plain copy); they cannot be read from inside this program.
+# The summary of that measurement names the kernel source it was taken on by its SHA-256; the figure is
+# reported only while that source is unchanged, otherwise `traffic` is null.
+TRAFFIC_PROFILE = {
+    "llama2-70b-gqa-b64-ctx4096": ("profiles/attn_decode_mfma_llama2-70b-gqa-b64-ctx4096_hbm_counters.md", "glinthawk_amd/csrc/gh_attn_decode.hip"),
+}
 
 # the decode configurations that fit one GPU as a single stage (the first is the headline)
 WORKLOADS = {
@@ -42,6 +53,12 @@ WORKLOADS = {
                                    "Llama2-70B GQA shape, one stage of 10 layers, fp16, decode batch 64, 4096 keys per context"),
     "llama2-7b-b32-ctx1024": ("llama2-7b", 8, 8, 32, 1024,
                               "Llama2-7B MHA shape, one stage of 8 layers, fp16, decode batch 32, 1024 keys per context"),
+}
+METRICS = {
+    "llama2-70b-gqa-b64-ctx4096": "decode attn HBM GB/s (% of peak) + stage tokens/s, Llama2-70B GQA, B=64, ctx 4096",
+    "llama2-7b-b32-ctx1024": "decode attn HBM GB/s (% of peak) + stage tokens/s, Llama2-7B MHA, B=32, ctx 1024",
+    "llama2-13b-prefill-8x2048": "prefill prompt tokens/s (+ decode ms/step), Llama2-13B shape, 8 x 2048 tokens, 10 layers",
+    "llama2-70b-churn-256": "tokens/s (decode + refill prefill), ragged slot churn, Llama2-70B GQA shape, 256 slots, 10 layers",
 }
 SHAPES = {
     "llama2-70b-4k": dict(dim=8192, n_heads=64, n_kv_heads=8, hidden_dim=28672, seq_len=4096, n_layers=80),
@@ -55,20 +72,48 @@ OTHER_WORKLOADS = {
     "llama2-70b-churn-256": "Llama2-70B GQA shape, one stage of 10 layers, fp16: 256 context slots with lengths U[16,4096]; every "
                             "step decodes all slots, then 10 % of them finish and are refilled in place with 128-token prefills",
 }
-MFMA_PEAK_TFLOPS = 2500.0
+LAYER_TENSORS = ("rms_att_weight", "wq", "wkv", "wo", "rms_ffn_weight", "w1", "w2", "w3")
+
+
+def kv_dim_of(shape):
+    return shape["dim"] // (shape["n_heads"] // shape["n_kv_heads"])
 
 
 def attention_bytes(shape, batch, keys, elem=2):
     """Algorithmic bytes of one layer's decode attention: every cached K and V element once, plus
     q read, output write and the appended row."""
-    kv_dim = shape["dim"] // (shape["n_heads"] // shape["n_kv_heads"])
+    kv_dim = kv_dim_of(shape)
     return batch * keys * 2 * kv_dim * elem + batch * (2 * shape["dim"] + 2 * kv_dim) * elem
 
 
 def layer_weight_bytes(shape, elem=2):
     d, h = shape["dim"], shape["hidden_dim"]
-    kv_dim = d // (shape["n_heads"] // shape["n_kv_heads"])
-    return (2 * d + 2 * d * d + 2 * d * kv_dim + 3 * d * h) * elem
+    return (2 * d + 2 * d * d + 2 * d * kv_dim_of(shape) + 3 * d * h) * elem
+
+
+def layer_matmul_flops(shape, tokens):
+    d, h = shape["dim"], shape["hidden_dim"]
+    return 2 * tokens * (2 * d * d + 2 * d * kv_dim_of(shape) + 3 * d * h)
+
+
+def measured_traffic(workload):
+    """(bytes per launch or None, note): the counter figure of the committed profile summary, if it was taken on
+    the kernel source as it is now."""
+    if workload not in TRAFFIC_PROFILE:
+        return None, "no counter profile for this workload"
+    summary, source = (os.path.join(ROOT, p) for p in TRAFFIC_PROFILE[workload])
+    try:
+        text = open(summary).read()
+        digest = hashlib.sha256(open(source, "rb").read()).hexdigest()
+    except OSError:
+        return None, "counter profile summary not present"
+    m_bytes = re.search(r"traffic_bytes_per_launch:\s*(\d+)", text)
+    m_hash = re.search(r"kernel_source_sha256:\s*([0-9a-f]{64})", text)
+    if not m_bytes or not m_hash:
+        return None, "counter profile summary carries no figure"
+    if m_hash.group(1) != digest:
+        return None, "kernel source changed since the counters were read"
+    return int(m_bytes.group(1)), os.path.relpath(summary, ROOT)
 
 
 def calibration_copy(n_bytes):
@@ -88,7 +133,58 @@ def calibration_copy(n_bytes):
     _lib.check(L.gh_free(dst))
 
 
-def gpu_bench(workload, steps, warmup):
+def download(ptr, n_elems, dtype):
+    import numpy as np
+
+    from glinthawk_amd import _lib
+    out = np.empty(n_elems, dtype=dtype)
+    _lib.check(_lib.lib().gh_memcpy(out.ctypes.data, ptr, out.nbytes, _lib.GH_D2H, 0, None), "gh_memcpy")
+    return out
+
+
+def layer_inputs_f32(st, shape, layer):
+    """The weights of one hosted layer and the RoPE tables as the GPU stage holds them, as fp32 for the CPU path."""
+    import numpy as np
+    d, h, kv = shape["dim"], shape["hidden_dim"], kv_dim_of(shape)
+    shapes = {"rms_att_weight": (d,), "wq": (d, d), "wkv": (2 * kv, d), "wo": (d, d), "rms_ffn_weight": (d,), "w1": (h, d), "w2": (d, h), "w3": (h, d)}
+    w = {name: st.get_layer_tensor(layer, name).astype(np.float32).reshape(shapes[name]) for name in LAYER_TENSORS}
+    hs = d // shape["n_heads"]
+    re = st.get_base_tensor("freq_cis_real").astype(np.float32).reshape(shape["seq_len"], hs // 2)
+    im = st.get_base_tensor("freq_cis_imag").astype(np.float32).reshape(shape["seq_len"], hs // 2)
+    return w, re, im
+
+
+def oracle_config(shape):
+    import oracle as O
+    return O.Config(dim=shape["dim"], n_layers=shape["n_layers"], n_heads=shape["n_heads"], n_kv_heads=shape["n_kv_heads"],
+                    hidden_dim=shape["hidden_dim"], seq_len=shape["seq_len"])
+
+
+def cpu_decode_layer(shape, w, re, im, layers, x, pos, reps=3):
+    """Median seconds of the oracle's layer (and of its attention ops alone) over `reps` runs after one warm-up."""
+    import numpy as np
+
+    import oracle as O
+    cfg = oracle_config(shape)
+    scratch = {}
+    layer_times, att_times = [], []
+    for rep in range(reps + 1):
+        xx = np.ascontiguousarray(x, dtype=np.float32).copy()
+        t0 = time.perf_counter()
+        scratch = O.layer_forward(cfg, w, re, im, xx, layers, pos, scratch)
+        t1 = time.perf_counter()
+        q = scratch["q"].copy()
+        O.attention_ops(cfg, pos, re, im, q, layers, att=scratch["att"])
+        t2 = time.perf_counter()
+        if rep:
+            layer_times.append(t1 - t0)
+            att_times.append(t2 - t1)
+    return float(np.median(layer_times)), float(np.median(att_times)), O.num_threads()
+
+
+def decode_bench(workload, steps, warmup, fused=True, cpu=True, events=True):
+    """A decode workload: K stage steps timed plain, K more with events around the attention launches, a plain
+    copy as the practical bandwidth ceiling, and (cpu) the oracle on the first hosted layer's own inputs."""
     import numpy as np
     import torch
 
@@ -100,13 +196,13 @@ def gpu_bench(workload, steps, warmup):
     ops.init(0)
     L = _lib.lib()
 
-    st = S.Stage(cfg_name, "f16", first, n_hosted, batch, batch, fused=True, seed=4, weight_std=0.02)
+    st = S.Stage(cfg_name, "f16", first, n_hosted, batch, batch, fused=fused, seed=4, weight_std=0.02)
     st.new_state(batch, next_layer=first)
     for i in range(batch):
         st.set_prompt(i, 1000 + i, 1, pos)
     assert st.acquire_contexts()
     # pre-fill: every slot gets N(0,1) rows for every hosted layer
-    kv_dim = shape["dim"] // (shape["n_heads"] // shape["n_kv_heads"])
+    kv_dim = kv_dim_of(shape)
     layer_elems = shape["seq_len"] * 2 * kv_dim
     for i in range(batch):
         for l in range(first, first + n_hosted):
@@ -133,25 +229,53 @@ def gpu_bench(workload, steps, warmup):
     ops.sync()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
-    # pass 2: the same steps with HIP events around every attention launch (an event record holds
-    # the next kernel back by a few microseconds, so this pass is not the one the step is timed on)
-    L.gh_attn_timing_enable(1)
-    L.gh_attn_timing_reset()
-    t2 = time.perf_counter()
-    for _ in range(steps):
-        one_step()
-    ops.sync()
-    torch.cuda.synchronize()
-    t3 = time.perf_counter()
-    k_ms, m_ms, n = C.c_double(0), C.c_double(0), C.c_uint64(0)
-    _lib.check(L.gh_attn_timing_read(C.byref(k_ms), C.byref(m_ms), C.byref(n)))
-    L.gh_attn_timing_enable(0)
+    res = dict(ms_per_step=(t1 - t0) * 1e3 / steps, batch=batch, device=ops.device_name())
+    a_bytes = attention_bytes(shape, batch, keys)
+    res.update(attn_bytes=a_bytes, stage_bytes=n_hosted * (a_bytes + layer_weight_bytes(shape)))
+    if events and fused:
+        # pass 2: the same steps with HIP events around every attention launch (an event record holds
+        # the next kernel back by a few microseconds, so this pass is not the one the step is timed on)
+        L.gh_attn_timing_enable(1)
+        L.gh_attn_timing_reset()
+        t2 = time.perf_counter()
+        for _ in range(steps):
+            one_step()
+        ops.sync()
+        torch.cuda.synchronize()
+        t3 = time.perf_counter()
+        k_ms, m_ms, n = C.c_double(0), C.c_double(0), C.c_uint64(0)
+        _lib.check(L.gh_attn_timing_read(C.byref(k_ms), C.byref(m_ms), C.byref(n)))
+        L.gh_attn_timing_enable(0)
+        launches = max(1, n.value)
+        res.update(ms_per_step_with_events=(t3 - t2) * 1e3 / steps, attn_kernel_ms=k_ms.value / launches,
+                   attn_merge_ms=m_ms.value / launches, attn_launches=int(n.value))
 
     out = st.activations().astype(np.float32)
     assert np.all(np.isfinite(out)), "stage output is not finite"
 
-    # what a plain device-to-device copy reaches on this box (bytes read + bytes written per second):
-    # the practical ceiling beside the published peak
+    if cpu:
+        # the CPU path on the first hosted layer: the same weights, the same cache rows, the same activations
+        w, re, im = layer_inputs_f32(st, shape, first)
+        layers = [download(st.context_layer_ptr(i, first), layer_elems, np.float16).astype(np.float32).reshape(shape["seq_len"], 2 * kv_dim)
+                  for i in range(batch)]
+        layer_s, att_s, cores = cpu_decode_layer(shape, w, re, im, layers, acts, [pos] * batch)
+        res["cpu_baseline"] = {
+            "value": batch / (layer_s * n_hosted), "unit": "tokens/s", "cores": cores, "kind": "port",
+            "sample": f"1 of {n_hosted} layers (B={batch}, {keys} keys) on the weights, cache rows and activations of the GPU run's first "
+                      f"hosted layer, held as fp32 like the reference's CPU build; median of 3 after 1 warm-up; layer time "
+                      f"{layer_s * 1e3:.0f} ms scaled x{n_hosted}",
+            "attn_GBps": attention_bytes(shape, batch, keys, elem=4) / att_s / 1e9,
+            "attn_ms_per_layer": att_s * 1e3, "layer_ms": layer_s * 1e3,
+        }
+        del w, layers
+    st.close()
+    return res
+
+
+def copy_ceiling_gbps():
+    """What a plain device-to-device copy reaches on this box (bytes read + bytes written per second): the
+    practical ceiling beside the published peak."""
+    import torch
     src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").zero_()
     dst = torch.empty_like(src)
     for _ in range(3):
@@ -162,38 +286,66 @@ def gpu_bench(workload, steps, warmup):
         dst.copy_(src)
     e1.record()
     torch.cuda.synchronize()
-    copy_gbps = 10 * 2 * src.numel() / (e0.elapsed_time(e1) * 1e-3) / 1e9
-    del src, dst
-
-    ms_per_step = (t1 - t0) * 1e3 / steps
-    launches = max(1, n.value)
-    kernel_ms = k_ms.value / launches
-    merge_ms = m_ms.value / launches
-    a_bytes = attention_bytes(shape, batch, keys)
-    stage_bytes = n_hosted * (a_bytes + layer_weight_bytes(shape))
-    res = dict(
-        ms_per_step=ms_per_step,
-        ms_per_step_with_events=(t3 - t2) * 1e3 / steps,
-        attn_kernel_ms=kernel_ms,
-        attn_merge_ms=merge_ms,
-        attn_launches=int(n.value),
-        attn_bytes=a_bytes,
-        stage_bytes=stage_bytes,
-        batch=batch,
-        device=ops.device_name(),
-        copy_gbps=copy_gbps,
-    )
-    st.close()
-    return res
+    return 10 * 2 * src.numel() / (e0.elapsed_time(e1) * 1e-3) / 1e9
 
 
-def layer_matmul_flops(shape, tokens):
-    d, h = shape["dim"], shape["hidden_dim"]
-    kv_dim = d // (shape["n_heads"] // shape["n_kv_heads"])
-    return 2 * tokens * (2 * d * d + 2 * d * kv_dim + 3 * d * h)
+def decode_line(workload, steps, warmup, attn_variant="auto", cpu=True):
+    """The JSON line of a decode workload."""
+    g = decode_bench(workload, steps, warmup, cpu=cpu)
+    cfg_name, first, n_hosted, batch, keys, desc = WORKLOADS[workload]
+    copy_gbps = copy_ceiling_gbps()
+    attn_op_ms = g["attn_kernel_ms"] + g["attn_merge_ms"]
+    value = g["attn_bytes"] / (attn_op_ms * 1e-3) / 1e9
+    achieved = g["attn_bytes"] / (g["attn_kernel_ms"] * 1e-3) / 1e9
+    tokens_per_s = batch / (g["ms_per_step"] * 1e-3)
+    stage_roofline_ms = g["stage_bytes"] / (HBM_PEAK_GBPS * 1e9) * 1e3
+    traffic, traffic_note = measured_traffic(workload)
+    return {
+        "metric": METRICS[workload],
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "pct_of_peak": round(100 * value / HBM_PEAK_GBPS, 2),
+        "copy_ceiling_gbps": round(copy_gbps, 1),
+        "pct_of_copy_ceiling": round(100 * value / copy_gbps, 2),
+        "stage_tokens_per_s": round(tokens_per_s, 1),
+        "stage_roofline_frac": round(stage_roofline_ms / g["ms_per_step"], 4),
+        "stage_bytes_per_step": g["stage_bytes"],
+        "n_gpus": 1,
+        "steps": steps,
+        "warmup": warmup,
+        "ms_per_step": round(g["ms_per_step"], 4),
+        "ms_per_step_with_attn_events": round(g["ms_per_step_with_events"], 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": workload, "description": desc, "stage_config": cfg_name, "first_layer": first,
+                   "hosted_layers": n_hosted, "batch": batch, "keys_per_context": keys, "device": g["device"],
+                   "attn_variant": attn_variant},
+        "attn_op_ms": round(attn_op_ms, 5),
+        "attn_kernel_ms": round(g["attn_kernel_ms"], 5),
+        "attn_merge_ms": round(g["attn_merge_ms"], 5),
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic, "traffic_source": traffic_note,
+                     "kernel": "attn_decode (split-K fused decode attention)", "launches_timed": g["attn_launches"],
+                     "algorithmic_bytes_per_launch": g["attn_bytes"]},
+        "cpu_baseline": g.get("cpu_baseline"),
+    }
 
 
-def prefill_bench(steps, warmup):
+def concept_path(workload, steps, warmup):
+    """The same stage driven only through the methods of the reference's operations interface, in the order its model
+    driver issues them (models/llama2/model.hh:326-427): separate projections, copy_kv_cache, apply_rope,
+    attention_0_gemm, attention_softmax, attention_2_gemm with the (batch, n_heads, seq_len) score buffer, and the
+    host-side context tables staged by every op.  What an unmodified model driver would execute on this backend."""
+    g = decode_bench(workload, steps, warmup, fused=False, cpu=False, events=False)
+    return {"ms_per_step": round(g["ms_per_step"], 4), "stage_tokens_per_s": round(g["batch"] / (g["ms_per_step"] * 1e-3), 1),
+            "stage_roofline_frac": round(g["stage_bytes"] / (HBM_PEAK_GBPS * 1e9) * 1e3 / g["ms_per_step"], 4),
+            "note": "unfused attention ops + score buffer, separate projection / element-wise ops, per-op host tables"}
+
+
+def prefill_bench(steps, warmup, cpu=True):
     """The prefill-heavy configuration.  One step = one batched prefill of 8 x 2048 prompt tokens through 10 layers
     (activations in and out over the boundary, like forward()); afterwards 64 decode steps on the same contexts."""
     import numpy as np
@@ -226,6 +378,27 @@ def prefill_bench(steps, warmup):
     t1 = time.perf_counter()
     assert np.isfinite(out.astype(np.float32)).all()
     ms = (t1 - t0) * 1e3 / steps
+
+    cpu_res = None
+    if cpu:
+        # The reference's CPU path feeds a prompt one token per forward (frontend/infer.cc:124-125): a step of all 8
+        # prompts at prompt position p costs one batch-8 layer pass over p + 1 keys.  Sampled at three positions on the
+        # first hosted layer, with the weights, the cache rows the GPU prefill wrote and the prompt's own input rows.
+        kv_dim = kv_dim_of(shape)
+        w, re, im = layer_inputs_f32(st, shape, first)
+        layers = [download(st.context_layer_ptr(i, first), T * 2 * kv_dim, np.float16).astype(np.float32).reshape(T, 2 * kv_dim) for i in range(batch)]
+        xin = x.reshape(batch, T, shape["dim"])
+        times = []
+        for p in (0, T // 2 - 1, T - 1):
+            layer_s, _, cores = cpu_decode_layer(shape, w, re, im, layers, xin[:, p], [p] * batch, reps=2)
+            times.append(layer_s)
+        mean_s = float(np.mean(times))
+        cpu_res = {"value": batch / (mean_s * n_hosted), "unit": "tokens/s", "cores": cores, "kind": "port",
+                   "sample": f"token-by-token prompt processing as the reference does it: 1 of {n_hosted} layers, the 8 prompts at positions "
+                             f"0, {T // 2 - 1} and {T - 1} (median of 2 after 1 warm-up each) on the GPU run's weights, cache rows and inputs held as "
+                             f"fp32; mean layer pass {mean_s * 1e3:.0f} ms scaled x{n_hosted}"}
+        del w, layers
+
     decode_steps = 64
     acts = x[:batch].copy()
     t0 = time.perf_counter()
@@ -242,7 +415,7 @@ def prefill_bench(steps, warmup):
     dev = ops.device_name()
     st.close()
     return {
-        "metric": "prefill prompt tokens/s (+ decode ms/step), Llama2-13B shape, 8 x 2048 tokens, 10 layers",
+        "metric": METRICS["llama2-13b-prefill-8x2048"],
         "value": round(batch * T / (ms * 1e-3), 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": round(ms, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
         "data": "synthetic",
@@ -252,13 +425,15 @@ def prefill_bench(steps, warmup):
                      "frac": round(flops / (ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4), "traffic": None,
                      "kernel": "whole prefill pass incl. host transfers (projection GEMMs + causal attention flops / step time)",
                      "algorithmic_flops_per_step": flops},
-        "cpu_baseline": None,
+        "cpu_baseline": cpu_res,
     }
 
 
-def churn_bench(steps, warmup):
+def churn_bench(steps, warmup, cpu=True):
     """The slot-churn configuration.  One step = decode of all 256 slots (ragged lengths), then the slots drawn
-    to finish (10 %, seeded) restart in place: a 128-token batched prefill into the same slot."""
+    to finish (10 %, seeded) restart in place: a 128-token batched prefill into the same slot.  The timed steps
+    start from the configuration's own length distribution U[16, 4096): the warm-up steps run first and the
+    positions are then set back (every row of every slot holds N(0,1) values, so any length is valid)."""
     import numpy as np
 
     from glinthawk_amd import _lib, ops, stage as S
@@ -269,23 +444,26 @@ def churn_bench(steps, warmup):
     L = _lib.lib()
     st = S.Stage(name, "f16", first, n_hosted, slots, slots, seed=5)
     rng = np.random.default_rng(5)
-    pos = rng.integers(16, 4096, slots)
+    start_pos = rng.integers(16, 4096, slots)
+    pos = start_pos.copy()
     ids = [1000 + i for i in range(slots)]
     st.new_state(slots, next_layer=first)
     for i in range(slots):
         st.set_prompt(i, ids[i], 1, int(pos[i]))
     assert st.acquire_contexts()
-    kv_dim = shape["dim"] // (shape["n_heads"] // shape["n_kv_heads"])
+    kv_dim = kv_dim_of(shape)
     for i in range(slots):
         for l in range(first, first + n_hosted):
             _lib.check(L.gh_fill_normal(st.context_layer_ptr(i, l), shape["seq_len"] * 2 * kv_dim, 0.0, 1.0, 7 + i * 131 + l, _lib.GH_F16, None))
     slot_of = [st.context_slot(i) for i in range(slots)]
+    first_layer_rows = [st.context_layer_ptr(i, first) for i in range(slots)]       # slots never move
     acts = rng.standard_normal((slots, shape["dim"])).astype(np.float16)
     prompt = ops.pinned_empty((slots * refill, shape["dim"]), np.float16)
     prompt[:] = rng.standard_normal(prompt.shape).astype(np.float16)
     decoded = prefilled = restarts = 0
     keys_read = 0
     t_decode = t_prefill = 0.0
+    per_step = []
 
     def one_step(count):
         nonlocal decoded, prefilled, restarts, keys_read, t_decode, t_prefill
@@ -301,6 +479,7 @@ def churn_bench(steps, warmup):
             decoded += slots
             keys_read += int((pos + 1).sum())
             t_decode += t1 - t0
+            per_step.append((float((pos + 1).mean()), (t1 - t0) * 1e3))
         pos[:] = pos + 1
         done = (rng.random(slots) < 0.10) | (pos >= shape["seq_len"] - 1)
         gone = np.nonzero(done)[0]
@@ -320,6 +499,7 @@ def churn_bench(steps, warmup):
     for _ in range(warmup):
         one_step(False)
     ops.sync()
+    pos[:] = start_pos
     t0 = time.perf_counter()
     for _ in range(steps):
         one_step(True)
@@ -328,11 +508,25 @@ def churn_bench(steps, warmup):
     counts = st.slot_counts()
     assert counts == dict(free=0, allocated=slots, total=slots), counts
     ms = (t1 - t0) * 1e3 / steps
+
+    cpu_res = None
+    if cpu:
+        # one decode step of all 256 slots at the starting lengths on the first hosted layer (the refill prefills are not in the sample)
+        w, re, im = layer_inputs_f32(st, shape, first)
+        layers = [download(first_layer_rows[i], (int(start_pos[i]) + 1) * 2 * kv_dim, np.float16).astype(np.float32)
+                  .reshape(int(start_pos[i]) + 1, 2 * kv_dim) for i in range(slots)]
+        layer_s, _, cores = cpu_decode_layer(shape, w, re, im, layers, acts, [int(p) for p in start_pos], reps=2)
+        cpu_res = {"value": slots / (layer_s * n_hosted), "unit": "tokens/s", "cores": cores, "kind": "port",
+                   "sample": f"decode part only: 1 of {n_hosted} layers, all 256 slots at their starting lengths (mean {float((start_pos + 1).mean()):.0f} keys) on "
+                             f"the GPU run's weights, cache rows and activations held as fp32; median of 2 after 1 warm-up; layer time "
+                             f"{layer_s * 1e3:.0f} ms scaled x{n_hosted}"}
+        del w, layers
     dev = ops.device_name()
     st.close()
     kv_bytes = keys_read * 2 * kv_dim * 2 * n_hosted
+    decode_bytes = kv_bytes + steps * n_hosted * layer_weight_bytes(shape)
     return {
-        "metric": "tokens/s (decode + refill prefill), ragged slot churn, Llama2-70B GQA shape, 256 slots, 10 layers",
+        "metric": METRICS["llama2-70b-churn-256"],
         "value": round((decoded + prefilled) / (t1 - t0), 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": round(ms, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
         "data": "synthetic",
@@ -340,71 +534,25 @@ def churn_bench(steps, warmup):
         "decode_tokens_per_s": round(decoded / t_decode, 1), "decode_ms_per_step": round(t_decode * 1e3 / steps, 3),
         "prefill_tokens_per_s": round(prefilled / max(t_prefill, 1e-9), 1), "prefill_ms_per_step": round(t_prefill * 1e3 / steps, 3),
         "restarts": restarts, "mean_keys_per_slot": round(keys_read / max(decoded, 1), 1),
-        "roofline": {"bound": "hbm", "achieved": round((kv_bytes + steps * n_hosted * layer_weight_bytes(shape)) / t_decode / 1e9, 1),
-                     "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round((kv_bytes + steps * n_hosted * layer_weight_bytes(shape)) / t_decode / 1e9 / HBM_PEAK_GBPS, 4),
+        "decode_ms_by_mean_keys": [[round(k), round(m, 2)] for k, m in per_step],
+        "roofline": {"bound": "hbm", "achieved": round(decode_bytes / t_decode / 1e9, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(decode_bytes / t_decode / 1e9 / HBM_PEAK_GBPS, 4),
                      "traffic": None, "kernel": "whole decode step (cached K/V read once + weights once) / decode time"},
-        "cpu_baseline": None,
+        "cpu_baseline": cpu_res,
     }
 
 
-def cpu_baseline(workload):
-    """The oracle (port of the reference's fp32 amd64/OpenMP path) on ONE layer of the workload,
-    fp32 weights and fp32 K/V like the reference's CPU build, median of 3 after one warm-up; the
-    stage figure scales that layer time by the number of hosted layers."""
-    import numpy as np
-
-    import oracle as O
-
-    cfg_name, first, n_hosted, batch, keys, _ = WORKLOADS[workload]
-    s = SHAPES[cfg_name]
-    cfg = O.Config(dim=s["dim"], n_layers=s["n_layers"], n_heads=s["n_heads"], n_kv_heads=s["n_kv_heads"],
-                   hidden_dim=s["hidden_dim"], seq_len=s["seq_len"])
-    rng = np.random.default_rng(1)
-    block = rng.standard_normal(1 << 22).astype(np.float32)
-
-    def tiled(shape, scale):
-        n = int(np.prod(shape))
-        reps = (n + block.size - 1) // block.size
-        return (np.tile(block, reps)[:n] * np.float32(scale)).reshape(shape)
-
-    w = {
-        "rms_att_weight": tiled((cfg.dim,), 0.02), "wq": tiled((cfg.dim, cfg.dim), 0.02),
-        "wkv": tiled((2 * cfg.kv_dim, cfg.dim), 0.02), "wo": tiled((cfg.dim, cfg.dim), 0.02),
-        "rms_ffn_weight": tiled((cfg.dim,), 0.02), "w1": tiled((cfg.hidden_dim, cfg.dim), 0.02),
-        "w2": tiled((cfg.dim, cfg.hidden_dim), 0.02), "w3": tiled((cfg.hidden_dim, cfg.dim), 0.02),
-    }
-    re, im = O.rope_tables(cfg.seq_len, cfg.head_size)
-    cache = tiled((batch, cfg.seq_len, 2 * cfg.kv_dim), 1.0)
-    layers = [cache[i] for i in range(batch)]
-    pos = [keys - 1] * batch
-    scratch = {}
-    att_times, layer_times = [], []
-    for rep in range(4):
-        x = tiled((batch, cfg.dim), 1.0).copy()
-        t0 = time.perf_counter()
-        scratch = O.layer_forward(cfg, w, re, im, x, layers, pos, scratch)
-        t1 = time.perf_counter()
-        q = scratch["q"].copy()
-        O.attention_ops(cfg, pos, re, im, q, layers, att=scratch["att"])
-        t2 = time.perf_counter()
-        if rep:
-            layer_times.append(t1 - t0)
-            att_times.append(t2 - t1)
-    layer_s = float(np.median(layer_times))
-    att_s = float(np.median(att_times))
-    a_bytes32 = attention_bytes(s, batch, keys, elem=4)
-    return {
-        "value": batch / (layer_s * n_hosted),
-        "unit": "tokens/s",
-        "cores": O.num_threads(),
-        "kind": "port",
-        "sample": f"1 of {n_hosted} layers (B={batch}, {keys} keys, fp32 weights and K/V as in the reference's CPU build), "
-                  f"median of 3 after 1 warm-up; layer time {layer_s * 1e3:.0f} ms scaled x{n_hosted}",
-        "attn_GBps": a_bytes32 / att_s / 1e9,
-        "attn_ms_per_layer": att_s * 1e3,
-        "layer_ms": layer_s * 1e3,
-    }
+def brief(line):
+    """What the headline line keeps of another configuration's line."""
+    keep = ("value", "unit", "ms_per_step", "steps", "warmup", "stage_tokens_per_s", "stage_roofline_frac", "attn_kernel_ms", "decode_ms_per_step",
+            "decode_tokens_per_s", "prefill_ms_per_step", "prefill_tokens_per_s", "mean_keys_per_slot", "decode_ms_by_mean_keys")
+    out = {"workload": line["config"]["workload"], "metric": line["metric"]}
+    out.update({k: line[k] for k in keep if k in line})
+    r = line["roofline"]
+    out["roofline"] = {k: r[k] for k in ("bound", "achieved", "peak", "unit", "frac", "kernel")}
+    c = line.get("cpu_baseline")
+    out["cpu_baseline"] = None if c is None else {k: (round(c[k], 2) if k == "value" else c[k]) for k in ("value", "unit", "cores", "kind", "sample")}
+    return out
 
 
 def main():
@@ -414,8 +562,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="llama2-70b-gqa-b64-ctx4096", choices=sorted(WORKLOADS) + sorted(OTHER_WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--skip-others", action="store_true",
+                    help="only the named workload: no concept-path run and no short runs of the other configurations")
     ap.add_argument("--attn-variant", default="auto", choices=["auto", "generic", "valu", "mfma"],
                     help="decode attention kernel the stage uses (measurement of the alternatives; auto = the library's choice)")
+    ap.add_argument("--concept-path", action="store_true", help="time the named decode workload through the reference's op sequence only")
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="also run a plain D2D copy of this many MiB (reference point for profiler byte counters)")
     args = ap.parse_args()
@@ -425,6 +576,7 @@ def main():
               "(the path shards by context, slot -> GPU, with no collective; only the one-GPU share is built)", file=sys.stderr)
         sys.exit(2)
 
+    cpu = not args.no_cpu_baseline
     if args.calibration_copy_mib > 0:
         from glinthawk_amd import ops
         ops.init(0)
@@ -434,55 +586,27 @@ def main():
         ops.init(0)
         _lib.check(_lib.lib().gh_attn_set_auto_variant({"generic": 1, "valu": 2, "mfma": 3}[args.attn_variant]))
     if args.workload == "llama2-13b-prefill-8x2048":
-        print(json.dumps(prefill_bench(args.steps, args.warmup)))
+        print(json.dumps(prefill_bench(args.steps, args.warmup, cpu)))
         return
     if args.workload == "llama2-70b-churn-256":
-        print(json.dumps(churn_bench(args.steps, args.warmup)))
+        print(json.dumps(churn_bench(args.steps, args.warmup, cpu)))
         return
-    g = gpu_bench(args.workload, args.steps, args.warmup)
-    cfg_name, first, n_hosted, batch, keys, desc = WORKLOADS[args.workload]
+    if args.concept_path:
+        print(json.dumps({"workload": args.workload, "concept_path": concept_path(args.workload, args.steps, args.warmup)}))
+        return
 
-    attn_op_ms = g["attn_kernel_ms"] + g["attn_merge_ms"]
-    value = g["attn_bytes"] / (attn_op_ms * 1e-3) / 1e9
-    achieved = g["attn_bytes"] / (g["attn_kernel_ms"] * 1e-3) / 1e9
-    tokens_per_s = batch / (g["ms_per_step"] * 1e-3)
-    stage_roofline_ms = g["stage_bytes"] / (HBM_PEAK_GBPS * 1e9) * 1e3
-
-    line = {
-        "metric": "decode attn HBM GB/s (% of peak) + stage tokens/s, Llama2-70B GQA, B=64, ctx 4096",
-        "value": round(value, 1),
-        "unit": "GB/s",
-        "pct_of_peak": round(100 * value / HBM_PEAK_GBPS, 2),
-        "copy_ceiling_gbps": round(g["copy_gbps"], 1),
-        "pct_of_copy_ceiling": round(100 * value / g["copy_gbps"], 2),
-        "stage_tokens_per_s": round(tokens_per_s, 1),
-        "stage_roofline_frac": round(stage_roofline_ms / g["ms_per_step"], 4),
-        "stage_bytes_per_step": g["stage_bytes"],
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": round(g["ms_per_step"], 4),
-        "ms_per_step_with_attn_events": round(g["ms_per_step_with_events"], 4),
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "f16",
-        "data": "synthetic",
-        "config": {"workload": args.workload, "description": desc, "stage_config": cfg_name, "first_layer": first,
-                   "hosted_layers": n_hosted, "batch": batch, "keys_per_context": keys, "device": g["device"],
-                   "attn_variant": args.attn_variant},
-        "attn_op_ms": round(attn_op_ms, 5),
-        "attn_kernel_ms": round(g["attn_kernel_ms"], 5),
-        "attn_merge_ms": round(g["attn_merge_ms"], 5),
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC.get(args.workload),
-                     "kernel": "attn_decode (split-K fused decode attention)", "launches_timed": g["attn_launches"],
-                     "algorithmic_bytes_per_launch": g["attn_bytes"]},
-    }
-    if not args.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_baseline(args.workload)
-    else:
-        line["cpu_baseline"] = None
+    line = decode_line(args.workload, args.steps, args.warmup, args.attn_variant, cpu)
+    if not args.skip_others and args.workload == "llama2-70b-gqa-b64-ctx4096":
+        # bounded runs of everything else the configurations name, in the same process and the same line
+        line["concept_path_ms_per_step"] = None
+        cp = concept_path(args.workload, min(args.steps, 10), 2)
+        line["concept_path_ms_per_step"] = cp["ms_per_step"]
+        line["concept_path"] = cp
+        line["other"] = {
+            "cfg2": brief(decode_line("llama2-7b-b32-ctx1024", min(args.steps, 20), 3, "auto", cpu)),
+            "cfg3": brief(prefill_bench(3, 1, cpu)),
+            "cfg5": brief(churn_bench(16, 3, cpu)),
+        }
     print(json.dumps(line))
 
 

@@ -26,6 +26,8 @@ struct StageBase
   virtual ~StageBase() = default;
   virtual void set_layer_tensor( size_t layer, size_t k, const void* host, uint64_t n ) = 0;
   virtual void set_base_tensor( size_t k, const void* host, uint64_t n ) = 0;
+  virtual const void* layer_tensor_ptr( size_t layer, size_t k, uint64_t* n ) = 0;
+  virtual const void* base_tensor_ptr( size_t k, uint64_t* n ) = 0;
   virtual std::string load_dir( const char* model_dir ) = 0;
   virtual std::string set_state_bytes( const void* bytes, uint64_t len ) = 0;
   virtual std::string get_state_bytes() = 0;
@@ -88,6 +90,27 @@ struct StageImpl : StageBase
     model.set_layer_tensor( layer, k, static_cast<const DType*>( host ), n );
   }
   void set_base_tensor( size_t k, const void* host, uint64_t n ) override { model.set_base_tensor( k, static_cast<const DType*>( host ), n ); }
+  // device address and element count of a resident tensor (file order), nullptr / 0 when the stage does not host it
+  const void* layer_tensor_ptr( size_t layer, size_t k, uint64_t* n ) override
+  {
+    *n = 0;
+    if ( layer >= Config::n_layers || k >= 8 ) {
+      return nullptr;
+    }
+    *n = WeightLayout<Config>::layer_in_memory( model.settings(), layer )[k];
+    return *n ? model.layer_weights( layer ).tensor( k ) : nullptr;
+  }
+  const void* base_tensor_ptr( size_t k, uint64_t* n ) override
+  {
+    *n = 0;
+    if ( k >= 5 ) {
+      return nullptr;
+    }
+    const auto& b = model.base_weights();
+    const DType* const t[5] = { b.token_embedding_table, b.rms_final_weight, b.freq_cis_real, b.freq_cis_imag, b.wcls };
+    *n = t[k] ? WeightLayout<Config>::base_in_memory( model.settings() )[k] : 0;
+    return t[k];
+  }
 
   void new_state( uint32_t batch, uint32_t next_layer, int next_stage ) override
   {
@@ -491,6 +514,8 @@ int64_t glint_model_dir_walk( const char* config, int dtype, uint32_t first_laye
 }
 void glint_stage_set_layer_tensor( void* h, uint32_t layer, uint32_t k, const void* host, uint64_t n ) { static_cast<StageBase*>( h )->set_layer_tensor( layer, k, host, n ); }
 void glint_stage_set_base_tensor( void* h, uint32_t k, const void* host, uint64_t n ) { static_cast<StageBase*>( h )->set_base_tensor( k, host, n ); }
+const void* glint_stage_layer_tensor_ptr( void* h, uint32_t layer, uint32_t k, uint64_t* n ) { return static_cast<StageBase*>( h )->layer_tensor_ptr( layer, k, n ); }
+const void* glint_stage_base_tensor_ptr( void* h, uint32_t k, uint64_t* n ) { return static_cast<StageBase*>( h )->base_tensor_ptr( k, n ); }
 void glint_stage_new_state( void* h, uint32_t batch, uint32_t next_layer, int next_stage ) { static_cast<StageBase*>( h )->new_state( batch, next_layer, next_stage ); }
 void glint_stage_set_prompt( void* h, uint32_t row, uint32_t context_id, uint32_t token, uint32_t pos, float temperature, uint32_t prompt_length,
                              uint32_t max_completion_length )

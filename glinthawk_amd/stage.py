@@ -41,6 +41,8 @@ def host_lib() -> C.CDLL:
             "glint_stage_destroy": (None, [vp]),
             "glint_stage_set_layer_tensor": (None, [vp, u32, u32, vp, u64]),
             "glint_stage_set_base_tensor": (None, [vp, u32, vp, u64]),
+            "glint_stage_layer_tensor_ptr": (vp, [vp, u32, u32, C.POINTER(u64)]),
+            "glint_stage_base_tensor_ptr": (vp, [vp, u32, C.POINTER(u64)]),
             "glint_stage_new_state": (None, [vp, u32, u32, C.c_int]),
             "glint_stage_set_prompt": (None, [vp, u32, u32, u32, u32, C.c_float, u32, u32]),
             "glint_stage_discard": (None, [vp, u32]),
@@ -129,6 +131,25 @@ class Stage:
             raise GlintError(host_lib().glint_last_error().decode(errors="replace"))
 
     # ---- weights
+    def get_layer_tensor(self, layer: int, name: str) -> np.ndarray:
+        """A copy of a resident tensor of a hosted layer (1-D, the stage's storage type)."""
+        n = C.c_uint64(0)
+        ptr = host_lib().glint_stage_layer_tensor_ptr(self._h, layer, LAYER_TENSORS.index(name), C.byref(n))
+        return self._download(ptr, n.value, f"layer {layer} {name}")
+
+    def get_base_tensor(self, name: str) -> np.ndarray:
+        n = C.c_uint64(0)
+        ptr = host_lib().glint_stage_base_tensor_ptr(self._h, BASE_TENSORS.index(name), C.byref(n))
+        return self._download(ptr, n.value, name)
+
+    def _download(self, ptr, n: int, what: str) -> np.ndarray:
+        from . import _lib
+        if not ptr or n == 0:
+            raise GlintError(f"the stage does not host {what}")
+        out = np.empty(n, dtype=self.np_dtype)
+        _lib.check(_lib.lib().gh_memcpy(out.ctypes.data, ptr, out.nbytes, _lib.GH_D2H, 0, None), "gh_memcpy")
+        return out
+
     def set_layer_tensor(self, layer: int, name: str, arr: np.ndarray) -> None:
         a = np.ascontiguousarray(arr, dtype=self.np_dtype)
         host_lib().glint_stage_set_layer_tensor(self._h, layer, LAYER_TENSORS.index(name), a.ctypes.data, a.size)
