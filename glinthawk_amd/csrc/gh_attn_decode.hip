@@ -20,6 +20,7 @@
 // Scores are kept in the log2 domain: s2 = (q . k) * scale * log2(e), weights are exp2(s2 - m).
 // Partial format per (context, query head, split): out[head_size] floats (un-normalised), then m and l.
 #include "gh_common.h"
+#include "gh_attn_tiles.h"
 
 #include <algorithm>
 
@@ -27,7 +28,6 @@ namespace gh {
 namespace {
 
 constexpr float LOG2E = 1.4426950408889634f;
-constexpr int HS = 128; // head size of the fast kernels
 
 // Split-K partials of gh_attn_decode_static: one array per GPU the library runs on, held until the
 // process ends.  Host code never uses the array's name as an address: the device address is looked
@@ -40,18 +40,11 @@ float* g_static_scratch[MAX_DEVICES] = {};
 uint32_t g_chunk_override = 0;
 int g_auto_variant = GH_ATTN_AUTO; // what GH_ATTN_AUTO resolves to when the shape allows it (gh_attn_set_auto_variant)
 
-typedef _Float16 f16x4 __attribute__( ( ext_vector_type( 4 ) ) );
-typedef _Float16 f16x8 __attribute__( ( ext_vector_type( 8 ) ) );
-typedef _Float16 f16x2 __attribute__( ( ext_vector_type( 2 ) ) );
-typedef float f32x4 __attribute__( ( ext_vector_type( 4 ) ) );
-
 struct Partials
 {
   float* out; // [batch][n_heads][max_splits][head_size]
   float* ml;  // [batch][n_heads][max_splits][2]
 };
-
-__device__ __forceinline__ float fast_exp2( float x ) { return __builtin_amdgcn_exp2f( x ); }
 
 // =================================================================================================
 // generic kernel
@@ -189,95 +182,6 @@ __global__ __launch_bounds__( 256 ) void attn_merge_kernel( Partials part,
       acc += part.out[( slot0 + s ) * head_size + d] * fast_exp2( part.ml[( slot0 + s ) * 2] - m );
     }
     xb[( (uint64_t)ctx * n_heads + head ) * head_size + d] = from_f32<T>( acc * inv );
-  }
-}
-
-// =================================================================================================
-// shared pieces of the two fast kernels
-// =================================================================================================
-struct WaveJob
-{
-  const __half* base; // layer rows of the context
-  uint32_t ctx, h, split, t_begin, t_end;
-  bool valid;
-};
-
-// block -> (group of 4 kv heads, split, context); wave -> kv head.  Adjacent blocks cover adjacent
-// head groups of the same token range so that concurrently running blocks read whole cache rows.
-__device__ __forceinline__ WaveJob wave_job( const __half* const* layer_rows,
-                                             const uint32_t* pos,
-                                             uint32_t n_kv_heads,
-                                             uint32_t chunk,
-                                             uint32_t max_splits )
-{
-  WaveJob j;
-  const uint32_t wave = threadIdx.x >> 6;
-  const uint32_t n_hg = ( n_kv_heads + 3 ) / 4;
-  uint32_t bid = blockIdx.x;
-  const uint32_t hg = bid % n_hg;
-  bid /= n_hg;
-  j.split = bid % max_splits;
-  j.ctx = bid / max_splits;
-  j.h = hg * 4 + wave;
-  j.base = layer_rows[j.ctx];
-  const uint32_t n_tok = min( pos[j.ctx] + 1, max_splits * chunk ); // never beyond what the host sized the grid and the partials for
-  j.t_begin = j.split * chunk;
-  j.t_end = min( n_tok, j.t_begin + chunk );
-  j.valid = j.h < n_kv_heads && j.base != nullptr && j.t_begin < n_tok;
-  return j;
-}
-
-__device__ __forceinline__ float dpp_quad_xor1( float v )
-{
-  return __builtin_bit_cast( float, __builtin_amdgcn_update_dpp( 0, __builtin_bit_cast( int, v ), 0xB1, 0xF, 0xF, true ) );
-}
-__device__ __forceinline__ float dpp_quad_xor2( float v )
-{
-  return __builtin_bit_cast( float, __builtin_amdgcn_update_dpp( 0, __builtin_bit_cast( int, v ), 0x4E, 0xF, 0xF, true ) );
-}
-__device__ __forceinline__ float dpp_half_mirror( float v )
-{
-  return __builtin_bit_cast( float, __builtin_amdgcn_update_dpp( 0, __builtin_bit_cast( int, v ), 0x141, 0xF, 0xF, true ) );
-}
-__device__ __forceinline__ float dpp_row_mirror( float v )
-{
-  return __builtin_bit_cast( float, __builtin_amdgcn_update_dpp( 0, __builtin_bit_cast( int, v ), 0x140, 0xF, 0xF, true ) );
-}
-// sum over the 16 lanes of a DPP row; every lane of the row gets the total
-__device__ __forceinline__ float row16_sum( float v )
-{
-  v += dpp_quad_xor1( v );
-  v += dpp_quad_xor2( v );
-  v += dpp_half_mirror( v );
-  v += dpp_row_mirror( v );
-  return v;
-}
-
-__device__ __forceinline__ uint4 load16( const __half* p ) { return *reinterpret_cast<const uint4*>( p ); }
-// cache rows are read once per launch: non-temporal, so that they do not push the queries and partials out of the L2
-typedef uint32_t u32x4_t __attribute__( ( ext_vector_type( 4 ) ) );
-__device__ __forceinline__ uint4 load16_stream( const __half* p )
-{
-  return __builtin_bit_cast( uint4, __builtin_nontemporal_load( reinterpret_cast<const u32x4_t*>( p ) ) );
-}
-
-__device__ __forceinline__ float dot8( const uint4& a, const uint4& b, float acc )
-{
-  acc = __builtin_amdgcn_fdot2( __builtin_bit_cast( f16x2, a.x ), __builtin_bit_cast( f16x2, b.x ), acc, false );
-  acc = __builtin_amdgcn_fdot2( __builtin_bit_cast( f16x2, a.y ), __builtin_bit_cast( f16x2, b.y ), acc, false );
-  acc = __builtin_amdgcn_fdot2( __builtin_bit_cast( f16x2, a.z ), __builtin_bit_cast( f16x2, b.z ), acc, false );
-  acc = __builtin_amdgcn_fdot2( __builtin_bit_cast( f16x2, a.w ), __builtin_bit_cast( f16x2, b.w ), acc, false );
-  return acc;
-}
-
-__device__ __forceinline__ void unpack8( const uint4& v, float out[8] )
-{
-  const uint32_t w[4] = { v.x, v.y, v.z, v.w };
-#pragma unroll
-  for ( int k = 0; k < 4; k++ ) {
-    const f16x2 h2 = __builtin_bit_cast( f16x2, w[k] );
-    out[2 * k] = (float)h2.x;
-    out[2 * k + 1] = (float)h2.y;
   }
 }
 

@@ -412,6 +412,81 @@ def test_unfused_attention_ops(dt, shape, host_tables):
     assert np.all(got[3] == 5.0)
 
 
+def _seq(shape, seq_len):
+    return Shape(dim=shape.dim, n_layers=1, n_heads=shape.n_heads, n_kv_heads=shape.n_kv_heads, hidden_dim=64, seq_len=seq_len)
+
+
+# the streaming kernels (f16, head size 128, row length a multiple of 8): every gqa they take, kv head counts that do not fill
+# a block, ragged positions around the 8- and 32-token boundaries, ranges long enough to be cut into several token ranges
+STREAM_CASES = [
+    ("mha", _seq(MHA128, 640), [639, 0, 31, 32, 300]),
+    ("mha-odd", _seq(MHA128_ODD, 304), [303, 7, 8, 9]),
+    ("gqa2", _seq(GQA2, 280), [279, 255, 256, 257]),
+    ("gqa4", _seq(GQA4, 336), [335, 33, 1]),
+    ("gqa8", _seq(GQA8, 704), [703, 500, 15, 16]),
+    ("gqa16", _seq(GQA16, 304), [303, 63, 64]),
+    ("gqa8-long", _seq(GQA8, 4096), [4095, 2048, 777]),
+    ("mha-long", _seq(MHA128, 2048), [2047, 1025]),
+]
+
+
+@pytest.mark.parametrize("name,shape,pos", STREAM_CASES, ids=[c[0] for c in STREAM_CASES])
+@pytest.mark.parametrize("host_tables", [False, True])
+def test_unfused_attention_ops_streaming_kernels(name, shape, pos, host_tables):
+    batch = len(pos) + 1
+    pos = list(pos) + [5]
+    present = [True] * (batch - 1) + [False]
+    cfg = oracle_cfg(shape)
+    arena = Arena(shape, batch, torch.float16, seed=21)
+    rng = np.random.default_rng(22)
+    q = rng.standard_normal((batch, shape.dim)).astype(np.float16)
+    layers = [arena.layer_ptr(i) if present[i] else 0 for i in range(batch)]
+    host_layers = [arena.host[i] if present[i] else None for i in range(batch)]
+    att0 = np.full((batch, shape.n_heads, shape.seq_len), 3.0, np.float16)
+    datt = torch.from_numpy(att0).cuda()
+    dq = torch.from_numpy(q).cuda()
+    dpos = torch.tensor(pos, dtype=torch.int32, device="cuda")
+
+    att = att0.copy()
+    O.attention_0_gemm(cfg, q, host_layers, att, pos)
+    if host_tables:
+        ops.attn_scores_host(dq, layers, datt, pos, shape)
+    else:
+        ops.attn_scores(dq, ops.row_table(layers), datt, dpos, shape)
+    got = datt.cpu().numpy()
+    np.testing.assert_allclose(got.astype(np.float64), att.astype(np.float64), rtol=4e-3, atol=4e-3)
+    _, frac = half_ulp_diff(got, att)
+    assert frac < 0.02                                   # same fp32 sums up to their order: nearly every score is bit-equal
+    for i in range(batch):                               # beyond pos and empty contexts: untouched
+        n = pos[i] + 1 if present[i] else 0
+        assert np.all(got[i, :, n:] == 3.0)
+
+    datt = torch.from_numpy(att).cuda()
+    O.attention_softmax(cfg, att, pos)
+    if host_tables:
+        ops.attn_softmax_host(datt, pos, shape)
+    else:
+        ops.attn_softmax(datt, dpos, shape)
+    got = datt.cpu().numpy()
+    for i in range(batch):
+        n = pos[i] + 1
+        ulps, frac = half_ulp_diff(got[i, :, :n], att[i, :, :n])
+        assert ulps <= 1 and frac < 0.05, (i, ulps, frac)   # same rounding points; the sum's order and expf may move the last place
+        assert np.array_equal(got[i, :, n:], att[i, :, n:])
+
+    datt = torch.from_numpy(att).cuda()
+    xb = np.full((batch, shape.dim), 5.0, np.float16)
+    dxb = torch.full((batch, shape.dim), 5.0, dtype=torch.float16, device="cuda")
+    O.attention_2_gemm(cfg, att, host_layers, xb, pos)
+    if host_tables:
+        ops.attn_pv_host(datt, layers, dxb, pos, shape)
+    else:
+        ops.attn_pv(datt, ops.row_table(layers), dxb, dpos, shape)
+    got = dxb.cpu().numpy()
+    np.testing.assert_allclose(got.astype(np.float64), xb.astype(np.float64), rtol=3e-3, atol=3e-3)
+    assert np.all(got[batch - 1] == 5.0)
+
+
 # ------------------------------------------------------------------ fused decode attention
 def run_fused_case(shape, dt, variant, pos, present, chunk, seed=13, host_tables=False, std=1.0):
     batch = len(pos)
