@@ -112,6 +112,7 @@ SIGNATURES = {
     "gh_attn_decode_static": (_i, [_vp, _vp, _vp, _vp, _u64, _u32, _shp, _i, _i, _vp]),
     "gh_attn_decode_host": (_i, [_vp, _vp, _vp, _vp, _u64, _shp, _i, _vp, _u64, _i, _vp]),
     "gh_prefill_tables": (_i, [_vp, _vp, _u64, _u32, _u64, _vp, _vp, _vp, _vp]),
+    "gh_attn_set_prefill_tiles": (_i, [_i]),
     "gh_attn_prefill_workspace": (_u64, [_u64, _u32, _shp]),
     "gh_attn_prefill": (_i, [_vp, _vp, _vp, _vp, _u64, _u32, _u32, _shp, _i, _vp, _u64, _i, _vp]),
     "gh_attn_timing_enable": (_i, [_i]),

@@ -4,16 +4,7 @@
 // frontend/infer.cc:124-125, models/llama2/model.hh:356-357); the result of this kernel equals T
 // sequential calls of the decode path.
 //
-// f16, head size 128: MFMA kernel.  A wave owns 16 query columns of one (context, kv head): 16/gqa
-// consecutive tokens x the gqa query heads that share the kv head.  It streams the keys in tiles of
-// 16 exactly like the decode kernel (K through a wave-private swizzled LDS tile into
-// v_mfma_f32_16x16x32_f16 operand order, S^T lands in the A-operand order of
-// v_mfma_f32_16x16x16_f16, V transposed in registers), with a per-column causal mask.  The four
-// waves of a block take neighbouring query groups and need almost the same keys: the block streams
-// them once, 64 keys per step into an LDS stage (every wave fetches a quarter, the next step's rows
-// are in flight in registers meanwhile), and each wave works through the four 16-key tiles of the
-// stage that its queries can see.  Four blocks per CU: the per-tile chain of MFMA, softmax and
-// shuffles is latency-bound, so occupancy matters more than the 4 spilled registers it costs.
+// f16, head size 128: a tiled MFMA kernel (see attn_prefill_mfma_kernel).
 //
 // Any other shape: the decode kernels are run on tables expanded to one entry per (context, token).
 #include "gh_common.h"
@@ -22,17 +13,24 @@ namespace gh {
 namespace {
 
 constexpr float LOG2E = 1.4426950408889634f;
+constexpr float LAZY = 8.0f; // see the softmax step of the tiled prefill kernel
 constexpr int HS = 128;
 #ifndef PF_WGS_PER_CU
-#define PF_WGS_PER_CU 4
+#define PF_WGS_PER_CU 1
 #endif
 
 typedef _Float16 f16x4 __attribute__( ( ext_vector_type( 4 ) ) );
 typedef _Float16 f16x8 __attribute__( ( ext_vector_type( 8 ) ) );
 typedef float f32x4 __attribute__( ( ext_vector_type( 4 ) ) );
+typedef float f32x16 __attribute__( ( ext_vector_type( 16 ) ) );
 
 __device__ __forceinline__ float fast_exp2( float x ) { return __builtin_amdgcn_exp2f( x ); }
-__device__ __forceinline__ uint4 load16( const __half* p ) { return *reinterpret_cast<const uint4*>( p ); }
+// Cache rows are reached through pointers read from a table, so the compiler cannot tell that they are global memory and would
+// use flat loads, which count against the LDS wait counter as well: every wait for an LDS read would then also wait for the rows
+// of the next stage that are meant to stay in flight.  The cast names the address space.
+typedef uint32_t u32x4_t __attribute__( ( ext_vector_type( 4 ) ) );
+typedef const u32x4_t __attribute__( ( address_space( 1 ) ) ) global_u32x4_t;
+__device__ __forceinline__ uint4 load16( const __half* p ) { return __builtin_bit_cast( uint4, *(global_u32x4_t*)( p ) ); }
 
 // one entry per (context, token): the decode-style tables of a prefill step
 __global__ __launch_bounds__( 256 ) void expand_tables_kernel( const void* const* __restrict__ layer_rows,
@@ -62,211 +60,315 @@ __global__ __launch_bounds__( 256 ) void expand_tables_kernel( const void* const
   }
 }
 
-// q, xb: (batch * n_tokens, n_kv_heads * G * 128), row index = context * n_tokens + token
-template<int G>
-__global__ __launch_bounds__( 256, PF_WGS_PER_CU ) void attn_prefill_mfma_kernel( const __half* __restrict__ q,
+// q, xb: (batch * n_tokens, n_kv_heads * G * 128), row index = context * n_tokens + token.
+// Query column c of a (context, kv head): token c / G, query head c % G (the G heads that share the kv head).
+//
+// block = 4 waves = 256 query columns; wave = 64 columns = two 32-column MFMA tiles.  Per 64-key stage (K and V rows in LDS,
+// the next stage's rows in flight in registers):
+//   S^T = K Q^T   v_mfma_f32_32x32x16_f16, A = K rows out of LDS (16-byte chunks, XOR-swizzled), B = Q^T in registers; every A
+//                 fragment feeds both column tiles.  A lane ends up with 16 of the 32 keys of a sub-tile for ITS query column,
+//                 the lane 32 further on with the other 16: maximum and sum stay inside a lane but for one exchange per stage
+//   O^T += V^T P^T  the scores of a lane are, as they lie, the B operand (keys x its column) of the same instruction; the A
+//                 operand V^T (4 consecutive dims x 8 keys per lane) is put together from 8-byte LDS reads with v_perm and again
+//                 feeds both column tiles.  Every accumulator of a lane belongs to its own column: rescaling needs no shuffle
+// Causal mask only on stages that reach a wave's diagonal; stages beyond it are skipped.
+template<int G, int NQT>
+__global__ __launch_bounds__( 256, NQT == 1 ? 2 : 1 ) void attn_prefill_mfma_kernel( const __half* __restrict__ q,
                                                                    const __half* const* __restrict__ layer_rows,
                                                                    const uint32_t* __restrict__ start_pos,
                                                                    __half* __restrict__ xb,
                                                                    uint32_t n_kv_heads,
                                                                    uint32_t n_tokens,
-                                                                   uint32_t groups_per_head, // ceil(n_tokens / (16 / G))
+                                                                   uint32_t col_blocks, // ceil(n_tokens * G / (128 * NQT))
                                                                    float scale_log2e )
 {
-  __shared__ uint4 s_kt[64 * 16]; // 64 keys x 256 bytes, 16-byte chunks XOR-swizzled per 16-key tile
+  __shared__ uint4 s_kt[64 * 16]; // 64 keys x 256 bytes, 16-byte chunks XOR-swizzled by the key's low bits
   __shared__ uint4 s_vt[64 * 16]; // the same keys' value rows, plain
-  constexpr uint32_t TPG = 16 / G; // tokens per query group
+  static_assert( 32 * NQT >= G, "a wave holds whole tokens" );
+  constexpr uint32_t TPW = 32 * NQT / G; // tokens per wave
 
-  const uint32_t wave = threadIdx.x >> 6;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane( threadIdx.x >> 6 ); // provably uniform: what derives from it stays in scalar registers
   const uint32_t lane = threadIdx.x & 63;
-  const uint32_t c = lane & 15;
-  const uint32_t g4 = lane >> 4;
-  // block -> (group quad, kv head, context); wave -> group inside the quad
-  const uint32_t quads = ( groups_per_head + 3 ) / 4;
+  const uint32_t r = lane & 31;
+  const uint32_t g2 = lane >> 5;
+  // block -> (column block, kv head, context); the column blocks with the most keys are numbered first
   uint32_t bid = blockIdx.x;
-  const uint32_t quad = bid % quads;
-  bid /= quads;
+  const uint32_t cb = col_blocks - 1 - bid % col_blocks;
+  bid /= col_blocks;
   const uint32_t h = bid % n_kv_heads;
   const uint32_t ctx = bid / n_kv_heads;
-  const uint32_t group = quad * 4 + wave;
   const __half* base = layer_rows[ctx];
   if ( base == nullptr ) {
     return; // the whole work-group
   }
-  const bool wave_ok = group < groups_per_head; // a wave without queries still loads its share of every tile
   const uint32_t n_heads = n_kv_heads * G;
   const uint64_t row_elems = 2ull * n_kv_heads * HS;
   const uint32_t v_off = n_kv_heads * HS;
   const uint32_t start = start_pos[ctx];
 
-  // this lane's query column: token tq, head gq; invalid beyond n_tokens
-  const uint32_t tq = group * TPG + c / G;
-  const uint32_t gq = c % G;
-  const bool col_ok = wave_ok && tq < n_tokens;
-  const int32_t qpos = col_ok ? (int32_t)( start + tq ) : -1; // last visible key of the column
-  const uint32_t last_tok = min( n_tokens, ( group + 1 ) * TPG ) - 1;
-  const uint32_t t_end = wave_ok ? start + last_tok + 1 : 0; // keys [0, t_end) are visible to some column of the group
-  // the work-group streams the keys its last group needs; every wave loads a quarter of each 64-key tile
-  const uint32_t last_group = min( groups_per_head, quad * 4 + 4 ) - 1;
-  const uint32_t wg_end = start + min( n_tokens, ( last_group + 1 ) * TPG );
+  const uint32_t wave_tok0 = ( cb * 4 + wave ) * TPW;          // first token of the wave
+  const bool wave_ok = wave_tok0 < n_tokens;                    // a wave without queries still loads its share of every stage
+  const uint32_t wave_last = min( n_tokens, wave_tok0 + TPW ) - 1;
+  const uint32_t t_end = wave_ok ? start + wave_last + 1 : 0;   // keys [0, t_end) are visible to some column of the wave
+  const uint32_t t_all = start + wave_tok0 + 1;                 // keys [0, t_all) are visible to every column of the wave
+  const uint32_t wg_end = start + min( n_tokens, ( cb + 1 ) * 4 * TPW );
 
-  f16x8 qb[4];
-  {
-    const __half* qp = q + ( ( (uint64_t)ctx * n_tokens + ( col_ok ? tq : 0 ) ) * n_heads + (uint64_t)h * G + gq ) * HS;
+  // this lane's two query columns (tile 0 and tile 1): token, head, last visible key
+  uint32_t tq[NQT], gq[NQT];
+  int32_t qpos[NQT];
+  f16x8 qb[NQT][8];
 #pragma unroll
-    for ( int kk = 0; kk < 4; kk++ ) {
-      uint4 v = load16( qp + 8 * ( 4 * kk + g4 ) );
-      if ( !col_ok ) {
+  for ( int qt = 0; qt < NQT; qt++ ) {
+    const uint32_t col = 32 * qt + r;
+    tq[qt] = wave_tok0 + col / G;
+    gq[qt] = col % G;
+    const bool ok = wave_ok && tq[qt] < n_tokens;
+    qpos[qt] = ok ? (int32_t)( start + tq[qt] ) : -1;
+    const __half* qp = q + ( ( (uint64_t)ctx * n_tokens + ( ok ? tq[qt] : 0 ) ) * n_heads + (uint64_t)h * G + gq[qt] ) * HS;
+#pragma unroll
+    for ( int s = 0; s < 8; s++ ) {
+      uint4 v = load16( qp + 8 * ( 2 * s + g2 ) );
+      if ( !ok ) {
         v = make_uint4( 0, 0, 0, 0 );
       }
-      qb[kk] = __builtin_bit_cast( f16x8, v );
+      qb[qt][s] = __builtin_bit_cast( f16x8, v );
     }
   }
 
-  f32x4 acc[8];
+  f32x16 acc[NQT][4]; // [column tile][dim block i]: element v <-> dim 4 * (8*(v/4) + 4*g2 + v%4) + i of this lane's column
 #pragma unroll
-  for ( int nn = 0; nn < 8; nn++ ) {
-    acc[nn] = f32x4 { 0.0f, 0.0f, 0.0f, 0.0f };
+  for ( int qt = 0; qt < NQT; qt++ ) {
+#pragma unroll
+    for ( int i = 0; i < 4; i++ ) {
+#pragma unroll
+      for ( int v = 0; v < 16; v++ ) {
+        acc[qt][i][v] = 0.0f;
+      }
+    }
   }
-  float m = -INFINITY;
-  float l = 0.0f;
+  float m[NQT]; // reference point of the column's exponentials (log2 domain), identical in the two lanes that share the column;
+               // within LAZY of the running maximum
+  float l[NQT];                          // this lane's share of the running sum
+#pragma unroll
+  for ( int qt = 0; qt < NQT; qt++ ) {
+    m[qt] = -INFINITY;
+    l[qt] = 0.0f;
+  }
 
-  const __half* kp = base + (uint64_t)h * HS + 8 * c;
+  // global -> registers: thread t fetches chunk t % 16 of keys t / 16 + 16 j, K and V
+  const uint32_t ld_chunk = threadIdx.x & 15;
+  const uint32_t ld_key = threadIdx.x >> 4;
+  const __half* kp = base + (uint64_t)h * HS + 8 * ld_chunk;
   const uint4 zero4 = make_uint4( 0, 0, 0, 0 );
   uint4 kn[4], vn[4];
+  // rows of the stage after the current one: thread t fetches keys ld_key + 16 j of it; the pointer moves 64 rows per stage
+  const __half* next_rows = kp + (uint64_t)ld_key * row_elems;
+  const uint64_t row16 = 16 * row_elems, stage_step = 64 * row_elems;
+  auto fetch_stage = [&]( uint32_t first_key ) {
+    if ( __builtin_amdgcn_readfirstlane( first_key + 64 <= wg_end ) ) { // the whole stage lies inside the key range: no per-row guards
 #pragma unroll
-  for ( int i = 0; i < 4; i++ ) {
-    const uint32_t tok = 16 * wave + 4 * g4 + i;
-    const bool ok = tok < wg_end;
-    const __half* row = kp + (uint64_t)tok * row_elems;
-    kn[i] = ok ? load16( row ) : zero4;
-    vn[i] = ok ? load16( row + v_off ) : zero4;
-  }
+      for ( int j = 0; j < 4; j++ ) {
+        kn[j] = load16( next_rows + j * row16 );
+        vn[j] = load16( next_rows + j * row16 + v_off );
+      }
+    } else {
+      // the last, partial stage: rows past the range may hold anything (a weight of zero times a NaN is a NaN), they read as zero
+#pragma unroll
+      for ( int j = 0; j < 4; j++ ) {
+        const bool ok = first_key + ld_key + 16 * j < wg_end;
+        kn[j] = ok ? load16( next_rows + j * row16 ) : zero4;
+        vn[j] = ok ? load16( next_rows + j * row16 + v_off ) : zero4;
+      }
+    }
+    next_rows += stage_step;
+  };
+  fetch_stage( 0 );
 
-  for ( uint32_t tile0 = 0; tile0 < wg_end; tile0 += 64 ) {
-    uint4* kt = s_kt;
-    uint4* vt = s_vt;
-    if ( tile0 != 0 ) {
-      __syncthreads(); // every wave is done with the previous tile
+  for ( uint32_t t0 = 0; t0 < wg_end; t0 += 64 ) {
+    if ( t0 != 0 ) {
+      __syncthreads(); // every wave is done with the previous stage
     }
 #pragma unroll
-    for ( int i = 0; i < 4; i++ ) {
-      const uint32_t tl = 4 * g4 + i;
-      kt[( 16 * wave + tl ) * 16 + ( c ^ tl )] = kn[i];
-      vt[( 16 * wave + tl ) * 16 + c] = vn[i];
+    for ( int j = 0; j < 4; j++ ) {
+      const uint32_t key = ld_key + 16 * j;
+      s_kt[key * 16 + ( ld_chunk ^ ( key & 15 ) )] = kn[j];
+      s_vt[key * 16 + ld_chunk] = vn[j];
     }
-#pragma unroll
-    for ( int i = 0; i < 4; i++ ) {
-      const uint32_t tok = tile0 + 64 + 16 * wave + 4 * g4 + i;
-      const bool ok = tok < wg_end;
-      const __half* row = kp + (uint64_t)tok * row_elems;
-      kn[i] = ok ? load16( row ) : zero4;
-      vn[i] = ok ? load16( row + v_off ) : zero4;
+    if ( __builtin_amdgcn_readfirstlane( t0 + 64 < wg_end ) ) {
+      fetch_stage( t0 + 64 );
     }
     __syncthreads();
+    if ( __builtin_amdgcn_readfirstlane( t0 >= t_end ) ) {
+      continue; // nothing of this stage is visible to the wave's queries (it still took part in the loads and barriers)
+    }
+    // a stage that reaches the wave's diagonal hides keys from some columns; before it every key is visible to every column
+    const bool masked = __builtin_amdgcn_readfirstlane( t0 + 64 > t_all );
 
-    for ( uint32_t sub = 0; sub < 4; sub++ ) {
-      const uint32_t t0 = tile0 + 16 * sub;
-      if ( t0 >= t_end ) {
-        break; // wave-uniform: nothing further is visible to this wave's queries
+    // ---- scores: st[qt][sub][v] = raw score of key t0 + 32 sub + 8*(v/4) + 4*g2 + v%4 for column tile qt.  The two sub-tiles are
+    //      independent accumulation chains that alternate in the matrix pipe (keys past the diagonal are computed and masked)
+    f32x16 st[NQT][2];
+#pragma unroll
+    for ( int qt = 0; qt < NQT; qt++ ) {
+#pragma unroll
+      for ( int sub = 0; sub < 2; sub++ ) {
+#pragma unroll
+        for ( int v = 0; v < 16; v++ ) {
+          st[qt][sub][v] = 0.0f;
+        }
       }
-      const uint4* tile = kt + 16 * sub * 16;
-      uint4 vc[4];
+    }
 #pragma unroll
-      for ( int i = 0; i < 4; i++ ) {
-        vc[i] = vt[( 16 * sub + 4 * g4 + i ) * 16 + c];
+    for ( int s = 0; s < 8; s++ ) {
+#pragma unroll
+      for ( int sub = 0; sub < 2; sub++ ) {
+        const uint32_t krow = 32 * sub + r;
+        const f16x8 a = __builtin_bit_cast( f16x8, s_kt[krow * 16 + ( ( 2 * s + g2 ) ^ ( krow & 15 ) )] );
+#pragma unroll
+        for ( int qt = 0; qt < NQT; qt++ ) {
+          st[qt][sub] = __builtin_amdgcn_mfma_f32_32x32x16_f16( a, qb[qt][s], st[qt][sub], 0, 0, 0 );
+        }
       }
-
-      f32x4 st = f32x4 { 0.0f, 0.0f, 0.0f, 0.0f };
+    }
+    if ( masked ) {
 #pragma unroll
-      for ( int kk = 0; kk < 4; kk++ ) {
-        const uint4 kf = tile[c * 16 + ( ( 4 * kk + g4 ) ^ c )];
-        st = __builtin_amdgcn_mfma_f32_16x16x32_f16( __builtin_bit_cast( f16x8, kf ), qb[kk], st, 0, 0, 0 );
-      }
-
-      // st[i] = score of key t0 + 4*g4 + i for query column c; causal mask per column
-      float s[4];
-      float mt = -INFINITY;
+      for ( int qt = 0; qt < NQT; qt++ ) {
 #pragma unroll
-      for ( int i = 0; i < 4; i++ ) {
-        const int32_t key = (int32_t)( t0 + 4 * g4 + i );
-        s[i] = key <= qpos ? st[i] * scale_log2e : -INFINITY;
-        mt = fmaxf( mt, s[i] );
-      }
-      mt = fmaxf( mt, __shfl_xor( mt, 16, WAVE ) );
-      mt = fmaxf( mt, __shfl_xor( mt, 32, WAVE ) );
-      const float m_new = fmaxf( m, mt );
-      const float m_safe = m_new == -INFINITY ? 0.0f : m_new; // padding columns never see a key
-      const float alpha = fast_exp2( m - m_safe );
-      float p[4];
+        for ( int sub = 0; sub < 2; sub++ ) {
 #pragma unroll
-      for ( int i = 0; i < 4; i++ ) {
-        p[i] = fast_exp2( s[i] - m_safe );
-      }
-      l = l * alpha + ( p[0] + p[1] ) + ( p[2] + p[3] );
-      m = m_new;
-
-      if ( __builtin_amdgcn_ballot_w64( alpha != 1.0f ) != 0 ) {
-#pragma unroll
-        for ( int i = 0; i < 4; i++ ) {
-          const float a = __shfl( alpha, (int)( 4 * g4 + i ), WAVE );
-#pragma unroll
-          for ( int nn = 0; nn < 8; nn++ ) {
-            acc[nn][i] *= a;
+          for ( int v = 0; v < 16; v++ ) {
+            const int32_t key = (int32_t)( t0 + 32 * sub + 8 * ( v / 4 ) + 4 * g2 + ( v % 4 ) );
+            st[qt][sub][v] = key <= qpos[qt] ? st[qt][sub][v] : -INFINITY;
           }
         }
       }
+    }
 
-      const f16x4 pa = f16x4 { (_Float16)p[0], (_Float16)p[1], (_Float16)p[2], (_Float16)p[3] };
-      const uint32_t vw[4][4] = { { vc[0].x, vc[0].y, vc[0].z, vc[0].w },
-                                  { vc[1].x, vc[1].y, vc[1].z, vc[1].w },
-                                  { vc[2].x, vc[2].y, vc[2].z, vc[2].w },
-                                  { vc[3].x, vc[3].y, vc[3].z, vc[3].w } };
+    // ---- online softmax per column tile; p packed as B operands: pk[qt][2 sub + jj] = keys 32 sub + 16 jj + 8 (e/4) + 4 g2 + e%4, e = 0..7
+    f16x8 pk[NQT][4];
 #pragma unroll
-      for ( int w = 0; w < 4; w++ ) {
-        const uint2 lo = make_uint2( __builtin_amdgcn_perm( vw[1][w], vw[0][w], 0x05040100u ), __builtin_amdgcn_perm( vw[3][w], vw[2][w], 0x05040100u ) );
-        const uint2 hi = make_uint2( __builtin_amdgcn_perm( vw[1][w], vw[0][w], 0x07060302u ), __builtin_amdgcn_perm( vw[3][w], vw[2][w], 0x07060302u ) );
-        acc[2 * w] = __builtin_amdgcn_mfma_f32_16x16x16f16( pa, __builtin_bit_cast( f16x4, lo ), acc[2 * w], 0, 0, 0 );
-        acc[2 * w + 1] = __builtin_amdgcn_mfma_f32_16x16x16f16( pa, __builtin_bit_cast( f16x4, hi ), acc[2 * w + 1], 0, 0, 0 );
+    for ( int qt = 0; qt < NQT; qt++ ) {
+      float mx = st[qt][0][0];
+#pragma unroll
+      for ( int sub = 0; sub < 2; sub++ ) {
+#pragma unroll
+        for ( int v = 0; v < 16; v++ ) {
+          mx = fmaxf( mx, st[qt][sub][v] );
+        }
+      }
+      mx = fmaxf( mx, __shfl_xor( mx, 32, WAVE ) ) * scale_log2e; // log2 domain from here on
+      // The reference point of the exponentials only moves when the maximum has grown by more than 2^LAZY since it was set:
+      // weights stay below 2^LAZY (fine for fp32 sums and fp16 operands) and the 64 accumulators are rescaled rarely.  The
+      // result does not depend on the reference point.  -inf: a column that has seen no key yet (padding, or hidden so far).
+      if ( __builtin_amdgcn_ballot_w64( mx > m[qt] + LAZY ) != 0 ) {
+        const float m_new = fmaxf( m[qt], mx );
+        const float alpha = m_new == -INFINITY ? 1.0f : fast_exp2( m[qt] - m_new );
+        m[qt] = m_new;
+        l[qt] *= alpha;
+#pragma unroll
+        for ( int i = 0; i < 4; i++ ) {
+#pragma unroll
+          for ( int v = 0; v < 16; v++ ) {
+            acc[qt][i][v] *= alpha;
+          }
+        }
+      }
+      const float ms = m[qt] == -INFINITY ? 0.0f : m[qt];
+      float sum[2] = { 0.0f, 0.0f };
+#pragma unroll
+      for ( int sub = 0; sub < 2; sub++ ) {
+#pragma unroll
+        for ( int jj = 0; jj < 2; jj++ ) {
+          float p[8];
+#pragma unroll
+          for ( int e = 0; e < 8; e++ ) {
+            p[e] = fast_exp2( st[qt][sub][8 * jj + e] * scale_log2e - ms );
+            sum[e & 1] += p[e];
+          }
+          pk[qt][2 * sub + jj] = f16x8 { (_Float16)p[0], (_Float16)p[1], (_Float16)p[2], (_Float16)p[3],
+                                         (_Float16)p[4], (_Float16)p[5], (_Float16)p[6], (_Float16)p[7] };
+        }
+      }
+      l[qt] += sum[0] + sum[1];
+    }
+
+    // ---- O^T += V^T P^T: per 16 keys (kk) the lane reads dims 4r .. 4r+3 of its 8 key slots and transposes them into 4 A operands,
+    //      one per dim block i; the four dim blocks are independent accumulation chains
+#pragma unroll
+    for ( int kk = 0; kk < 4; kk++ ) {
+      uint2 vr[8];
+#pragma unroll
+      for ( int e = 0; e < 8; e++ ) {
+        const uint32_t key = 16 * kk + 8 * ( e / 4 ) + 4 * g2 + ( e % 4 );
+        vr[e] = *reinterpret_cast<const uint2*>( reinterpret_cast<const char*>( s_vt ) + key * 256 + 8 * r );
+      }
+#pragma unroll
+      for ( int i = 0; i < 4; i++ ) {
+        // dim 4r + i of the 8 keys: halves (i % 2) of word (i / 2) of every key's 8 bytes
+        const uint32_t sel = ( i % 2 ) ? 0x07060302u : 0x05040100u;
+        uint32_t w[8];
+#pragma unroll
+        for ( int e = 0; e < 8; e++ ) {
+          w[e] = ( i / 2 ) ? vr[e].y : vr[e].x;
+        }
+        const uint4 a4 = make_uint4( __builtin_amdgcn_perm( w[1], w[0], sel ), __builtin_amdgcn_perm( w[3], w[2], sel ),
+                                     __builtin_amdgcn_perm( w[5], w[4], sel ), __builtin_amdgcn_perm( w[7], w[6], sel ) );
+        const f16x8 a = __builtin_bit_cast( f16x8, a4 );
+#pragma unroll
+        for ( int qt = 0; qt < NQT; qt++ ) {
+          acc[qt][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16( a, pk[qt][kk], acc[qt][i], 0, 0, 0 );
+        }
       }
     }
   }
 
-  l += __shfl_xor( l, 16, WAVE );
-  l += __shfl_xor( l, 32, WAVE );
-
-  // the accumulators of this lane belong to query columns 4*g4 + i
+  // ---- normalise and store: element v of acc[qt][i] is dim 4 * (8*(v/4) + 4*g2 + v%4) + i of the lane's column
 #pragma unroll
-  for ( int i = 0; i < 4; i++ ) {
-    const uint32_t col = 4 * g4 + i;
-    const float lc = __shfl( l, (int)col, WAVE );
-    const uint32_t tok = group * TPG + col / G;
-    const uint32_t hd = col % G;
-    if ( tok < n_tokens ) {
-      const float inv = 1.0f / lc;
+  for ( int qt = 0; qt < NQT; qt++ ) {
+    const float lsum = l[qt] + __shfl_xor( l[qt], 32, WAVE );
+    if ( qpos[qt] < 0 ) {
+      continue; // padding column
+    }
+    const float inv = 1.0f / lsum;
+    __half* out = xb + ( ( (uint64_t)ctx * n_tokens + tq[qt] ) * n_heads + (uint64_t)h * G + gq[qt] ) * HS;
+#pragma unroll
+    for ( int v = 0; v < 16; v++ ) {
+      const uint32_t d0 = 4 * ( 8 * ( v / 4 ) + 4 * g2 + ( v % 4 ) );
       union
       {
-        uint4 raw;
-        __half hv[8];
+        uint2 raw;
+        __half hv[4];
       } o;
 #pragma unroll
-      for ( int nn = 0; nn < 8; nn++ ) {
-        o.hv[nn] = __float2half_rn( acc[nn][i] * inv );
+      for ( int i = 0; i < 4; i++ ) {
+        o.hv[i] = __float2half_rn( acc[qt][i][v] * inv );
       }
-      *reinterpret_cast<uint4*>( xb + ( ( (uint64_t)ctx * n_tokens + tok ) * n_heads + (uint64_t)h * G + hd ) * HS + 8 * c ) = o.raw;
+      *reinterpret_cast<uint2*>( out + d0 ) = o.raw;
     }
   }
 }
+
+template<int G, int NQT>
+void launch_prefill_tiles( hipStream_t st, const void* q, const void* const* rows, const uint32_t* start, void* xb, uint64_t batch, uint32_t n_tokens,
+                           const gh_shape* s )
+{
+  const uint32_t col_blocks = (uint32_t)( ( (uint64_t)n_tokens * G + 128 * NQT - 1 ) / ( 128 * NQT ) );
+  const uint64_t blocks = batch * s->n_kv_heads * col_blocks;
+  attn_prefill_mfma_kernel<G, NQT><<<(unsigned)blocks, 256, 0, st>>>( static_cast<const __half*>( q ), reinterpret_cast<const __half* const*>( rows ), start,
+                                                                     static_cast<__half*>( xb ), s->n_kv_heads, n_tokens, col_blocks,
+                                                                     LOG2E / sqrtf( (float)s->head_size ) );
+}
+
+int g_prefill_tiles = 1; // column tiles per wave
 
 template<int G>
 void launch_prefill( hipStream_t st, const void* q, const void* const* rows, const uint32_t* start, void* xb, uint64_t batch, uint32_t n_tokens,
                      const gh_shape* s )
 {
-  const uint32_t groups = ( n_tokens + ( 16 / G ) - 1 ) / ( 16 / G );
-  const uint64_t blocks = batch * s->n_kv_heads * ( ( groups + 3 ) / 4 );
-  attn_prefill_mfma_kernel<G><<<(unsigned)blocks, 256, 0, st>>>( static_cast<const __half*>( q ), reinterpret_cast<const __half* const*>( rows ), start,
-                                                                static_cast<__half*>( xb ), s->n_kv_heads, n_tokens, groups,
-                                                                LOG2E / sqrtf( (float)s->head_size ) );
+  if ( g_prefill_tiles == 2 ) {
+    launch_prefill_tiles<G, 2>( st, q, rows, start, xb, batch, n_tokens, s );
+  } else {
+    launch_prefill_tiles<G, 1>( st, q, rows, start, xb, batch, n_tokens, s );
+  }
 }
 
 } // namespace
@@ -291,6 +393,13 @@ int gh_prefill_tables( const void* const* layer_rows_dev, const uint32_t* start_
   expand_tables_kernel<<<(unsigned)( ( n + 255 ) / 256 ), 256, 0, as_stream( stream )>>>( layer_rows_dev, start_pos_dev, (uint32_t)batch, n_tokens, row_bytes,
                                                                                        layer_rows_out, token_rows_out, pos_out );
   GH_LAUNCH_CHECK();
+  return GH_OK;
+}
+
+int gh_attn_set_prefill_tiles( int column_tiles_per_wave )
+{
+  GH_REQUIRE( column_tiles_per_wave == 1 || column_tiles_per_wave == 2, "gh_attn_set_prefill_tiles: 1 or 2 column tiles per wave" );
+  g_prefill_tiles = column_tiles_per_wave;
   return GH_OK;
 }
 

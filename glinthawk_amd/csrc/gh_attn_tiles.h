@@ -76,12 +76,16 @@ __device__ __forceinline__ float row16_sum( float v )
   return v;
 }
 
-__device__ __forceinline__ uint4 load16( const __half* p ) { return *reinterpret_cast<const uint4*>( p ); }
-// cache rows are read once per launch: non-temporal, so that they do not push the queries and partials out of the L2
+// Cache rows are reached through pointers that come out of a table, so the compiler cannot tell that they are global memory
+// and would use flat loads.  Those count against the LDS wait counter as well: a wait for an LDS read would then also wait for
+// the rows of the next tile, which are meant to stay in flight.  The casts below name the address space.
 typedef uint32_t u32x4_t __attribute__( ( ext_vector_type( 4 ) ) );
+typedef const u32x4_t __attribute__( ( address_space( 1 ) ) ) global_u32x4_t;
+__device__ __forceinline__ uint4 load16( const __half* p ) { return __builtin_bit_cast( uint4, *(global_u32x4_t*)( p ) ); }
+// cache rows are read once per launch: non-temporal, so that they do not push the queries and partials out of the L2
 __device__ __forceinline__ uint4 load16_stream( const __half* p )
 {
-  return __builtin_bit_cast( uint4, __builtin_nontemporal_load( reinterpret_cast<const u32x4_t*>( p ) ) );
+  return __builtin_bit_cast( uint4, __builtin_nontemporal_load( (global_u32x4_t*)( p ) ) );
 }
 
 __device__ __forceinline__ float dot8( const uint4& a, const uint4& b, float acc )

@@ -254,6 +254,8 @@ int gh_prefill_tables( const void* const* layer_rows_dev, const uint32_t* start_
  * kernel; other shapes run the decode kernels on expanded tables (workspace needed, see
  * gh_attn_prefill_workspace).  max_start_pos: host-side upper bound of start_pos. */
 uint64_t gh_attn_prefill_workspace( uint64_t batch, uint32_t n_tokens, const gh_shape* shape );
+/* measurement hook: 32-column query tiles a wave of the tiled MFMA kernel owns (1: two waves per SIMD, the default; 2: one) */
+int gh_attn_set_prefill_tiles( int column_tiles_per_wave );
 int gh_attn_prefill( const void* q, const void* const* layer_rows_dev, const uint32_t* start_pos_dev, void* xb, uint64_t batch, uint32_t n_tokens,
                      uint32_t max_start_pos, const gh_shape* shape, gh_dtype dt, void* workspace, uint64_t workspace_bytes, int variant, gh_stream stream );
 
