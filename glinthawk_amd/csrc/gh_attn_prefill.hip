@@ -23,6 +23,11 @@ typedef _Float16 f16x4 __attribute__( ( ext_vector_type( 4 ) ) );
 typedef _Float16 f16x8 __attribute__( ( ext_vector_type( 8 ) ) );
 typedef float f32x4 __attribute__( ( ext_vector_type( 4 ) ) );
 typedef float f32x16 __attribute__( ( ext_vector_type( 16 ) ) );
+typedef __attribute__( ( address_space( 3 ) ) ) void* lds_ptr;
+typedef __attribute__( ( address_space( 3 ) ) ) char lds_char;
+typedef short v4s __attribute__( ( ext_vector_type( 4 ) ) );
+typedef short v8s __attribute__( ( ext_vector_type( 8 ) ) );
+typedef __attribute__( ( address_space( 3 ) ) ) v4s* lds_v4s;
 
 __device__ __forceinline__ float fast_exp2( float x ) { return __builtin_amdgcn_exp2f( x ); }
 // Cache rows are reached through pointers read from a table, so the compiler cannot tell that they are global memory and would
@@ -69,8 +74,8 @@ __global__ __launch_bounds__( 256 ) void expand_tables_kernel( const void* const
 //                 fragment feeds both column tiles.  A lane ends up with 16 of the 32 keys of a sub-tile for ITS query column,
 //                 the lane 32 further on with the other 16: maximum and sum stay inside a lane but for one exchange per stage
 //   O^T += V^T P^T  the scores of a lane are, as they lie, the B operand (keys x its column) of the same instruction; the A
-//                 operand V^T (4 consecutive dims x 8 keys per lane) is put together from 8-byte LDS reads with v_perm and again
-//                 feeds both column tiles.  Every accumulator of a lane belongs to its own column: rescaling needs no shuffle
+//                 operand V^T (one dim x 8 keys per lane) comes out of LDS with transposing reads (ds_read_b64_tr_b16).  Every
+//                 accumulator of a lane belongs to its own column: rescaling needs no shuffle
 // Causal mask only on stages that reach a wave's diagonal; stages beyond it are skipped.
 template<int G, int NQT>
 __global__ __launch_bounds__( 256, NQT == 1 ? 2 : 1 ) void attn_prefill_mfma_kernel( const __half* __restrict__ q,
@@ -80,10 +85,11 @@ __global__ __launch_bounds__( 256, NQT == 1 ? 2 : 1 ) void attn_prefill_mfma_ker
                                                                    uint32_t n_kv_heads,
                                                                    uint32_t n_tokens,
                                                                    uint32_t col_blocks, // ceil(n_tokens * G / (128 * NQT))
+                                                                   uint32_t n_pairs,    // batch * n_kv_heads
                                                                    float scale_log2e )
 {
-  __shared__ uint4 s_kt[64 * 16]; // 64 keys x 256 bytes, 16-byte chunks XOR-swizzled by the key's low bits
-  __shared__ uint4 s_vt[64 * 16]; // the same keys' value rows, plain
+  __shared__ uint4 s_kt[2][64 * 16]; // two stages of 64 keys x 256 bytes, 16-byte chunks XOR-swizzled by the key's low bits
+  __shared__ uint4 s_vt[2][64 * 16]; // the same keys' value rows, plain
   static_assert( 32 * NQT >= G, "a wave holds whole tokens" );
   constexpr uint32_t TPW = 32 * NQT / G; // tokens per wave
 
@@ -91,12 +97,18 @@ __global__ __launch_bounds__( 256, NQT == 1 ? 2 : 1 ) void attn_prefill_mfma_ker
   const uint32_t lane = threadIdx.x & 63;
   const uint32_t r = lane & 31;
   const uint32_t g2 = lane >> 5;
-  // block -> (column block, kv head, context); the column blocks with the most keys are numbered first
-  uint32_t bid = blockIdx.x;
-  const uint32_t cb = col_blocks - 1 - bid % col_blocks;
-  bid /= col_blocks;
-  const uint32_t h = bid % n_kv_heads;
-  const uint32_t ctx = bid / n_kv_heads;
+  // block -> (column block, kv head, context).  Work-groups go to the 8 XCDs in turn and every XCD has its own L2: all column
+  // blocks of a (context, kv head) pair are given to one XCD, next to each other in time, so that the pair's K and V rows are
+  // fetched into one L2 once instead of into all eight.  The column blocks with the most keys come first.
+  const uint32_t xcd = blockIdx.x & 7;
+  const uint32_t slot = blockIdx.x >> 3;
+  const uint32_t cb = col_blocks - 1 - slot % col_blocks;
+  const uint32_t pair = ( slot / col_blocks ) * 8 + xcd;
+  if ( pair >= n_pairs ) {
+    return; // padding of the grid to a multiple of 8 pairs (whole work-group)
+  }
+  const uint32_t h = pair % n_kv_heads;
+  const uint32_t ctx = pair / n_kv_heads;
   const __half* base = layer_rows[ctx];
   if ( base == nullptr ) {
     return; // the whole work-group
@@ -135,7 +147,7 @@ __global__ __launch_bounds__( 256, NQT == 1 ? 2 : 1 ) void attn_prefill_mfma_ker
     }
   }
 
-  f32x16 acc[NQT][4]; // [column tile][dim block i]: element v <-> dim 4 * (8*(v/4) + 4*g2 + v%4) + i of this lane's column
+  f32x16 acc[NQT][4]; // [column tile][dim block i4]: element v <-> dim 32 i4 + 8*(v/4) + 4*g2 + v%4 of this lane's column
 #pragma unroll
   for ( int qt = 0; qt < NQT; qt++ ) {
 #pragma unroll
@@ -155,58 +167,43 @@ __global__ __launch_bounds__( 256, NQT == 1 ? 2 : 1 ) void attn_prefill_mfma_ker
     l[qt] = 0.0f;
   }
 
-  // global -> registers: thread t fetches chunk t % 16 of keys t / 16 + 16 j, K and V
-  const uint32_t ld_chunk = threadIdx.x & 15;
-  const uint32_t ld_key = threadIdx.x >> 4;
-  const __half* kp = base + (uint64_t)h * HS + 8 * ld_chunk;
-  const uint4 zero4 = make_uint4( 0, 0, 0, 0 );
-  uint4 kn[4], vn[4];
-  // rows of the stage after the current one: thread t fetches keys ld_key + 16 j of it; the pointer moves 64 rows per stage
-  const __half* next_rows = kp + (uint64_t)ld_key * row_elems;
-  const uint64_t row16 = 16 * row_elems, stage_step = 64 * row_elems;
-  auto fetch_stage = [&]( uint32_t first_key ) {
-    if ( __builtin_amdgcn_readfirstlane( first_key + 64 <= wg_end ) ) { // the whole stage lies inside the key range: no per-row guards
-#pragma unroll
-      for ( int j = 0; j < 4; j++ ) {
-        kn[j] = load16( next_rows + j * row16 );
-        vn[j] = load16( next_rows + j * row16 + v_off );
-      }
-    } else {
-      // the last, partial stage: rows past the range may hold anything (a weight of zero times a NaN is a NaN), they read as zero
-#pragma unroll
-      for ( int j = 0; j < 4; j++ ) {
-        const bool ok = first_key + ld_key + 16 * j < wg_end;
-        kn[j] = ok ? load16( next_rows + j * row16 ) : zero4;
-        vn[j] = ok ? load16( next_rows + j * row16 + v_off ) : zero4;
-      }
-    }
-    next_rows += stage_step;
-  };
-  fetch_stage( 0 );
-
-  for ( uint32_t t0 = 0; t0 < wg_end; t0 += 64 ) {
-    if ( t0 != 0 ) {
-      __syncthreads(); // every wave is done with the previous stage
-    }
+  // global -> LDS without passing through registers (`buffer_load ... lds`, 16 bytes per lane): lane l of a wave lands at the
+  // wave's base + 16 l, i.e. an instruction fills 4 rows of 256 bytes; wave w fills rows 16 w + 4 j + l / 16, j = 0..3, of a stage.
+  // The swizzle of the K tile is applied to the address a lane fetches: the chunk that belongs in its slot.  The descriptor
+  // ends with the last key the work-group needs: rows past it read as zero whatever they hold (a weight of zero times a NaN
+  // would be a NaN).
+  const uint32_t row_bytes = (uint32_t)row_elems * 2;
+  const __amdgpu_buffer_rsrc_t kv_rsrc = __builtin_amdgcn_make_buffer_rsrc( const_cast<__half*>( base + (uint64_t)h * HS ), 0, (int)( wg_end * row_bytes ), 0x00020000 );
+  const uint32_t ld_g = lane >> 4, ld_pos = lane & 15;
+  const uint32_t k_voff = ld_g * row_bytes + ( ( ld_pos ^ ld_g ) * 16 ); // row 4 j + ld_g keeps chunk (ld_pos ^ ld_g ^ 4 j) in slot ld_pos
+  // V rows: the 32-byte pairs of a key's row are XORed with the key's low 3 bits, so that the transposing reads below (4 lanes per
+  // key and 32 bytes, 8 keys per instruction and half-wave) spread evenly over the banks: row 4 j + ld_g (low bits 4 (j & 1) + ld_g)
+  // keeps chunk ld_pos ^ 2 ld_g ^ 8 (j & 1) in slot ld_pos
+  const uint32_t v_voff = ld_g * row_bytes + ( ( ld_pos ^ ( 2 * ld_g ) ) * 16 ) + v_off * 2;
+  auto fetch_k = [&]( uint32_t buf, uint32_t stage ) {
 #pragma unroll
     for ( int j = 0; j < 4; j++ ) {
-      const uint32_t key = ld_key + 16 * j;
-      s_kt[key * 16 + ( ld_chunk ^ ( key & 15 ) )] = kn[j];
-      s_vt[key * 16 + ld_chunk] = vn[j];
+      __builtin_amdgcn_raw_ptr_buffer_load_lds( kv_rsrc, (lds_ptr)( s_kt[buf] + ( 16 * wave + 4 * j ) * 16 ), 16, k_voff ^ ( 64 * j ),
+                                                ( 64 * stage + 16 * wave + 4 * j ) * row_bytes, 0, 0 );
     }
-    if ( __builtin_amdgcn_readfirstlane( t0 + 64 < wg_end ) ) {
-      fetch_stage( t0 + 64 );
+  };
+  auto fetch_v = [&]( uint32_t buf, uint32_t stage ) {
+#pragma unroll
+    for ( int j = 0; j < 4; j++ ) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds( kv_rsrc, (lds_ptr)( s_vt[buf] + ( 16 * wave + 4 * j ) * 16 ), 16, v_voff ^ ( 128 * ( j & 1 ) ),
+                                                ( 64 * stage + 16 * wave + 4 * j ) * row_bytes, 0, 0 );
     }
-    __syncthreads();
-    if ( __builtin_amdgcn_readfirstlane( t0 >= t_end ) ) {
-      continue; // nothing of this stage is visible to the wave's queries (it still took part in the loads and barriers)
-    }
-    // a stage that reaches the wave's diagonal hides keys from some columns; before it every key is visible to every column
-    const bool masked = __builtin_amdgcn_readfirstlane( t0 + 64 > t_all );
+  };
 
-    // ---- scores: st[qt][sub][v] = raw score of key t0 + 32 sub + 8*(v/4) + 4*g2 + v%4 for column tile qt.  The two sub-tiles are
-    //      independent accumulation chains that alternate in the matrix pipe (keys past the diagonal are computed and masked)
-    f32x16 st[NQT][2];
+  // transposing V reads: lane j = 4 e + q of a 16-lane group points at key slot e (0..3) of its half-wave, dims 16 grp + 4 q .. + 3
+  // of dim block 0; the chunk index carries the V tile's swizzle (2 x the key's low 3 bits = 8 g2 + 2 e), dim block i4 flips bits 2, 3
+  const uint32_t tr_e = ( lane & 15 ) >> 2, tr_q = lane & 3, tr_grp = ( lane >> 4 ) & 1;
+  const uint32_t v_lane = ( 4 * g2 + tr_e ) * 256 + ( ( ( 2 * tr_grp + ( tr_q >> 1 ) ) ^ ( 8 * g2 + 2 * tr_e ) ) * 16 ) + ( tr_q & 1 ) * 8;
+
+  // scores of one stage: st[qt][sub][v] = raw score of key 32 sub + 8*(v/4) + 4*g2 + v%4 of the stage for column tile qt.  The two
+  // sub-tiles are independent accumulation chains that alternate in the matrix pipe; the K fragments of the next 16 dims are
+  // requested from LDS before the MFMAs of these
+  auto scores = [&]( f32x16 ( &st )[NQT][2], uint32_t buf ) {
 #pragma unroll
     for ( int qt = 0; qt < NQT; qt++ ) {
 #pragma unroll
@@ -217,19 +214,62 @@ __global__ __launch_bounds__( 256, NQT == 1 ? 2 : 1 ) void attn_prefill_mfma_ker
         }
       }
     }
-#pragma unroll
-    for ( int s = 0; s < 8; s++ ) {
+    f16x8 ka[2][2];
+    auto read_k = [&]( int s ) {
 #pragma unroll
       for ( int sub = 0; sub < 2; sub++ ) {
         const uint32_t krow = 32 * sub + r;
-        const f16x8 a = __builtin_bit_cast( f16x8, s_kt[krow * 16 + ( ( 2 * s + g2 ) ^ ( krow & 15 ) )] );
+        ka[s & 1][sub] = __builtin_bit_cast( f16x8, s_kt[buf][krow * 16 + ( ( 2 * s + g2 ) ^ ( krow & 15 ) )] );
+      }
+    };
+    read_k( 0 );
+#pragma unroll
+    for ( int s = 0; s < 8; s++ ) {
+      if ( s + 1 < 8 ) {
+        read_k( s + 1 );
+      }
+#pragma unroll
+      for ( int sub = 0; sub < 2; sub++ ) {
 #pragma unroll
         for ( int qt = 0; qt < NQT; qt++ ) {
-          st[qt][sub] = __builtin_amdgcn_mfma_f32_32x32x16_f16( a, qb[qt][s], st[qt][sub], 0, 0, 0 );
+          st[qt][sub] = __builtin_amdgcn_mfma_f32_32x32x16_f16( ka[s & 1][sub], qb[qt][s], st[qt][sub], 0, 0, 0 );
         }
       }
     }
-    if ( masked ) {
+  };
+
+  // Two LDS buffers each for K and V, one barrier per stage.  Behind the barrier of iteration i every wave is done with K of
+  // stage i (its scores were computed in iteration i-1) and with V of stage i-1, so K of stage i+2 and V of stage i+1 are
+  // requested into those buffers; the barrier of iteration i+1 waits for them.  The wave then turns the scores of stage i into
+  // weights (vector ALU), computes the scores of stage i+1 (matrix pipe, independent of the weights) and adds stage i's
+  // weighted values.
+  const uint32_t n_stages = ( wg_end + 63 ) / 64;
+  const uint32_t my_stages = ( t_end + 63 ) / 64; // stages that hold keys visible to this wave (it takes part in the loads and barriers of all)
+  fetch_k( 0, 0 );
+  fetch_k( 1, 1 );
+  fetch_v( 0, 0 );
+  __syncthreads();
+  f32x16 st[NQT][2];
+  if ( my_stages > 0 ) {
+    scores( st, 0 );
+  }
+
+  for ( uint32_t i = 0; i < n_stages; i++ ) {
+    const uint32_t t0 = 64 * i;
+    const uint32_t buf = i & 1;
+    __syncthreads();
+    if ( i + 2 < n_stages ) {
+      fetch_k( buf, i + 2 );
+    }
+    if ( i + 1 < n_stages ) {
+      fetch_v( buf ^ 1, i + 1 );
+    }
+    if ( i >= my_stages ) {
+      continue; // wave-uniform
+    }
+    // a stage that reaches the wave's diagonal hides keys from some columns; before it every key is visible to every column
+    if ( __builtin_amdgcn_readfirstlane( t0 + 64 > t_all ) ) {
+      asm volatile( "" ::: "memory" ); // keeps this a branch: the selects are only paid for on the diagonal
 #pragma unroll
       for ( int qt = 0; qt < NQT; qt++ ) {
 #pragma unroll
@@ -265,10 +305,10 @@ __global__ __launch_bounds__( 256, NQT == 1 ? 2 : 1 ) void attn_prefill_mfma_ker
         m[qt] = m_new;
         l[qt] *= alpha;
 #pragma unroll
-        for ( int i = 0; i < 4; i++ ) {
+        for ( int i4 = 0; i4 < 4; i4++ ) {
 #pragma unroll
           for ( int v = 0; v < 16; v++ ) {
-            acc[qt][i][v] *= alpha;
+            acc[qt][i4][v] *= alpha;
           }
         }
       }
@@ -291,37 +331,46 @@ __global__ __launch_bounds__( 256, NQT == 1 ? 2 : 1 ) void attn_prefill_mfma_ker
       l[qt] += sum[0] + sum[1];
     }
 
-    // ---- O^T += V^T P^T: per 16 keys (kk) the lane reads dims 4r .. 4r+3 of its 8 key slots and transposes them into 4 A operands,
-    //      one per dim block i; the four dim blocks are independent accumulation chains
+    // ---- the next stage's scores: nothing below depends on them
+    if ( i + 1 < my_stages ) {
+      scores( st, buf ^ 1 );
+    }
+
+    // ---- O^T += V^T P^T.  The A operand (32 dims x 16 keys; a lane: one dim, the 8 keys of its slots) comes out of LDS transposed:
+    //      ds_read_b64_tr_b16 hands lane i of a 16-lane group element i of each of four 32-byte rows that the group's lanes point
+    //      at (lanes 4 e .. 4 e + 3 at row e), i.e. 4 keys of one dim per instruction.  Dim block i4 holds dims 32 i4 .. 32 i4 + 31.
+    //      The four dim blocks are independent accumulation chains; the reads of the next 16 keys go out first.
+    v4s va[2][4][2];
+    auto read_v = [&]( int kk ) {
+#pragma unroll
+      for ( int i4 = 0; i4 < 4; i4++ ) {
+#pragma unroll
+        for ( int half = 0; half < 2; half++ ) {
+          va[kk & 1][i4][half] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (lds_v4s)( (lds_char*)s_vt[buf] + ( v_lane ^ ( 64 * i4 ) ) + ( 16 * kk + 8 * half ) * 256 ) );
+        }
+      }
+    };
+    read_v( 0 );
 #pragma unroll
     for ( int kk = 0; kk < 4; kk++ ) {
-      uint2 vr[8];
-#pragma unroll
-      for ( int e = 0; e < 8; e++ ) {
-        const uint32_t key = 16 * kk + 8 * ( e / 4 ) + 4 * g2 + ( e % 4 );
-        vr[e] = *reinterpret_cast<const uint2*>( reinterpret_cast<const char*>( s_vt ) + key * 256 + 8 * r );
+      if ( kk + 1 < 4 ) {
+        read_v( kk + 1 );
       }
 #pragma unroll
-      for ( int i = 0; i < 4; i++ ) {
-        // dim 4r + i of the 8 keys: halves (i % 2) of word (i / 2) of every key's 8 bytes
-        const uint32_t sel = ( i % 2 ) ? 0x07060302u : 0x05040100u;
-        uint32_t w[8];
-#pragma unroll
-        for ( int e = 0; e < 8; e++ ) {
-          w[e] = ( i / 2 ) ? vr[e].y : vr[e].x;
-        }
-        const uint4 a4 = make_uint4( __builtin_amdgcn_perm( w[1], w[0], sel ), __builtin_amdgcn_perm( w[3], w[2], sel ),
-                                     __builtin_amdgcn_perm( w[5], w[4], sel ), __builtin_amdgcn_perm( w[7], w[6], sel ) );
-        const f16x8 a = __builtin_bit_cast( f16x8, a4 );
+      for ( int i4 = 0; i4 < 4; i4++ ) {
+        const v4s lo = va[kk & 1][i4][0], hi = va[kk & 1][i4][1];
+        const v8s a8 = v8s { lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3] };
+        const f16x8 a = __builtin_bit_cast( f16x8, a8 );
 #pragma unroll
         for ( int qt = 0; qt < NQT; qt++ ) {
-          acc[qt][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16( a, pk[qt][kk], acc[qt][i], 0, 0, 0 );
+          acc[qt][i4] = __builtin_amdgcn_mfma_f32_32x32x16_f16( a, pk[qt][kk], acc[qt][i4], 0, 0, 0 );
         }
       }
     }
   }
 
-  // ---- normalise and store: element v of acc[qt][i] is dim 4 * (8*(v/4) + 4*g2 + v%4) + i of the lane's column
+  // ---- normalise and store: element v of acc[qt][i4] is dim 32 i4 + 8 (v / 4) + 4 g2 + v % 4 of the lane's column
 #pragma unroll
   for ( int qt = 0; qt < NQT; qt++ ) {
     const float lsum = l[qt] + __shfl_xor( l[qt], 32, WAVE );
@@ -331,18 +380,20 @@ __global__ __launch_bounds__( 256, NQT == 1 ? 2 : 1 ) void attn_prefill_mfma_ker
     const float inv = 1.0f / lsum;
     __half* out = xb + ( ( (uint64_t)ctx * n_tokens + tq[qt] ) * n_heads + (uint64_t)h * G + gq[qt] ) * HS;
 #pragma unroll
-    for ( int v = 0; v < 16; v++ ) {
-      const uint32_t d0 = 4 * ( 8 * ( v / 4 ) + 4 * g2 + ( v % 4 ) );
-      union
-      {
-        uint2 raw;
-        __half hv[4];
-      } o;
+    for ( int i4 = 0; i4 < 4; i4++ ) {
 #pragma unroll
-      for ( int i = 0; i < 4; i++ ) {
-        o.hv[i] = __float2half_rn( acc[qt][i][v] * inv );
+      for ( int a = 0; a < 4; a++ ) {
+        union
+        {
+          uint2 raw;
+          __half hv[4];
+        } o;
+#pragma unroll
+        for ( int e = 0; e < 4; e++ ) {
+          o.hv[e] = __float2half_rn( acc[qt][i4][4 * a + e] * inv );
+        }
+        *reinterpret_cast<uint2*>( out + 32 * i4 + 8 * a + 4 * g2 ) = o.raw;
       }
-      *reinterpret_cast<uint2*>( out + d0 ) = o.raw;
     }
   }
 }
@@ -352,9 +403,10 @@ void launch_prefill_tiles( hipStream_t st, const void* q, const void* const* row
                            const gh_shape* s )
 {
   const uint32_t col_blocks = (uint32_t)( ( (uint64_t)n_tokens * G + 128 * NQT - 1 ) / ( 128 * NQT ) );
-  const uint64_t blocks = batch * s->n_kv_heads * col_blocks;
+  const uint64_t n_pairs = batch * s->n_kv_heads;
+  const uint64_t blocks = ( n_pairs + 7 ) / 8 * 8 * col_blocks;
   attn_prefill_mfma_kernel<G, NQT><<<(unsigned)blocks, 256, 0, st>>>( static_cast<const __half*>( q ), reinterpret_cast<const __half* const*>( rows ), start,
-                                                                     static_cast<__half*>( xb ), s->n_kv_heads, n_tokens, col_blocks,
+                                                                     static_cast<__half*>( xb ), s->n_kv_heads, n_tokens, col_blocks, (uint32_t)n_pairs,
                                                                      LOG2E / sqrtf( (float)s->head_size ) );
 }
 
