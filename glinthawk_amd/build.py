@@ -8,6 +8,7 @@ import glob
 import os
 import subprocess
 import sys
+from concurrent.futures import ThreadPoolExecutor
 
 PKG = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(PKG)
@@ -36,9 +37,16 @@ def _run(cmd: list[str]) -> None:
 
 
 def build_kernels() -> str:
+    """Every .hip source to an object file (in parallel), then one shared library."""
     os.makedirs(LIB_DIR, exist_ok=True)
+    obj_dir = os.path.join(PKG, "build")
+    os.makedirs(obj_dir, exist_ok=True)
     sources = sorted(glob.glob(os.path.join(CSRC, "*.hip")))
-    _run([HIPCC, *DEVICE_FLAGS, *COMMON_FLAGS, "-std=c++17", "-shared", "-o", LIB, *sources])
+    jobs = max(1, min(len(sources), int(os.environ.get("MAX_JOBS", "0")) or os.cpu_count() or 1, 16))
+    objects = [os.path.join(obj_dir, os.path.splitext(os.path.basename(src))[0] + ".o") for src in sources]
+    with ThreadPoolExecutor(max_workers=jobs) as pool:
+        list(pool.map(lambda so: _run([HIPCC, *DEVICE_FLAGS, *COMMON_FLAGS, "-std=c++17", "-c", so[0], "-o", so[1]]), zip(sources, objects)))
+    _run([HIPCC, "--offload-arch=gfx950", "-fPIC", "-shared", "-o", LIB, *objects])
     return LIB
 
 
