@@ -61,6 +61,17 @@ def build_host() -> str | None:
     return HOST_LIB
 
 
+def build_host_sanitized() -> str:
+    """The host layer with AddressSanitizer and UndefinedBehaviorSanitizer (host code only; GPU sanitizers are not used), for the
+    CPU test suite: tests/test_sanitizers.py loads it through GLINT_HOST_LIB with the sanitizer runtime preloaded."""
+    sources = sorted(glob.glob(os.path.join(HOST, "*.cc")))
+    out = os.path.join(LIB_DIR, "libglint_host_san.so")
+    _run([HIPCC, *COMMON_FLAGS[1:], "-O1", "-g", "-fno-omit-frame-pointer", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined",
+          "-shared-libasan", "-std=c++20", "-x", "c++", "-I" + HOST, "-shared", "-o", out, *sources,
+          "-L" + LIB_DIR, "-lglint_hip", "-Wl,-rpath,$ORIGIN", "-pthread"])
+    return out
+
+
 def build_tools() -> list[str]:
     """profile-stage-hip and profile-gemm-hip: the reference's profiling front ends for this target."""
     built = []

@@ -234,6 +234,9 @@ class BatchedInferenceState
   // rows [first, first + n) of `from` become rows [at, at + n) of this state's buffers
   void copy_rows( size_t at, const BatchedInferenceState& from, size_t first, size_t n )
   {
+    if ( n == 0 ) {
+      return; // nothing to move; an empty buffer's null pointer must not reach memcpy
+    }
     if ( metadata_.has_activations ) {
       std::memcpy( activations_.data() + at * activation_len(), from.activations_.data() + first * activation_len(), n * activation_len() );
     }
@@ -338,11 +341,15 @@ public:
     s.metadata_ = m;
     s.prompts_.resize( m.batch_size );
     const char* p = bytes.data() + sizeof( m );
-    std::memcpy( reinterpret_cast<char*>( s.prompts_.data() ), p, sizeof( PromptData ) * (size_t)m.batch_size );
+    if ( m.batch_size > 0 ) { // an empty vector has no storage: a null pointer must not reach memcpy, even with a length of zero
+      std::memcpy( reinterpret_cast<char*>( s.prompts_.data() ), p, sizeof( PromptData ) * (size_t)m.batch_size );
+    }
     p += sizeof( PromptData ) * (size_t)m.batch_size;
     auto take = [&]( DataBuffer& buf, size_t n ) {
       buf = DataBuffer( n );
-      std::memcpy( buf.data(), p, n );
+      if ( n > 0 ) {
+        std::memcpy( buf.data(), p, n );
+      }
       p += n;
     };
     if ( m.has_activations ) {

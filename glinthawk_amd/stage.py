@@ -12,7 +12,8 @@ import numpy as np
 from ._lib import GlintError
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
-_HOST_LIB_PATH = os.path.join(_PKG, "lib", "libglint_host.so")
+# GLINT_HOST_LIB: another build of the same sources (the sanitizer build of the CPU test suite)
+_HOST_LIB_PATH = os.environ.get("GLINT_HOST_LIB") or os.path.join(_PKG, "lib", "libglint_host.so")
 
 STAGE_PRE, STAGE_ATT, STAGE_POST, STAGE_CLS = 0, 1, 2, 3
 FWD_ALL, FWD_PRE, FWD_ATT, FWD_POST, FWD_CLS = 0, 1, 2, 3, 4

@@ -20,7 +20,8 @@ from typing import Optional, Sequence
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_LIB_PATH = os.path.join(_HERE, "libglint_oracle.so")
+# GLINT_ORACLE_LIB: another build of the same source (the sanitizer build of the CPU test suite)
+_LIB_PATH = os.environ.get("GLINT_ORACLE_LIB") or os.path.join(_HERE, "libglint_oracle.so")
 
 
 def build(force: bool = False) -> str:
