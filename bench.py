@@ -43,8 +43,17 @@ MFMA_PEAK_TFLOPS = 2500.0
 # The summary of that measurement names the kernel source it was taken on by its SHA-256; the figure is
 # reported only while that source is unchanged, otherwise `traffic` is null.
 TRAFFIC_PROFILE = {
-    "llama2-70b-gqa-b64-ctx4096": ("profiles/attn_decode_mfma_llama2-70b-gqa-b64-ctx4096_hbm_counters.md", "glinthawk_amd/csrc/gh_attn_decode.hip"),
+    "llama2-70b-gqa-b64-ctx4096": ("profiles/attn_decode_mfma_llama2-70b-gqa-b64-ctx4096_hbm_counters.md",
+                                   ("glinthawk_amd/csrc/gh_attn_decode.hip", "glinthawk_amd/csrc/gh_attn_tiles.h")),
 }
+
+
+def kernel_source_digest(sources):
+    """sha256 over the kernel's source files, in the order given."""
+    h = hashlib.sha256()
+    for p in sources:
+        h.update(open(os.path.join(ROOT, p), "rb").read())
+    return h.hexdigest()
 
 # the decode configurations that fit one GPU as a single stage (the first is the headline)
 WORKLOADS = {
@@ -101,10 +110,11 @@ def measured_traffic(workload):
     the kernel source as it is now."""
     if workload not in TRAFFIC_PROFILE:
         return None, "no counter profile for this workload"
-    summary, source = (os.path.join(ROOT, p) for p in TRAFFIC_PROFILE[workload])
+    summary, sources = TRAFFIC_PROFILE[workload]
+    summary = os.path.join(ROOT, summary)
     try:
         text = open(summary).read()
-        digest = hashlib.sha256(open(source, "rb").read()).hexdigest()
+        digest = kernel_source_digest(sources)
     except OSError:
         return None, "counter profile summary not present"
     m_bytes = re.search(r"traffic_bytes_per_launch:\s*(\d+)", text)

@@ -612,3 +612,37 @@ def test_fused_rejects_bad_arguments():
             ops.attn_decode(q, rows, pos, xb, 500, shape, workspace=torch.empty(64, dtype=torch.uint8, device="cuda"))
         finally:
             ops.attn_set_chunk(0)
+
+
+# ------------------------------------------------------------------ paged arena, straight through the C-ABI
+def test_vmm_commit_out_of_range_is_refused():
+    """VirtualMemoryRegion::allocate_span refuses a span outside the reservation ("Out of bounds allocation",
+    arch/amd64/common/vmem.hh:67-69); the C-ABI reports it as GH_ERR_INVALID and leaves the region as it was."""
+    import ctypes as C
+    from glinthawk_amd import _lib
+    L = _lib.lib()
+    gran = C.c_uint64(0)
+    _lib.check(L.gh_vmm_granularity(C.byref(gran)))
+    g = gran.value
+    assert g > 0 and g & (g - 1) == 0
+    region = C.c_void_p()
+    _lib.check(L.gh_vmm_reserve(C.byref(region), 4 * g))
+    assert L.gh_vmm_max_len(region) == 4 * g and L.gh_vmm_ptr(region)
+    assert L.gh_vmm_commit(region, g, g) == 0                         # inside: fine
+    assert L.gh_vmm_committed_bytes(region) == g
+    for off, length in ((4 * g, g), (3 * g, 2 * g), (0, 5 * g), (1 << 60, g)):
+        assert L.gh_vmm_commit(region, off, length) == -1, (off, length)      # GH_ERR_INVALID
+        assert b"outside" in L.gh_last_error()
+    assert L.gh_vmm_commit(region, 0, 0) == -1                        # empty span
+    assert L.gh_vmm_commit(region, g // 2, g) == -1 and b"granularity" in L.gh_last_error()
+    assert L.gh_vmm_commit(None, 0, g) == -1
+    assert L.gh_vmm_committed_bytes(region) == g                      # nothing of the refused spans was mapped
+    # the committed block is ordinary device memory
+    t = torch.arange(1024, dtype=torch.int32, device="cuda")
+    _lib.check(L.gh_memcpy(L.gh_vmm_ptr(region) + g, t.data_ptr(), 4096, _lib.GH_D2D, 0, None))
+    back = torch.zeros_like(t)
+    _lib.check(L.gh_memcpy(back.data_ptr(), L.gh_vmm_ptr(region) + g, 4096, _lib.GH_D2D, 0, None))
+    assert torch.equal(back, t)
+    _lib.check(L.gh_vmm_clear(region))
+    assert L.gh_vmm_committed_bytes(region) == 0
+    _lib.check(L.gh_vmm_free(region))
