@@ -68,10 +68,10 @@ __global__ __launch_bounds__( 256 ) void expand_tables_kernel( const void* const
 // q, xb: (batch * n_tokens, n_kv_heads * G * 128), row index = context * n_tokens + token.
 // Query column c of a (context, kv head): token c / G, query head c % G (the G heads that share the kv head).
 //
-// block = 4 waves = 256 query columns; wave = 64 columns = two 32-column MFMA tiles.  Per 64-key stage (K and V rows in LDS,
-// the next stage's rows in flight in registers):
+// block = 4 waves; wave = NQT 32-column MFMA tiles (NQT = 1 by default: 128 query columns per block, two blocks per CU).  Per
+// 64-key stage (K and V rows go from global memory straight into LDS, two buffers each, see the loop below):
 //   S^T = K Q^T   v_mfma_f32_32x32x16_f16, A = K rows out of LDS (16-byte chunks, XOR-swizzled), B = Q^T in registers; every A
-//                 fragment feeds both column tiles.  A lane ends up with 16 of the 32 keys of a sub-tile for ITS query column,
+//                 fragment feeds all column tiles.  A lane ends up with 16 of the 32 keys of a sub-tile for ITS query column,
 //                 the lane 32 further on with the other 16: maximum and sum stay inside a lane but for one exchange per stage
 //   O^T += V^T P^T  the scores of a lane are, as they lie, the B operand (keys x its column) of the same instruction; the A
 //                 operand V^T (one dim x 8 keys per lane) comes out of LDS with transposing reads (ds_read_b64_tr_b16).  Every
@@ -125,7 +125,7 @@ __global__ __launch_bounds__( 256, NQT == 1 ? 2 : 1 ) void attn_prefill_mfma_ker
   const uint32_t t_all = start + wave_tok0 + 1;                 // keys [0, t_all) are visible to every column of the wave
   const uint32_t wg_end = start + min( n_tokens, ( cb + 1 ) * 4 * TPW );
 
-  // this lane's two query columns (tile 0 and tile 1): token, head, last visible key
+  // this lane's query column in each of the wave's tiles: token, head, last visible key
   uint32_t tq[NQT], gq[NQT];
   int32_t qpos[NQT];
   f16x8 qb[NQT][8];
