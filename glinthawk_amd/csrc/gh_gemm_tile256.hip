@@ -38,7 +38,14 @@
 //                 its time, LDS reads take 4 cycles per instruction without conflicts).  Tried and
 //                 not kept: a third stage for the activations (their loads two steps ahead, -6..+7 %),
 //                 that plus the weights two steps ahead through registers (-5..+3 %), five 32-k
-//                 stages as a ring (two barriers per 64 k: -5..-15 %), non-temporal loads (-10 %).
+//                 stages as a ring (two barriers per 64 k: -5..-15 %), non-temporal loads (-10 %), the
+//                 barrier in front of the last MFMA group of a step with the next stage's first
+//                 fragments requested right behind it, so that the waves leave the barrier with matrix
+//                 work in hand (256 rows -5..-8 %, 384 rows +-1 %).
+//   clock       the graphics clock counter (GRBM_GUI_ACTIVE over the kernel's duration) reads 1.69-1.80 GHz
+//                 while this kernel runs and 2.3-2.4 GHz in the bandwidth-bound decode kernels: under
+//                 sustained matrix load the part lowers its clock, so at 70-78 % matrix-pipe use the
+//                 kernel delivers 1.2-1.3 PFLOP/s, and 100 % at that clock would be 1.77, not 2.5.
 //   tile order  as in the 128 x 128 kernel: each XCD owns every 8th row tile and walks patches of
 //                 tiles that are resident together.  The row tiles beyond a multiple of 8 are cut
 //                 into 8 equal runs of tiles instead, so that every XCD gets the same number of
