@@ -25,7 +25,9 @@ bool gemm_stream_gate_applicable( uint64_t s, uint64_t hidden, uint64_t b, const
 int gemm_stream_gate_launch( __half* hb, const __half* x, const __half* w13, uint64_t s, uint64_t hidden, uint64_t b, hipStream_t st );
 // 256 x 256 tile kernel for products with enough tiles (gh_gemm_tile256.hip)
 bool gemm_tile256_applicable( uint64_t s, uint64_t r, uint64_t b, const void* x, const void* w, const void* xout );
-int gemm_tile256_launch( __half* xout, float* partial, const __half* x, const __half* w, uint64_t s, uint64_t r, uint64_t b, int epilogue, hipStream_t st );
+int gemm_tile256_launch( __half* xout, float* partial, const __half* x, const __half* w, uint64_t s, uint64_t r, uint64_t b, int epilogue, hipStream_t st,
+                         uint32_t splits, uint32_t k_len );
+void gemm_tile256_split_plan( uint64_t s, uint64_t r, uint64_t b, const void* x, const void* w, uint32_t* splits, uint32_t* k_len );
 void gemm_tile256_tuning( int rows );
 // large-batch (prefill) kernel (gh_gemm_tile.hip)
 bool gemm_tile_applicable( uint64_t s, uint64_t r, uint64_t b, const void* x, const void* w, const void* xout );
@@ -255,7 +257,7 @@ int gemm_tile_epilogue_launch( void* xout, const void* x, const void* w, uint64_
     return GH_OK;
   }
   *done = true;
-  return gemm_tile256_launch( static_cast<__half*>( xout ), nullptr, static_cast<const __half*>( x ), static_cast<const __half*>( w ), s, r, b, epilogue, st );
+  return gemm_tile256_launch( static_cast<__half*>( xout ), nullptr, static_cast<const __half*>( x ), static_cast<const __half*>( w ), s, r, b, epilogue, st, 1, 0 );
 }
 
 int gemm_partials( void* xout, const void* x, const void* w, uint64_t s, uint64_t r, uint64_t b, gh_dtype dt, hipStream_t st, bool want_partials,
@@ -289,7 +291,20 @@ int gemm_partials( void* xout, const void* x, const void* w, uint64_t s, uint64_
       *partial_out = ws;
       *splits_out = 1;
     }
-    return gemm_tile256_launch( static_cast<__half*>( xout ), ws, static_cast<const __half*>( x ), static_cast<const __half*>( w ), s, r, b, 0, st );
+    return gemm_tile256_launch( static_cast<__half*>( xout ), ws, static_cast<const __half*>( x ), static_cast<const __half*>( w ), s, r, b, 0, st, 1, 0 );
+  }
+  if ( g_force_kernel == 0 || g_force_kernel == 4 ) { // some hundred rows and few tiles: the same kernel with the K range split
+    uint32_t splits = 0, k_len = 0;
+    gemm_tile256_split_plan( s, r, b, x, w, &splits, &k_len );
+    if ( splits > 1 ) {
+      float* ws = nullptr;
+      if ( int rc = ensure_workspace( (uint64_t)splits * b * r * sizeof( float ), &ws, st ) ) {
+        return rc;
+      }
+      *partial_out = ws;
+      *splits_out = splits;
+      return gemm_tile256_launch( nullptr, ws, static_cast<const __half*>( x ), static_cast<const __half*>( w ), s, r, b, 0, st, splits, k_len );
+    }
   }
   GH_REQUIRE( g_force_kernel != 4, "gh_matmul: the 256 x 256 tile kernel needs b >= 192, at least 192 tiles with a last round that is not mostly empty, s %% 64 == 0 and 16-byte aligned operands" );
   if ( ( g_force_kernel == 0 || g_force_kernel == 3 ) && gemm_tile_applicable( s, r, b, x, w, xout ? xout : x ) ) {

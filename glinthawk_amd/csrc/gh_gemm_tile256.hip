@@ -87,7 +87,8 @@ constexpr int T256_THREADS = 512;
 // divisions and exponentials, and the separate element-wise kernel is faster.)
 constexpr int EPI_STORE = 0, EPI_ACCUM = 1, EPI_PARTIAL = 3;
 
-// grid: 8 x (padded tiles of one XCD).  s % 64 == 0, 16-byte aligned operands.
+// grid: 8 x (padded tiles of one XCD) by K splits (more than one only with EPI_PARTIAL: split z leaves its sums in
+// partial[z]).  s % 64 == 0, k_len % 64 == 0, 16-byte aligned operands.
 // NA: 32-row accumulator tiles per wave, 2 (256 weight rows per work-group) or 3 (384).
 template<int EPI, int NA>
 __global__ __launch_bounds__( T256_THREADS, 1 ) void gemm_tile256_kernel( __half* __restrict__ xout,
@@ -97,6 +98,7 @@ __global__ __launch_bounds__( T256_THREADS, 1 ) void gemm_tile256_kernel( __half
                                                                         uint32_t s,
                                                                         uint32_t r,
                                                                         uint32_t b,
+                                                                        uint32_t k_len, // k per split
                                                                         TileOrder ord )
 {
   // Four separate arrays, not [2][...]: the compiler orders an LDS read behind an outstanding
@@ -137,8 +139,11 @@ __global__ __launch_bounds__( T256_THREADS, 1 ) void gemm_tile256_kernel( __half
   const uint32_t ld_bytes = s * 2;
   const uint32_t w_rows = min( (uint32_t)TM, r - tile_row0 );
   const uint32_t x_cols = min( (uint32_t)TN2, b - tile_col0 );
-  const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc( const_cast<__half*>( w + (uint64_t)tile_row0 * s ), 0, (int)( w_rows * ld_bytes ), 0x00020000 );
-  const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc( const_cast<__half*>( x + (uint64_t)tile_col0 * s ), 0, (int)( x_cols * ld_bytes ), 0x00020000 );
+  const uint32_t k0 = blockIdx.y * k_len; // this split's k range starts here; the descriptors start there too and end with the tile's last row
+  const __amdgpu_buffer_rsrc_t w_rsrc
+    = __builtin_amdgcn_make_buffer_rsrc( const_cast<__half*>( w + (uint64_t)tile_row0 * s + k0 ), 0, (int)( w_rows * ld_bytes - k0 * 2 ), 0x00020000 );
+  const __amdgpu_buffer_rsrc_t x_rsrc
+    = __builtin_amdgcn_make_buffer_rsrc( const_cast<__half*>( x + (uint64_t)tile_col0 * s + k0 ), 0, (int)( x_cols * ld_bytes - k0 * 2 ), 0x00020000 );
   // A load-to-LDS writes lane l of a wave to (wave's base) + 16 l: thread t fills slot t % 8 of row
   // t / 8 (+ 64 i), so it fetches the chunk that the swizzle keeps in that slot.
   const uint32_t voff = ( threadIdx.x >> 3 ) * ld_bytes + ( ( threadIdx.x & 7 ) ^ ( ( threadIdx.x >> 4 ) & 7 ) ) * 16;
@@ -155,7 +160,7 @@ __global__ __launch_bounds__( T256_THREADS, 1 ) void gemm_tile256_kernel( __half
       }
     }
   }
-  const uint32_t n_steps = s / TKS;
+  const uint32_t n_steps = min( k_len, s - k0 ) / TKS;
   const uint32_t fr = lane & 31, g2 = lane >> 5;
   // global -> LDS stage, 1 KiB per wave and instruction: loads [from, to) of the list W0 X0 W1 X1 W2 X2 W3 X3 (W4 W5)
   constexpr int N_LOADS = 2 * NA + 4;
@@ -361,7 +366,7 @@ __global__ __launch_bounds__( T256_THREADS, 1 ) void gemm_tile256_kernel( __half
         const uint32_t row = tile_row0 + 32 * NA * wr + 32 * rt + 8 * q4 + 4 * g2;
         const bool whole = row + 3 < r && ( r & 3 ) == 0;
         if ( PARTIAL ) {
-          float* dst = partial + (uint64_t)col * r + row;
+          float* dst = partial + ( (uint64_t)blockIdx.y * b + col ) * r + row;
           if ( whole ) {
             *reinterpret_cast<float4*>( dst ) = make_float4( acc[rt][t][4 * q4], acc[rt][t][4 * q4 + 1], acc[rt][t][4 * q4 + 2], acc[rt][t][4 * q4 + 3] );
           } else {
@@ -438,11 +443,44 @@ bool gemm_tile256_applicable( uint64_t s, uint64_t r, uint64_t b, const void* x,
          && ( ( reinterpret_cast<uintptr_t>( x ) | reinterpret_cast<uintptr_t>( w ) | reinterpret_cast<uintptr_t>( xout ) ) & 15u ) == 0;
 }
 
-// `partial` != nullptr: fp32 sums (1, b, r) instead of xout; else `epilogue` 0 stores, 1 accumulates into xout (needs r % 8 == 0)
-int gemm_tile256_launch( __half* xout, float* partial, const __half* x, const __half* w, uint64_t s, uint64_t r, uint64_t b, int epilogue, hipStream_t st )
+// Few tiles (a decode step of some hundred rows, or a narrow product): the K range is split over several work-groups per tile so
+// that the chip is full in one round, and the fp32 sums of each split go to partial[split].  *splits = 0: not for this shape.
+void gemm_tile256_split_plan( uint64_t s, uint64_t r, uint64_t b, const void* x, const void* w, uint32_t* splits, uint32_t* k_len )
+{
+  *splits = 0;
+  *k_len = 0;
+  const uint64_t tiles = ( ( r + TM2 - 1 ) / TM2 ) * ( ( b + TN2 - 1 ) / TN2 );
+  const uint64_t cus = (uint64_t)cu_count();
+  if ( b < 192 || tiles * 2 > cus || s % TKS != 0 || s >= ( 1u << 22 ) || ( ( reinterpret_cast<uintptr_t>( x ) | reinterpret_cast<uintptr_t>( w ) ) & 15u ) != 0 ) {
+    return;
+  }
+  const uint64_t steps = s / TKS;
+  // Very few tiles and a short K (70B wo at 256 rows: 32 tiles, 8 splits of 16 steps, fp32 sums half the size of the weights):
+  // the 128 x 128 kernel with two work-groups per CU hides more of such a short work-group's start-up (60 against 73 us).
+  if ( tiles * 8 <= cus && steps <= 128 ) {
+    return;
+  }
+  uint64_t n = std::min<uint64_t>( cus / tiles, steps / 16 ); // at least 16 steps of 64 k per split
+  if ( n < 2 ) {
+    return;
+  }
+  const uint64_t steps_per_split = ( steps + n - 1 ) / n;
+  *k_len = (uint32_t)( steps_per_split * TKS );
+  *splits = (uint32_t)( ( steps + steps_per_split - 1 ) / steps_per_split );
+}
+
+// `partial` != nullptr: fp32 sums (splits, b, r) instead of xout; else `epilogue` 0 stores, 1 accumulates into xout (needs r % 8 == 0).
+// splits > 1 (from gemm_tile256_split_plan, with its k_len) needs `partial`.
+int gemm_tile256_launch( __half* xout, float* partial, const __half* x, const __half* w, uint64_t s, uint64_t r, uint64_t b, int epilogue, hipStream_t st,
+                         uint32_t splits, uint32_t k_len )
 {
   TileOrder ord;
-  const uint32_t tile_rows = tile256_rows( s, r, b );
+  GH_REQUIRE( splits >= 1 && ( splits == 1 || ( partial != nullptr && k_len % TKS == 0 && (uint64_t)k_len * splits >= s && (uint64_t)k_len * ( splits - 1 ) < s ) ),
+              "gh_matmul: bad K split for the 256-token tile kernel" );
+  if ( splits == 1 ) {
+    k_len = (uint32_t)s;
+  }
+  const uint32_t tile_rows = splits > 1 ? 256 : tile256_rows( s, r, b );
   ord.row_tiles = (uint32_t)( ( r + tile_rows - 1 ) / tile_rows );
   ord.token_tiles = (uint32_t)( ( b + TN2 - 1 ) / TN2 );
   ord.gn = std::min<uint32_t>( ord.token_tiles, 8 );
@@ -457,12 +495,12 @@ int gemm_tile256_launch( __half* xout, float* partial, const __half* x, const __
   GH_REQUIRE( gx < ( 1ull << 31 ), "gh_matmul: grid too large" );
   ord.main_per_xcd = (uint32_t)main_per_xcd;
   ord.rest_share = (uint32_t)rest_share;
-  const dim3 grid( (unsigned)gx ), block( T256_THREADS );
+  const dim3 grid( (unsigned)gx, splits ), block( T256_THREADS );
   const uint32_t s32 = (uint32_t)s, r32 = (uint32_t)r, b32 = (uint32_t)b;
   const int epi = partial != nullptr ? EPI_PARTIAL : epilogue;
   GH_REQUIRE( epi == EPI_STORE || epi == EPI_ACCUM || epi == EPI_PARTIAL, "gh_matmul: unknown tile epilogue %d", epi );
   GH_REQUIRE( epi != EPI_ACCUM || r % 8 == 0, "gh_matmul: the accumulating tile epilogue needs r %% 8 == 0" );
-#define GH_TILE256_LAUNCH( E, N ) gemm_tile256_kernel<E, N><<<grid, block, 0, st>>>( xout, partial, x, w, s32, r32, b32, ord )
+#define GH_TILE256_LAUNCH( E, N ) gemm_tile256_kernel<E, N><<<grid, block, 0, st>>>( xout, partial, x, w, s32, r32, b32, k_len, ord )
 #define GH_TILE256_ROWS( E ) ( tile_rows == 384 ? GH_TILE256_LAUNCH( E, 3 ) : GH_TILE256_LAUNCH( E, 2 ) )
   switch ( epi ) {
     case EPI_STORE: GH_TILE256_ROWS( EPI_STORE ); break;

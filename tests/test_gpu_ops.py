@@ -253,6 +253,26 @@ def test_matmul_streaming_kernel_sweep(b, s, r):
     assert err.max().item() < 2e-2 and (err.mean() / want.abs().mean()).item() < 1e-3
 
 
+# some hundred rows (the decode step of a large slot arena): whatever the dispatcher picks at each batch size (streaming kernel up
+# to 64 rows, 128 x 128 tiles with or without a K split, 256-token tiles with the K range split over work-groups when the tiles are
+# few), ragged edges in rows, tokens and K steps.  One-hot activations: every output is one weight, bit for bit.
+@pytest.mark.parametrize("b", [65, 128, 192, 256, 300, 512])
+@pytest.mark.parametrize("s,r", [(2048, 1024), (2112, 1000), (8192, 2560), (4096, 516)])
+def test_matmul_some_hundred_rows(b, s, r):
+    g = torch.Generator(device="cuda").manual_seed(b * 13 + r)
+    w = (torch.randn((r, s), generator=g, device="cuda") / s ** 0.5).half()
+    hot = torch.zeros((b, s), dtype=torch.float16, device="cuda")
+    cols = torch.tensor([(7919 * i + 3) % s for i in range(b)], device="cuda")
+    hot[torch.arange(b, device="cuda"), cols] = 1
+    x = torch.randn((b, s), generator=g, device="cuda").half()
+    got_hot = ops.matmul(hot, w)
+    got = ops.matmul(x, w)
+    assert torch.equal(got_hot, w[:, cols].t().contiguous())
+    want = x.float() @ w.float().t()
+    err = (got.float() - want).abs()
+    assert err.max().item() < 2e-2 and (err.mean() / want.abs().mean()).item() < 1e-3
+
+
 def test_matmul_layout_one_hot():
     s, r = 256, 192
     w = torch.arange(r * s, dtype=torch.float32).reshape(r, s).remainder(1000).half().cuda()
