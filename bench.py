@@ -457,6 +457,7 @@ def churn_bench(steps, warmup, cpu=True):
     start_pos = rng.integers(16, 4096, slots)
     pos = start_pos.copy()
     ids = [1000 + i for i in range(slots)]
+    ones = np.ones(slots, np.uint32)
     st.new_state(slots, next_layer=first)
     for i in range(slots):
         st.set_prompt(i, ids[i], 1, int(pos[i]))
@@ -479,8 +480,7 @@ def churn_bench(steps, warmup, cpu=True):
         nonlocal decoded, prefilled, restarts, keys_read, t_decode, t_prefill
         t0 = time.perf_counter()
         st.new_state(slots, next_layer=first)
-        for i in range(slots):
-            st.set_prompt(i, ids[i], 1, int(pos[i]))
+        st.set_prompts(ids, ones, pos)
         st.activations(allocate=True)[:] = acts.reshape(-1)
         assert st.forward()
         t1 = time.perf_counter()

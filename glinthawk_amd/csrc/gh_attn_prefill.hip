@@ -15,10 +15,8 @@ namespace {
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr float LAZY = 8.0f; // see the softmax step of the tiled prefill kernel
 constexpr int HS = 128;
-#ifndef PF_WGS_PER_CU
-#define PF_WGS_PER_CU 1
-#endif
 
+typedef _Float16 f16x2 __attribute__( ( ext_vector_type( 2 ) ) );
 typedef _Float16 f16x4 __attribute__( ( ext_vector_type( 4 ) ) );
 typedef _Float16 f16x8 __attribute__( ( ext_vector_type( 8 ) ) );
 typedef float f32x4 __attribute__( ( ext_vector_type( 4 ) ) );
@@ -77,6 +75,9 @@ __global__ __launch_bounds__( 256 ) void expand_tables_kernel( const void* const
 //                 operand V^T (one dim x 8 keys per lane) comes out of LDS with transposing reads (ds_read_b64_tr_b16).  Every
 //                 accumulator of a lane belongs to its own column: rescaling needs no shuffle
 // Causal mask only on stages that reach a wave's diagonal; stages beyond it are skipped.
+// A wave's stage: softmax of the stage's scores (vector ALU), then 16 pairs of (one MFMA of O^T += V^T P^T, one MFMA of the NEXT
+// stage's S^T), their LDS operands requested four pairs ahead and the second half of the exponentials computed beside the first pairs.
+// (Two tiles per wave, NQT = 2, is kept for measurement: it does not fit the registers of two work-groups per CU and runs at half the rate.)
 template<int G, int NQT>
 __global__ __launch_bounds__( 256, NQT == 1 ? 2 : 1 ) void attn_prefill_mfma_kernel( const __half* __restrict__ q,
                                                                    const __half* const* __restrict__ layer_rows,
@@ -86,10 +87,15 @@ __global__ __launch_bounds__( 256, NQT == 1 ? 2 : 1 ) void attn_prefill_mfma_ker
                                                                    uint32_t n_tokens,
                                                                    uint32_t col_blocks, // ceil(n_tokens * G / (128 * NQT))
                                                                    uint32_t n_pairs,    // batch * n_kv_heads
+                                                                   uint32_t paired,     // a work-group takes two column blocks (else one)
                                                                    float scale_log2e )
 {
-  __shared__ uint4 s_kt[2][64 * 16]; // two stages of 64 keys x 256 bytes, 16-byte chunks XOR-swizzled by the key's low bits
-  __shared__ uint4 s_vt[2][64 * 16]; // the same keys' value rows, plain
+  // Two stages of 64 keys x 256 bytes for K (16-byte chunks XOR-swizzled by the key's low bits) and two for the same keys' value
+  // rows.  Four separate arrays, and the loop below names the stage it works on at compile time: the compiler orders an LDS read
+  // behind the outstanding loads-to-LDS (a wait for ALL of them, the ones just issued included) whenever it cannot tell that they
+  // go to a different array.
+  __shared__ uint4 s_k0[64 * 16], s_k1[64 * 16];
+  __shared__ uint4 s_v0[64 * 16], s_v1[64 * 16];
   static_assert( 32 * NQT >= G, "a wave holds whole tokens" );
   constexpr uint32_t TPW = 32 * NQT / G; // tokens per wave
 
@@ -97,13 +103,17 @@ __global__ __launch_bounds__( 256, NQT == 1 ? 2 : 1 ) void attn_prefill_mfma_ker
   const uint32_t lane = threadIdx.x & 63;
   const uint32_t r = lane & 31;
   const uint32_t g2 = lane >> 5;
-  // block -> (column block, kv head, context).  Work-groups go to the 8 XCDs in turn and every XCD has its own L2: all column
+  // block -> (two column blocks, kv head, context).  Work-groups go to the 8 XCDs in turn and every XCD has its own L2: all column
   // blocks of a (context, kv head) pair are given to one XCD, next to each other in time, so that the pair's K and V rows are
-  // fetched into one L2 once instead of into all eight.  The column blocks with the most keys come first.
+  // fetched into one L2 once instead of into all eight.  Column block c attends (c + 1) x 128 / G keys (plus the start position),
+  // so a work-group takes column block col_blocks - 1 - j and then column block j: every work-group of a launch has the same
+  // number of key stages, and no CU idles while another finishes a long column block.  (Not for small launches: `paired` = 0
+  // keeps one column block per work-group, longest first, so that there are enough work-groups to go round.)
   const uint32_t xcd = blockIdx.x & 7;
   const uint32_t slot = blockIdx.x >> 3;
-  const uint32_t cb = col_blocks - 1 - slot % col_blocks;
-  const uint32_t pair = ( slot / col_blocks ) * 8 + xcd;
+  const uint32_t half_blocks = paired ? ( col_blocks + 1 ) / 2 : col_blocks;
+  const uint32_t cb_first = col_blocks - 1 - slot % half_blocks, cb_second = paired ? slot % half_blocks : cb_first;
+  const uint32_t pair = ( slot / half_blocks ) * 8 + xcd;
   if ( pair >= n_pairs ) {
     return; // padding of the grid to a multiple of 8 pairs (whole work-group)
   }
@@ -118,6 +128,14 @@ __global__ __launch_bounds__( 256, NQT == 1 ? 2 : 1 ) void attn_prefill_mfma_ker
   const uint32_t v_off = n_kv_heads * HS;
   const uint32_t start = start_pos[ctx];
 
+  for ( uint32_t part = 0; part < 2; part++ ) {
+  const uint32_t cb = part == 0 ? cb_first : cb_second;
+  if ( part == 1 ) {
+    if ( cb_second == cb_first ) {
+      break; // odd number of column blocks: the middle one is alone
+    }
+    __syncthreads(); // every wave is done with the LDS stages of the first column block
+  }
   const uint32_t wave_tok0 = ( cb * 4 + wave ) * TPW;          // first token of the wave
   const bool wave_ok = wave_tok0 < n_tokens;                    // a wave without queries still loads its share of every stage
   const uint32_t wave_last = min( n_tokens, wave_tok0 + TPW ) - 1;
@@ -176,97 +194,117 @@ __global__ __launch_bounds__( 256, NQT == 1 ? 2 : 1 ) void attn_prefill_mfma_ker
   const __amdgpu_buffer_rsrc_t kv_rsrc = __builtin_amdgcn_make_buffer_rsrc( const_cast<__half*>( base + (uint64_t)h * HS ), 0, (int)( wg_end * row_bytes ), 0x00020000 );
   const uint32_t ld_g = lane >> 4, ld_pos = lane & 15;
   const uint32_t k_voff = ld_g * row_bytes + ( ( ld_pos ^ ld_g ) * 16 ); // row 4 j + ld_g keeps chunk (ld_pos ^ ld_g ^ 4 j) in slot ld_pos
-  // V rows: the 32-byte pairs of a key's row are XORed with the key's low 3 bits, so that the transposing reads below (4 lanes per
-  // key and 32 bytes, 8 keys per instruction and half-wave) spread evenly over the banks: row 4 j + ld_g (low bits 4 (j & 1) + ld_g)
-  // keeps chunk ld_pos ^ 2 ld_g ^ 8 (j & 1) in slot ld_pos
-  const uint32_t v_voff = ld_g * row_bytes + ( ( ld_pos ^ ( 2 * ld_g ) ) * 16 ) + v_off * 2;
-  auto fetch_k = [&]( uint32_t buf, uint32_t stage ) {
+  // V rows: the 16-byte chunks of a key's row are XORed with 4 x the key's low 2 bits, so that the transposing reads below (a
+  // half-wave: 4 keys x 2 groups of 16 dims x 4 lanes x 8 bytes) touch 32 different 8-byte slots, i.e. every bank once: row
+  // 4 j + ld_g keeps chunk ld_pos ^ 4 ld_g in slot ld_pos.  (With 2 x the low 3 bits instead, lanes of the two dim groups met in
+  // the same banks at neighbouring keys: as many bank-conflict cycles as active LDS cycles.)
+  const uint32_t v_voff = ld_g * row_bytes + ( ( ld_pos ^ ( 4 * ld_g ) ) * 16 ) + v_off * 2;
+  auto fetch_k = [&]( uint4* kt, uint32_t stage ) {
 #pragma unroll
     for ( int j = 0; j < 4; j++ ) {
-      __builtin_amdgcn_raw_ptr_buffer_load_lds( kv_rsrc, (lds_ptr)( s_kt[buf] + ( 16 * wave + 4 * j ) * 16 ), 16, k_voff ^ ( 64 * j ),
+      __builtin_amdgcn_raw_ptr_buffer_load_lds( kv_rsrc, (lds_ptr)( kt + ( 16 * wave + 4 * j ) * 16 ), 16, k_voff ^ ( 64 * j ),
                                                 ( 64 * stage + 16 * wave + 4 * j ) * row_bytes, 0, 0 );
     }
   };
-  auto fetch_v = [&]( uint32_t buf, uint32_t stage ) {
+  auto fetch_v = [&]( uint4* vt, uint32_t stage ) {
 #pragma unroll
     for ( int j = 0; j < 4; j++ ) {
-      __builtin_amdgcn_raw_ptr_buffer_load_lds( kv_rsrc, (lds_ptr)( s_vt[buf] + ( 16 * wave + 4 * j ) * 16 ), 16, v_voff ^ ( 128 * ( j & 1 ) ),
+      __builtin_amdgcn_raw_ptr_buffer_load_lds( kv_rsrc, (lds_ptr)( vt + ( 16 * wave + 4 * j ) * 16 ), 16, v_voff,
                                                 ( 64 * stage + 16 * wave + 4 * j ) * row_bytes, 0, 0 );
     }
   };
 
   // transposing V reads: lane j = 4 e + q of a 16-lane group points at key slot e (0..3) of its half-wave, dims 16 grp + 4 q .. + 3
-  // of dim block 0; the chunk index carries the V tile's swizzle (2 x the key's low 3 bits = 8 g2 + 2 e), dim block i4 flips bits 2, 3
+  // of dim block 0; the chunk index carries the V tile's swizzle (4 x the key's low 2 bits = 4 e), dim block i4 flips bits 2, 3 as well
   const uint32_t tr_e = ( lane & 15 ) >> 2, tr_q = lane & 3, tr_grp = ( lane >> 4 ) & 1;
-  const uint32_t v_lane = ( 4 * g2 + tr_e ) * 256 + ( ( ( 2 * tr_grp + ( tr_q >> 1 ) ) ^ ( 8 * g2 + 2 * tr_e ) ) * 16 ) + ( tr_q & 1 ) * 8;
+  const uint32_t v_lane = ( 4 * g2 + tr_e ) * 256 + ( ( ( 2 * tr_grp + ( tr_q >> 1 ) ) ^ ( 4 * tr_e ) ) * 16 ) + ( tr_q & 1 ) * 8;
 
-  // scores of one stage: st[qt][sub][v] = raw score of key 32 sub + 8*(v/4) + 4*g2 + v%4 of the stage for column tile qt.  The two
-  // sub-tiles are independent accumulation chains that alternate in the matrix pipe; the K fragments of the next 16 dims are
-  // requested from LDS before the MFMAs of these
-  auto scores = [&]( f32x16 ( &st )[NQT][2], uint32_t buf ) {
+  // The two products of a stage run as 16 pairs of MFMA steps, pair n = (P-step n, S-step n):
+  //   P-step n  O^T += V^T P^T for keys 16 kk .. 16 kk + 15 (kk = n / 4) and dims 32 i4 .. 32 i4 + 31 (i4 = n % 4).  The A operand (32 dims x
+  //             16 keys; a lane: one dim, the 8 keys of its slots) comes out of LDS transposed: ds_read_b64_tr_b16 hands lane i of a
+  //             16-lane group element i of each of four 32-byte rows that the group's lanes point at (lanes 4 e .. 4 e + 3 at row e),
+  //             i.e. 4 keys of one dim per instruction.  The four dim blocks are independent accumulation chains.
+  //   S-step n  S^T = K Q^T of the NEXT stage for keys 32 sub .. 32 sub + 31 (sub = n / 8) and dims 16 s .. 16 s + 15 (s = n % 8):
+  //             st[qt][sub][v] = raw score of key 32 sub + 8*(v/4) + 4*g2 + v%4 of the stage for column tile qt.
+  // Operands sit in rings of four register sets: the LDS read for step n + 4 is issued right behind step n, i.e. four pairs (some 250
+  // cycles of matrix work) before its use; under this kernel's load an LDS read takes about 200 cycles to return, and with the reads one
+  // step ahead both products ran at the pace of that latency.
+  f16x8 ka[4];
+  auto read_k = [&]( const uint4* kt, int n ) {
+    const uint32_t krow = 32 * ( n >> 3 ) + r;
+    ka[n & 3] = __builtin_bit_cast( f16x8, kt[krow * 16 + ( ( 2 * ( n & 7 ) + g2 ) ^ ( krow & 15 ) )] );
+  };
+  auto score_step = [&]( f32x16 ( &st )[NQT][2], int n ) {
 #pragma unroll
     for ( int qt = 0; qt < NQT; qt++ ) {
-#pragma unroll
-      for ( int sub = 0; sub < 2; sub++ ) {
-#pragma unroll
-        for ( int v = 0; v < 16; v++ ) {
-          st[qt][sub][v] = 0.0f;
-        }
+      if ( ( n & 7 ) == 0 ) {
+        const f32x16 zero = { 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0 };
+        st[qt][n >> 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16( ka[n & 3], qb[qt][n & 7], zero, 0, 0, 0 );
+      } else {
+        st[qt][n >> 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16( ka[n & 3], qb[qt][n & 7], st[qt][n >> 3], 0, 0, 0 );
       }
     }
-    f16x8 ka[2][2];
-    auto read_k = [&]( int s ) {
+  };
+  v4s va[4][2];
+  auto read_v = [&]( const uint4* vt, int n ) {
 #pragma unroll
-      for ( int sub = 0; sub < 2; sub++ ) {
-        const uint32_t krow = 32 * sub + r;
-        ka[s & 1][sub] = __builtin_bit_cast( f16x8, s_kt[buf][krow * 16 + ( ( 2 * s + g2 ) ^ ( krow & 15 ) )] );
-      }
-    };
-    read_k( 0 );
-#pragma unroll
-    for ( int s = 0; s < 8; s++ ) {
-      if ( s + 1 < 8 ) {
-        read_k( s + 1 );
-      }
-#pragma unroll
-      for ( int sub = 0; sub < 2; sub++ ) {
-#pragma unroll
-        for ( int qt = 0; qt < NQT; qt++ ) {
-          st[qt][sub] = __builtin_amdgcn_mfma_f32_32x32x16_f16( ka[s & 1][sub], qb[qt][s], st[qt][sub], 0, 0, 0 );
-        }
-      }
+    for ( int half = 0; half < 2; half++ ) {
+      va[n & 3][half]
+        = __builtin_amdgcn_ds_read_tr16_b64_v4i16( (lds_v4s)( (lds_char*)vt + ( v_lane ^ ( 64 * ( n & 3 ) ) ) + ( 16 * ( n >> 2 ) + 8 * half ) * 256 ) );
     }
   };
 
   // Two LDS buffers each for K and V, one barrier per stage.  Behind the barrier of iteration i every wave is done with K of
   // stage i (its scores were computed in iteration i-1) and with V of stage i-1, so K of stage i+2 and V of stage i+1 are
   // requested into those buffers; the barrier of iteration i+1 waits for them.  The wave then turns the scores of stage i into
-  // weights (vector ALU), computes the scores of stage i+1 (matrix pipe, independent of the weights) and adds stage i's
-  // weighted values.
+  // weights and, pair by pair, adds stage i's weighted values and computes the scores of stage i+1 (which do not depend on the
+  // weights).
   const uint32_t n_stages = ( wg_end + 63 ) / 64;
   const uint32_t my_stages = ( t_end + 63 ) / 64; // stages that hold keys visible to this wave (it takes part in the loads and barriers of all)
-  fetch_k( 0, 0 );
-  fetch_k( 1, 1 );
-  fetch_v( 0, 0 );
+  fetch_k( s_k0, 0 );
+  fetch_k( s_k1, 1 );
+  fetch_v( s_v0, 0 );
+  __builtin_amdgcn_s_waitcnt( 0x0F70 ); // vmcnt(0)
   __syncthreads();
-  f32x16 st[NQT][2];
+  f32x16 st_a[NQT][2], st_b[NQT][2]; // scores of even and of odd stages
   if ( my_stages > 0 ) {
-    scores( st, 0 );
+#pragma unroll
+    for ( int n = 0; n < 4; n++ ) {
+      read_k( s_k0, n );
+    }
+#pragma unroll
+    for ( int n = 0; n < 16; n++ ) {
+      score_step( st_a, n );
+      if ( n + 4 < 16 ) {
+        read_k( s_k0, n + 4 );
+      }
+    }
   }
 
-  for ( uint32_t i = 0; i < n_stages; i++ ) {
+  // stage i with its K in k_cur and its V in v_cur, its scores in st; k_nxt, v_nxt, st_nxt: the other set
+  auto stage = [&]( uint32_t i, uint4* k_cur, uint4* v_cur, uint4* k_nxt, uint4* v_nxt, f32x16 ( &st )[NQT][2], f32x16 ( &st_nxt )[NQT][2] ) {
     const uint32_t t0 = 64 * i;
-    const uint32_t buf = i & 1;
+    // Every load-to-LDS this wave has issued (K of stage i + 1, V of stage i) has landed before the wave enters the barrier, so
+    // behind it all of them have.  Said explicitly: the barrier's own fence only orders LDS instructions, and the compiler's
+    // tracking of loads-to-LDS against the reads of the distinct arrays is not relied upon.
+    __builtin_amdgcn_s_waitcnt( 0x0F70 ); // vmcnt(0)
     __syncthreads();
     if ( i + 2 < n_stages ) {
-      fetch_k( buf, i + 2 );
+      fetch_k( k_cur, i + 2 );
     }
     if ( i + 1 < n_stages ) {
-      fetch_v( buf ^ 1, i + 1 );
+      fetch_v( v_nxt, i + 1 );
     }
     if ( i >= my_stages ) {
-      continue; // wave-uniform
+      return; // wave-uniform
     }
+    // the operands of the first four pairs are requested now: the softmax below gives them the time to arrive
+#pragma unroll
+    for ( int n = 0; n < 4; n++ ) {
+      read_v( v_cur, n );
+      read_k( k_nxt, n );
+    }
+    __builtin_amdgcn_sched_barrier( 0 );
     // a stage that reaches the wave's diagonal hides keys from some columns; before it every key is visible to every column
     if ( __builtin_amdgcn_readfirstlane( t0 + 64 > t_all ) ) {
       asm volatile( "" ::: "memory" ); // keeps this a branch: the selects are only paid for on the diagonal
@@ -283,8 +321,8 @@ __global__ __launch_bounds__( 256, NQT == 1 ? 2 : 1 ) void attn_prefill_mfma_ker
       }
     }
 
-    // ---- online softmax per column tile; p packed as B operands: pk[qt][2 sub + jj] = keys 32 sub + 16 jj + 8 (e/4) + 4 g2 + e%4, e = 0..7
-    f16x8 pk[NQT][4];
+    // ---- online softmax per column tile: the reference point first
+    float ms[NQT];
 #pragma unroll
     for ( int qt = 0; qt < NQT; qt++ ) {
       float mx = st[qt][0][0];
@@ -312,54 +350,50 @@ __global__ __launch_bounds__( 256, NQT == 1 ? 2 : 1 ) void attn_prefill_mfma_ker
           }
         }
       }
-      const float ms = m[qt] == -INFINITY ? 0.0f : m[qt];
-      float sum[2] = { 0.0f, 0.0f };
+      ms[qt] = m[qt] == -INFINITY ? 0.0f : m[qt];
+    }
+    // weights of keys 16 kk .. 16 kk + 15 of the stage, packed as the B operand of their P-steps:
+    // pk[qt][kk] = keys 32 (kk / 2) + 16 (kk % 2) + 8 (e / 4) + 4 g2 + e % 4, e = 0..7.  Elements e0, e0 + 1 at a time, so that the
+    // exponentials of 16 keys can be spread over four pairs.
+    f16x8 pk[NQT][4];
+    float p[NQT][8];
+    f16x2 pk2[NQT][4];
+    float sum[NQT][2];
 #pragma unroll
-      for ( int sub = 0; sub < 2; sub++ ) {
+    for ( int qt = 0; qt < NQT; qt++ ) {
+      sum[qt][0] = sum[qt][1] = 0.0f;
+    }
+    auto weights = [&]( int kk, int e0 ) {
 #pragma unroll
-        for ( int jj = 0; jj < 2; jj++ ) {
-          float p[8];
+      for ( int qt = 0; qt < NQT; qt++ ) {
 #pragma unroll
-          for ( int e = 0; e < 8; e++ ) {
-            p[e] = fast_exp2( st[qt][sub][8 * jj + e] * scale_log2e - ms );
-            sum[e & 1] += p[e];
-          }
-          pk[qt][2 * sub + jj] = f16x8 { (_Float16)p[0], (_Float16)p[1], (_Float16)p[2], (_Float16)p[3],
-                                         (_Float16)p[4], (_Float16)p[5], (_Float16)p[6], (_Float16)p[7] };
+        for ( int e = e0; e < e0 + 2; e++ ) {
+          p[qt][e] = fast_exp2( st[qt][kk >> 1][8 * ( kk & 1 ) + e] * scale_log2e - ms[qt] );
         }
-      }
-      l[qt] += sum[0] + sum[1];
-    }
-
-    // ---- the next stage's scores: nothing below depends on them
-    if ( i + 1 < my_stages ) {
-      scores( st, buf ^ 1 );
-    }
-
-    // ---- O^T += V^T P^T.  The A operand (32 dims x 16 keys; a lane: one dim, the 8 keys of its slots) comes out of LDS transposed:
-    //      ds_read_b64_tr_b16 hands lane i of a 16-lane group element i of each of four 32-byte rows that the group's lanes point
-    //      at (lanes 4 e .. 4 e + 3 at row e), i.e. 4 keys of one dim per instruction.  Dim block i4 holds dims 32 i4 .. 32 i4 + 31.
-    //      The four dim blocks are independent accumulation chains; the reads of the next 16 keys go out first.
-    v4s va[2][4][2];
-    auto read_v = [&]( int kk ) {
-#pragma unroll
-      for ( int i4 = 0; i4 < 4; i4++ ) {
-#pragma unroll
-        for ( int half = 0; half < 2; half++ ) {
-          va[kk & 1][i4][half] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (lds_v4s)( (lds_char*)s_vt[buf] + ( v_lane ^ ( 64 * i4 ) ) + ( 16 * kk + 8 * half ) * 256 ) );
+        // the running sum takes the weights as the product will see them (rounded to half), two per instruction
+        const f16x2 p2 = { (_Float16)p[qt][e0], (_Float16)p[qt][e0 + 1] };
+        sum[qt][( e0 >> 1 ) & 1] = __builtin_amdgcn_fdot2( p2, f16x2 { (_Float16)1.0f, (_Float16)1.0f }, sum[qt][( e0 >> 1 ) & 1], false );
+        pk2[qt][e0 >> 1] = p2;
+        if ( e0 == 6 ) {
+          pk[qt][kk] = f16x8 { pk2[qt][0][0], pk2[qt][0][1], pk2[qt][1][0], pk2[qt][1][1], pk2[qt][2][0], pk2[qt][2][1], pk2[qt][3][0], pk2[qt][3][1] };
         }
       }
     };
-    read_v( 0 );
+    // The weights of the first 32 keys before the pairs (their scores' registers are then free for the next stage's), those of the
+    // other 32 beside the MFMAs of pairs 0..7.
 #pragma unroll
-    for ( int kk = 0; kk < 4; kk++ ) {
-      if ( kk + 1 < 4 ) {
-        read_v( kk + 1 );
+    for ( int kk = 0; kk < 2; kk++ ) {
+#pragma unroll
+      for ( int e0 = 0; e0 < 8; e0 += 2 ) {
+        weights( kk, e0 );
       }
+    }
+    __builtin_amdgcn_sched_barrier( 0 );
 #pragma unroll
-      for ( int i4 = 0; i4 < 4; i4++ ) {
-        const v4s lo = va[kk & 1][i4][0], hi = va[kk & 1][i4][1];
+    for ( int n = 0; n < 16; n++ ) {
+      const int kk = n >> 2, i4 = n & 3;
+      {
+        const v4s lo = va[n & 3][0], hi = va[n & 3][1];
         const v8s a8 = v8s { lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3] };
         const f16x8 a = __builtin_bit_cast( f16x8, a8 );
 #pragma unroll
@@ -367,6 +401,28 @@ __global__ __launch_bounds__( 256, NQT == 1 ? 2 : 1 ) void attn_prefill_mfma_ker
           acc[qt][i4] = __builtin_amdgcn_mfma_f32_32x32x16_f16( a, pk[qt][kk], acc[qt][i4], 0, 0, 0 );
         }
       }
+      // The next stage's scores are also computed behind the wave's last stage, where nothing uses them (one stage's worth of
+      // S-steps per column block): a branch around every S-step cuts the sequence into pieces that the register allocator handles
+      // badly (89 spilled registers), and so do two copies of the whole stage, with and without them (224).
+      score_step( st_nxt, n );
+      if ( n + 4 < 16 ) {
+        read_v( v_cur, n + 4 );
+        read_k( k_nxt, n + 4 );
+      }
+      if ( n < 8 ) {
+        weights( 2 + kk, 2 * i4 ); // vector ALU work beside the MFMAs of this pair
+      }
+      __builtin_amdgcn_sched_barrier( 0 );
+    }
+#pragma unroll
+    for ( int qt = 0; qt < NQT; qt++ ) {
+      l[qt] += sum[qt][0] + sum[qt][1];
+    }
+  };
+  for ( uint32_t i = 0; i < n_stages; i += 2 ) {
+    stage( i, s_k0, s_v0, s_k1, s_v1, st_a, st_b );
+    if ( i + 1 < n_stages ) {
+      stage( i + 1, s_k1, s_v1, s_k0, s_v0, st_b, st_a );
     }
   }
 
@@ -396,6 +452,7 @@ __global__ __launch_bounds__( 256, NQT == 1 ? 2 : 1 ) void attn_prefill_mfma_ker
       }
     }
   }
+  } // the work-group's two column blocks
 }
 
 template<int G, int NQT>
@@ -404,9 +461,13 @@ void launch_prefill_tiles( hipStream_t st, const void* q, const void* const* row
 {
   const uint32_t col_blocks = (uint32_t)( ( (uint64_t)n_tokens * G + 128 * NQT - 1 ) / ( 128 * NQT ) );
   const uint64_t n_pairs = batch * s->n_kv_heads;
-  const uint64_t blocks = ( n_pairs + 7 ) / 8 * 8 * col_blocks;
+  // two column blocks per work-group (equal work for all) when that still leaves at least four work-groups for each of the two
+  // places a CU has; a small launch keeps one column block per work-group
+  const uint64_t padded_pairs = ( n_pairs + 7 ) / 8 * 8;
+  const uint32_t paired = padded_pairs * ( ( col_blocks + 1 ) / 2 ) >= 8ull * (uint64_t)cu_count() ? 1 : 0;
+  const uint64_t blocks = padded_pairs * ( paired ? ( col_blocks + 1 ) / 2 : col_blocks );
   attn_prefill_mfma_kernel<G, NQT><<<(unsigned)blocks, 256, 0, st>>>( static_cast<const __half*>( q ), reinterpret_cast<const __half* const*>( rows ), start,
-                                                                     static_cast<__half*>( xb ), s->n_kv_heads, n_tokens, col_blocks, (uint32_t)n_pairs,
+                                                                     static_cast<__half*>( xb ), s->n_kv_heads, n_tokens, col_blocks, (uint32_t)n_pairs, paired,
                                                                      LOG2E / sqrtf( (float)s->head_size ) );
 }
 

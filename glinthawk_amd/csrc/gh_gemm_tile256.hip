@@ -254,9 +254,11 @@ __global__ __launch_bounds__( T256_THREADS, 1 ) void gemm_tile256_kernel( __half
         }
       }
     }
+    __builtin_amdgcn_s_waitcnt( 0x0F70 ); // vmcnt(0): this wave's loads-to-LDS have landed (the barrier's own fence only orders LDS instructions)
     __syncthreads();
   };
   fetch( s_w0, s_x0, 0, 0, N_LOADS );
+  __builtin_amdgcn_s_waitcnt( 0x0F70 );
   __syncthreads();
   for ( uint32_t j = 0;; ) {
     step( s_w0, s_x0, s_w1, s_x1, j );

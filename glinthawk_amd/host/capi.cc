@@ -121,9 +121,14 @@ struct StageImpl : StageBase
   }
   void set_prompt( size_t i, uint32_t context_id, uint32_t token, uint32_t pos, float temp, uint32_t plen, uint32_t mcl ) override
   {
+    GLINT_CHECK( i < state.batch_size() );
     state.set_prompt( i, context_id, token, pos, temp, plen, mcl );
   }
-  void discard( size_t i ) override { state.discard( i ); }
+  void discard( size_t i ) override
+  {
+    GLINT_CHECK( i < state.batch_size() );
+    state.discard( i );
+  }
   void set_next( uint32_t layer, int stage ) override
   {
     state.set_next_layer( layer );
@@ -521,6 +526,15 @@ void glint_stage_set_prompt( void* h, uint32_t row, uint32_t context_id, uint32_
                              uint32_t max_completion_length )
 {
   static_cast<StageBase*>( h )->set_prompt( row, context_id, token, pos, temperature, prompt_length, max_completion_length );
+}
+// rows [0, n) at once: one call per batch instead of one per row (a serving loop fills hundreds of rows per step)
+void glint_stage_set_prompts( void* h, uint32_t n, const uint32_t* context_ids, const uint32_t* tokens, const uint32_t* positions, float temperature,
+                              uint32_t prompt_length, uint32_t max_completion_length )
+{
+  auto* stage = static_cast<StageBase*>( h );
+  for ( uint32_t i = 0; i < n; i++ ) {
+    stage->set_prompt( i, context_ids[i], tokens[i], positions[i], temperature, prompt_length, max_completion_length );
+  }
 }
 void glint_stage_discard( void* h, uint32_t row ) { static_cast<StageBase*>( h )->discard( row ); }
 void glint_stage_set_next( void* h, uint32_t layer, int stage ) { static_cast<StageBase*>( h )->set_next( layer, stage ); }

@@ -46,6 +46,7 @@ def host_lib() -> C.CDLL:
             "glint_stage_base_tensor_ptr": (vp, [vp, u32, C.POINTER(u64)]),
             "glint_stage_new_state": (None, [vp, u32, u32, C.c_int]),
             "glint_stage_set_prompt": (None, [vp, u32, u32, u32, u32, C.c_float, u32, u32]),
+            "glint_stage_set_prompts": (None, [vp, u32, vp, vp, vp, C.c_float, u32, u32]),
             "glint_stage_discard": (None, [vp, u32]),
             "glint_stage_set_next": (None, [vp, u32, C.c_int]),
             "glint_stage_acquire_contexts": (C.c_int, [vp]),
@@ -167,6 +168,17 @@ class Stage:
                    prompt_length: int = 1, max_completion_length: int = 0) -> None:
         host_lib().glint_stage_set_prompt(self._h, row, context_id, token, pos, temperature, prompt_length,
                                           max_completion_length)
+
+    def set_prompts(self, context_ids, tokens, positions, temperature: float = 0.0, prompt_length: int = 1,
+                    max_completion_length: int = 0) -> None:
+        """set_prompt for rows 0 .. n-1 in one call (three arrays of n values)."""
+        ids = np.ascontiguousarray(context_ids, dtype=np.uint32)
+        tok = np.ascontiguousarray(tokens, dtype=np.uint32)
+        pos = np.ascontiguousarray(positions, dtype=np.uint32)
+        if not (ids.ndim == tok.ndim == pos.ndim == 1 and ids.size == tok.size == pos.size):
+            raise ValueError("set_prompts: three one-dimensional arrays of equal length")
+        host_lib().glint_stage_set_prompts(self._h, ids.size, ids.ctypes.data, tok.ctypes.data, pos.ctypes.data, temperature,
+                                           prompt_length, max_completion_length)
 
     def discard(self, row: int) -> None:
         host_lib().glint_stage_discard(self._h, row)

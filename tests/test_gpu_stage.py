@@ -303,3 +303,22 @@ def test_paged_contexts_equal_static_and_follow_block_rule():
     # positions 0, 1, 2 and the restart see only rows written in this run: identical bits in both modes
     for k in (0, 1, 2, 7, 8):
         assert np.array_equal(outs[0][k], outs[1][k])
+
+
+def test_set_prompts_equals_row_by_row():
+    name = "test-tiny"
+    cfg = SHAPES[name]
+    a = S.Stage(name, "f32", 0, cfg.n_layers, 5, 5, with_cls=True)
+    b = S.Stage(name, "f32", 0, cfg.n_layers, 5, 5, with_cls=True)
+    ids, tokens, pos = [40, 41, 42, 43, 44], [3, 1, 4, 1, 5], [0, 7, 2, 9, 1]
+    a.new_state(5)
+    b.new_state(5)
+    for i in range(5):
+        a.set_prompt(i, ids[i], tokens[i], pos[i], 0.5, 3, 2)
+    b.set_prompts(ids, tokens, pos, 0.5, 3, 2)
+    assert [a.row(i) for i in range(5)] == [b.row(i) for i in range(5)]
+    assert a.get_state_bytes() == b.get_state_bytes()
+    with pytest.raises(ValueError):
+        b.set_prompts(ids, tokens[:4], pos)
+    a.close()
+    b.close()
