@@ -27,6 +27,7 @@ int gemm_stream_gate_launch( __half* hb, const __half* x, const __half* w13, uin
 bool gemm_tile256_applicable( uint64_t s, uint64_t r, uint64_t b, const void* x, const void* w, const void* xout );
 int gemm_tile256_launch( __half* xout, float* partial, const __half* x, const __half* w, uint64_t s, uint64_t r, uint64_t b, int epilogue, hipStream_t st,
                          uint32_t splits, uint32_t k_len );
+uint64_t gemm_tile256_token_split( uint64_t s, uint64_t r, uint64_t b );
 void gemm_tile256_split_plan( uint64_t s, uint64_t r, uint64_t b, const void* x, const void* w, uint32_t* splits, uint32_t* k_len );
 void gemm_tile256_tuning( int rows );
 // large-batch (prefill) kernel (gh_gemm_tile.hip)
@@ -241,6 +242,17 @@ int gemm_gate_one_launch( void* hb, const void* x, const void* w13, uint64_t s, 
   return gemm_stream_gate_launch( static_cast<__half*>( hb ), static_cast<const __half*>( x ), static_cast<const __half*>( w13 ), s, hidden, b, st );
 }
 
+// Tokens of the first part when a many-row product is better run as two products along the tokens (see
+// gemm_tile256_token_split), 0 otherwise.
+uint64_t gemm_token_split( uint64_t s, uint64_t r, uint64_t b, gh_dtype dt, const void* x, const void* w, const void* xout )
+{
+  if ( dt != GH_F16 || g_force_kernel != 0 || !gemm_tile256_applicable( s, r, b, x, w, xout ) ) {
+    return 0;
+  }
+  const uint64_t b1 = gemm_tile256_token_split( s, r, b );
+  return b1 != 0 && gemm_tile256_applicable( s, r, b1, x, w, xout ) && ( b1 * r * 2 ) % 16 == 0 && ( b1 * s * 2 ) % 16 == 0 ? b1 : 0;
+}
+
 // Many rows: the large tile kernel with the op that follows the product in its epilogue, 1 = xout += product
 // (accum).  *done = false: nothing was launched (shape or alignment not for that kernel), the caller takes
 // its other route.
@@ -414,6 +426,13 @@ int gh_matmul( void* xout, const void* x, const void* w, uint64_t s, uint64_t r,
   GH_REQUIRE( xout && x && w, "gh_matmul: NULL pointer" );
   GH_REQUIRE( s > 0 && s <= 0x7fffffffull && r <= 0x7fffffffull && b <= 0x7fffffffull, "gh_matmul: bad shape" );
   hipStream_t st = as_stream( stream );
+  if ( const uint64_t b1 = gemm_token_split( s, r, b, dt, x, w, xout ) ) { // two products along the tokens
+    const uint64_t elem = 2;
+    if ( int rc = gh_matmul( xout, x, w, s, r, b1, dt, stream ) ) {
+      return rc;
+    }
+    return gh_matmul( static_cast<char*>( xout ) + b1 * r * elem, static_cast<const char*>( x ) + b1 * s * elem, w, s, r, b - b1, dt, stream );
+  }
   float* partial = nullptr;
   uint32_t splits = 0;
   if ( int rc = gemm_partials( xout, x, w, s, r, b, dt, st, false, &partial, &splits ) ) {

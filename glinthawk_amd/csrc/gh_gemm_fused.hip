@@ -11,6 +11,7 @@ namespace gh {
 int gemm_partials( void* xout, const void* x, const void* w, uint64_t s, uint64_t r, uint64_t b, gh_dtype dt, hipStream_t st, bool want_partials,
                    float** partial_out, uint32_t* splits_out );
 int gemm_gate_one_launch( void* hb, const void* x, const void* w13, uint64_t s, uint64_t hidden, uint64_t b, gh_dtype dt, hipStream_t st, bool* done );
+uint64_t gemm_token_split( uint64_t s, uint64_t r, uint64_t b, gh_dtype dt, const void* x, const void* w, const void* xout );
 int gemm_tile_epilogue_launch( void* xout, const void* x, const void* w, uint64_t s, uint64_t r, uint64_t b, gh_dtype dt, int epilogue, hipStream_t st,
                                bool* done );
 
@@ -304,6 +305,14 @@ int gh_matmul_accum( void* residual, const void* x, const void* w, uint64_t s, u
   GH_REQUIRE( residual != nullptr, "gh_matmul_accum: NULL residual" );
   GH_REQUIRE( ( norm_out == nullptr ) == ( norm_weight == nullptr ), "gh_matmul_accum: norm_out and norm_weight go together" );
   hipStream_t st = as_stream( stream );
+  if ( const uint64_t b1 = gemm_token_split( s, r, b, dt, x, w, residual ) ) { // two products along the tokens (rows are independent)
+    const uint64_t elem = 2;
+    if ( int rc = gh_matmul_accum( residual, x, w, s, r, b1, norm_out, norm_weight, dt, stream ) ) {
+      return rc;
+    }
+    return gh_matmul_accum( static_cast<char*>( residual ) + b1 * r * elem, static_cast<const char*>( x ) + b1 * s * elem, w, s, r, b - b1,
+                            norm_out ? static_cast<char*>( norm_out ) + b1 * r * elem : nullptr, norm_weight, dt, stream );
+  }
   // many rows (prompt tokens): the residual is added in the tile kernel's epilogue, no fp32 partials;
   // the norm of the new residual, when asked for, is the plain row kernel
   bool done = false;

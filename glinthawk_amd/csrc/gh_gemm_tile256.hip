@@ -445,6 +445,37 @@ bool gemm_tile256_applicable( uint64_t s, uint64_t r, uint64_t b, const void* x,
          && ( ( reinterpret_cast<uintptr_t>( x ) | reinterpret_cast<uintptr_t>( w ) | reinterpret_cast<uintptr_t>( xout ) ) & 15u ) == 0;
 }
 
+// A launch is as slow as its number of rounds (one work-group per CU), so a product whose tiles leave the last round mostly
+// empty pays for a whole round there: 8192 rows x 4480 tokens are 576 tiles of 256 x 256, 2.25 rounds, and take 3.  Such a product
+// is cut in two along the tokens: the first part a number of tokens whose tiles fill their rounds, the rest a product of a few
+// hundred tokens that goes its own way (smaller tiles, or this kernel with the K range split).  Returns the tokens of the first
+// part, 0 to leave the product whole.  Costs in percent of a round of 256-row tiles; a round of 384-row tiles as in tile256_rows().
+uint64_t gemm_tile256_token_split( uint64_t s, uint64_t r, uint64_t b )
+{
+  if ( g_tile_rows != 0 || b < 3 * TN2 ) {
+    return 0;
+  }
+  const uint64_t cost384 = s >= 7168 ? 143 : 136;
+  auto cost = [&]( uint64_t tokens ) { return std::min( 100 * rounds_per_xcd( r, tokens, 256 ), cost384 * rounds_per_xcd( r, tokens, 384 ) ); };
+  const uint64_t whole = cost( b );
+  uint64_t best = whole, best_b1 = 0;
+  const uint64_t token_tiles = b / TN2;
+  for ( uint64_t t = token_tiles; t + 8 >= token_tiles && t >= 2; t-- ) {
+    const uint64_t b1 = t * TN2;
+    if ( b1 >= b ) {
+      continue;
+    }
+    // the rest: its flops in rounds of this kernel, at 60 % of this kernel's rate, plus a start-up
+    const uint64_t rest = 100 * ( b - b1 ) * r / ( (uint64_t)TM2 * TN2 * (uint64_t)cu_count() ) * 10 / 6 + 15;
+    const uint64_t c = cost( b1 ) + rest;
+    if ( c < best ) {
+      best = c;
+      best_b1 = b1;
+    }
+  }
+  return 100 * best < 92 * whole ? best_b1 : 0;
+}
+
 // Few tiles (a decode step of some hundred rows, or a narrow product): the K range is split over several work-groups per tile so
 // that the chip is full in one round, and the fp32 sums of each split go to partial[split].  *splits = 0: not for this shape.
 void gemm_tile256_split_plan( uint64_t s, uint64_t r, uint64_t b, const void* x, const void* w, uint32_t* splits, uint32_t* k_len )

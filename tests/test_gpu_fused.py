@@ -22,7 +22,7 @@ def _init():
                                    # more rows than one streaming slab: the tile kernels write the partials
                                    (100, 512, 260), (256, 1024, 512), (300, 4096, 1000),
                                    # enough 256-token tiles: the residual is added in the large tile kernel's epilogue (f16, r % 8 == 0)
-                                   (768, 8192, 16384), (2048, 512, 6152), (3000, 1024, 6144),
+                                   (768, 8192, 16384), (2048, 512, 6152), (3000, 1024, 6144), (2300, 512, 8192),
                                    (2048, 512, 6150)])          # r % 8 != 0: fp32 partials and the row kernel
 def test_matmul_accum_and_norm(dt, b, s, r):
     g = torch.Generator(device="cuda").manual_seed(1)
