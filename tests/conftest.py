@@ -37,7 +37,7 @@ def pytest_sessionfinish(session, exitstatus):
         return
     if not helpers.DRIFT:
         return
-    out = os.path.join(ROOT, "gpurun_out")
+    out = os.path.join(ROOT, os.environ.get("GLINT_TEST_OUTPUT_DIR", "gpurun_out"))
     os.makedirs(out, exist_ok=True)
     with open(os.path.join(out, "fp16_drift.txt"), "w") as f:
         f.write("mean-relative distances: HIP vs fp16 oracle | HIP vs fp32 oracle | fp16 oracle vs fp32 oracle\n")

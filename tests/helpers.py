@@ -26,7 +26,7 @@ def assert_close(got, want, max_abs=MAX_ABS_TOL, mean_rel=MEAN_REL_TOL, what="")
 
 
 # Measured distances of the fp16 stage outputs: (what, HIP vs fp16 oracle, HIP vs fp32 oracle, fp16 oracle vs fp32 oracle),
-# mean-relative; written to gpurun_out/fp16_drift.txt at the end of a test session (conftest.py).
+# mean-relative; written to a text file (fp16_drift.txt) at the end of a test session (conftest.py).
 DRIFT = []
 
 

@@ -77,6 +77,36 @@ def test_prefill_generic_shapes(shape, dt, n_tokens):
     run_case(shape, dt, GH_ATTN_AUTO, n_tokens, starts, [True, True, True])
 
 
+# launches large enough for the kernel to give each work-group two column blocks (the longest with the shortest, and so on), with
+# ragged start positions, an odd number of column blocks (the middle one alone) and an absent context: against the decode kernels
+# run on one row per (context, token)
+@pytest.mark.parametrize("shape,batch,n_tokens", [(Shape(dim=5120, n_layers=1, n_heads=40, n_kv_heads=40, hidden_dim=64, seq_len=4096), 11, 1152),
+                                                  (Shape(dim=8192, n_layers=1, n_heads=64, n_kv_heads=8, hidden_dim=64, seq_len=4096), 9, 1008)],
+                         ids=["mha40-9-column-blocks", "gqa8-63-column-blocks"])
+def test_prefill_mfma_paired_column_blocks(shape, batch, n_tokens):
+    g = torch.Generator(device="cuda").manual_seed(batch)
+    cache = torch.randn((batch, shape.seq_len, 2 * shape.kv_dim), generator=g, device="cuda").half()
+    row_bytes = 2 * shape.kv_dim * 2
+    present = [i != 4 for i in range(batch)]
+    rows = ops.row_table([cache.data_ptr() + i * shape.seq_len * row_bytes if present[i] else 0 for i in range(batch)])
+    starts = [(977 * i) % (shape.seq_len - n_tokens) for i in range(batch)]
+    starts[0] = 0
+    start = torch.tensor(starts, dtype=torch.int32, device="cuda")
+    q = torch.randn((batch * n_tokens, shape.dim), generator=g, device="cuda").half()
+    got = torch.full_like(q, 5.0)
+    want = torch.full_like(q, 5.0)
+    ops.attn_prefill(q, rows, start, got, n_tokens, max(starts), shape, variant=GH_ATTN_MFMA)
+    ops.attn_prefill(q, rows, start, want, n_tokens, max(starts), shape, variant=GH_ATTN_GENERIC)
+    live = torch.tensor([present[i] for i in range(batch) for _ in range(n_tokens)], device="cuda")
+    assert torch.all(got[~live] == 5.0) and torch.all(want[~live] == 5.0)
+    assert torch.isfinite(got[live]).all()
+    a, r = errors(got[live].float().cpu().numpy(), want[live].float().cpu().numpy())
+    assert a < 4e-3 and r < 1e-3, (a, r)
+    # token 0 of the context that starts at position 0 attends key 0 only: weight exactly 1
+    v0 = cache[0, 0, shape.kv_dim:].reshape(shape.n_kv_heads, 1, shape.head_size).expand(-1, shape.gqa_size, -1).reshape(-1)
+    assert torch.equal(got[0], v0)
+
+
 def test_prefill_tables():
     layer_rows = ops.row_table([1 << 20, 0, 3 << 20])
     start = torch.tensor([0, 4, 10], dtype=torch.int32, device="cuda")
