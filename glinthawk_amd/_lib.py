@@ -63,6 +63,12 @@ SIGNATURES = {
     "gh_last_error": (C.c_char_p, []),
     "gh_device_name": (_i, [C.c_char_p, C.c_size_t]),
     "gh_sync": (_i, [_vp]),
+    "gh_stream_create": (_i, [C.POINTER(_vp)]),
+    "gh_stream_destroy": (_i, [_vp]),
+    "gh_event_create": (_i, [C.POINTER(_vp)]),
+    "gh_event_destroy": (_i, [_vp]),
+    "gh_event_record": (_i, [_vp, _vp]),
+    "gh_stream_wait_event": (_i, [_vp, _vp]),
     "gh_malloc": (_i, [C.POINTER(_vp), _u64]),
     "gh_free": (_i, [_vp]),
     "gh_host_malloc": (_i, [C.POINTER(_vp), _u64]),

@@ -299,6 +299,59 @@ int gh_device_name( char* out, size_t len )
   return GH_OK;
 }
 
+int gh_stream_create( gh_stream* out )
+{
+  if ( int rc = ensure_init() ) {
+    return rc;
+  }
+  GH_REQUIRE( out != nullptr, "gh_stream_create: NULL output" );
+  hipStream_t s = nullptr;
+  GH_HIP( hipStreamCreateWithFlags( &s, hipStreamNonBlocking ) ); // default priority
+  *out = s;
+  return GH_OK;
+}
+
+int gh_stream_destroy( gh_stream stream )
+{
+  GH_REQUIRE( stream != nullptr, "gh_stream_destroy: the default stream is not the caller's" );
+  GH_HIP( hipStreamSynchronize( as_stream( stream ) ) );
+  GH_HIP( hipStreamDestroy( as_stream( stream ) ) );
+  return GH_OK;
+}
+
+int gh_event_create( gh_event* out )
+{
+  if ( int rc = ensure_init() ) {
+    return rc;
+  }
+  GH_REQUIRE( out != nullptr, "gh_event_create: NULL output" );
+  hipEvent_t e = nullptr;
+  GH_HIP( hipEventCreateWithFlags( &e, hipEventDisableTiming ) );
+  *out = e;
+  return GH_OK;
+}
+
+int gh_event_destroy( gh_event event )
+{
+  GH_REQUIRE( event != nullptr, "gh_event_destroy: NULL event" );
+  GH_HIP( hipEventDestroy( static_cast<hipEvent_t>( event ) ) );
+  return GH_OK;
+}
+
+int gh_event_record( gh_event event, gh_stream stream )
+{
+  GH_REQUIRE( event != nullptr, "gh_event_record: NULL event" );
+  GH_HIP( hipEventRecord( static_cast<hipEvent_t>( event ), as_stream( stream ) ) );
+  return GH_OK;
+}
+
+int gh_stream_wait_event( gh_stream stream, gh_event event )
+{
+  GH_REQUIRE( event != nullptr, "gh_stream_wait_event: NULL event" );
+  GH_HIP( hipStreamWaitEvent( as_stream( stream ), static_cast<hipEvent_t>( event ), 0 ) );
+  return GH_OK;
+}
+
 int gh_sync( gh_stream stream )
 {
   if ( int rc = ensure_init() ) {

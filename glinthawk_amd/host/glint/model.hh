@@ -389,6 +389,21 @@ public:
     DType* pxb = pf_xb_.get();
     DType* pq = pf_q_.get();
     DType* phb = pf_hb_.get();
+    // Many tokens arriving from and leaving for the host: the rows are cut into four runs, and the copies of a run go over a
+    // stream of their own, so that the first layer's projections of run c (row-wise work: norm, wq, wkv, append, RoPE) overlap the
+    // upload of run c + 1 and the download of run c overlaps the last layer's w2 product of run c + 1.  Everything in between
+    // (attention needs all rows of a context) runs on all rows at once.
+    const bool pipelined = n >= 8192 && !( first_layer == 0 && token_ids != nullptr ) && ( acts_in_host != nullptr );
+    std::vector<std::pair<uint64_t, uint64_t>> chunks; // (first row, rows)
+    if ( pipelined ) {
+      ensure_copy_stream();
+      const uint64_t per = ( ( n + N_CHUNKS - 1 ) / N_CHUNKS + 255 ) / 256 * 256;
+      for ( uint64_t r0 = 0; r0 < n; r0 += per ) {
+        chunks.emplace_back( r0, std::min( per, n - r0 ) );
+      }
+    } else {
+      chunks.emplace_back( 0, n );
+    }
     if ( first_layer == 0 && token_ids != nullptr ) {
       for ( uint64_t r = 0; r < n; r++ ) {
         GLINT_CHECK( token_ids[r] < Config::vocab_size );
@@ -397,14 +412,23 @@ public:
       }
     } else {
       GLINT_CHECK( acts_in_host != nullptr );
-      ops_.copy( px, acts_in_host, n * Config::dim * sizeof( DType ), CopyType::HostToDevice, true );
+      if ( pipelined ) {
+        for ( size_t c = 0; c < chunks.size(); c++ ) {
+          const uint64_t off = chunks[c].first * Config::dim;
+          GLINT_GH( gh_memcpy( px + off, acts_in_host + off, chunks[c].second * Config::dim * sizeof( DType ), GH_HOST_TO_DEVICE, 1, copy_lane_->stream ) );
+          GLINT_GH( gh_event_record( copy_lane_->in[c], copy_lane_->stream ) );
+        }
+      } else {
+        ops_.copy( px, acts_in_host, n * Config::dim * sizeof( DType ), CopyType::HostToDevice, true );
+      }
     }
 
     const gh_shape shape = LlamaOperations::shape();
     const uint64_t row_bytes = 2ull * Config::kv_dim * sizeof( DType );
     const bool fuse_wo = n <= 65535 && gh_matmul_fuses_many_rows( Config::dim, Config::dim, n, hip::gh_type<DType>() ) == 1;
-    const bool fuse_w2 = n <= 65535 && gh_matmul_fuses_many_rows( Config::hidden_dim, Config::dim, n, hip::gh_type<DType>() ) == 1;
-    ops_.template rmsnorm<Config::dim>( pxb, px, reinterpret_cast<float32_t*>( temp_ ), layers_[run[0]].rms_att_weight, n );
+    if ( !pipelined ) {
+      ops_.template rmsnorm<Config::dim>( pxb, px, reinterpret_cast<float32_t*>( temp_ ), layers_[run[0]].rms_att_weight, n );
+    }
     for ( size_t k = 0; k < run.size(); k++ ) {
       const auto& w = layers_[run[k]];
       // one table entry per (context, token) for this layer's rows
@@ -424,11 +448,20 @@ public:
         DType* pkv = pf_kv_.get();
         DType* pxb2 = pf_xb2_.get();
         DType* phb2 = pf_hb2_.get();
-        ops_.template matmul<Config::dim, Config::dim>( pq, pxb, w.wq, n );
-        ops_.template matmul<Config::dim, Config::kv_dim * 2>( pkv, pxb, w.wkv, n );
-        GLINT_GH( gh_kv_append( pf_token_rows(), pkv, n, Config::kv_dim, hip::gh_type<DType>(), ops_.stream() ) );
-        GLINT_GH( gh_rope( n, pf_pos(), base_.freq_cis_real, base_.freq_cis_imag, pq, pf_token_rows(), Config::n_kv_heads, Config::gqa_size, Config::head_size,
-                           hip::gh_type<DType>(), ops_.stream() ) );
+        // the row-wise work in front of the attention: run by run while the runs arrive (first layer of a pipelined call), else on all rows
+        const bool by_run = pipelined && k == 0;
+        for ( size_t c = 0; c < ( by_run ? chunks.size() : 1 ); c++ ) {
+          const uint64_t r0 = by_run ? chunks[c].first : 0, rows = by_run ? chunks[c].second : n;
+          if ( by_run ) {
+            GLINT_GH( gh_stream_wait_event( ops_.stream(), copy_lane_->in[c] ) );
+            ops_.template rmsnorm<Config::dim>( pxb + r0 * Config::dim, px + r0 * Config::dim, reinterpret_cast<float32_t*>( temp_ ), w.rms_att_weight, rows );
+          }
+          ops_.template matmul<Config::dim, Config::dim>( pq + r0 * Config::dim, pxb + r0 * Config::dim, w.wq, rows );
+          ops_.template matmul<Config::dim, Config::kv_dim * 2>( pkv + r0 * Config::kv_dim * 2, pxb + r0 * Config::dim, w.wkv, rows );
+          GLINT_GH( gh_kv_append( pf_token_rows() + r0, pkv + r0 * Config::kv_dim * 2, rows, Config::kv_dim, hip::gh_type<DType>(), ops_.stream() ) );
+          GLINT_GH( gh_rope( rows, pf_pos() + r0, base_.freq_cis_real, base_.freq_cis_imag, pq + r0 * Config::dim, pf_token_rows() + r0, Config::n_kv_heads,
+                             Config::gqa_size, Config::head_size, hip::gh_type<DType>(), ops_.stream() ) );
+        }
         GLINT_GH( gh_attn_prefill( pq, layer_rows_dev( k ), pos_dev(), pxb, batch, n_tokens, max_start, &shape, hip::gh_type<DType>(), pf_attn_ws_.get(),
                                    pf_attn_ws_bytes_, GH_ATTN_AUTO, ops_.stream() ) );
         // the residual add rides in the tile kernel's epilogue where the library does that for the shape
@@ -444,20 +477,38 @@ public:
         ops_.template matmul<Config::dim, Config::hidden_dim>( phb2, pxb, w.w3, n );
         ops_.template silu<Config::hidden_dim>( phb, phb2, n );
         const DType* next_norm = k + 1 < run.size() ? layers_[run[k + 1]].rms_att_weight : nullptr;
-        if ( fuse_w2 ) {
-          ops_.template matmul_accum<Config::hidden_dim, Config::dim>( px, phb, w.w2, n, next_norm ? pxb : nullptr, next_norm );
-        } else {
-          ops_.template matmul<Config::hidden_dim, Config::dim>( pxb, phb, w.w2, n );
-          ops_.template accum<Config::dim>( px, pxb, n );
-          if ( next_norm != nullptr ) {
-            ops_.template rmsnorm<Config::dim>( pxb, px, reinterpret_cast<float32_t*>( temp_ ), next_norm, n );
+        // the last product of the call run by run when its result leaves for the host, each run's download behind it
+        const bool out_by_run = pipelined && k + 1 == run.size() && acts_out_host != nullptr;
+        for ( size_t c = 0; c < ( out_by_run ? chunks.size() : 1 ); c++ ) {
+          const uint64_t r0 = out_by_run ? chunks[c].first : 0, rows = out_by_run ? chunks[c].second : n;
+          DType* cx = px + r0 * Config::dim;
+          DType* cxb = pxb + r0 * Config::dim;
+          const DType* chb = phb + r0 * Config::hidden_dim;
+          // whether the residual add rides in the product's epilogue is a property of the shape, so it is asked per run
+          if ( rows <= 65535 && gh_matmul_fuses_many_rows( Config::hidden_dim, Config::dim, rows, hip::gh_type<DType>() ) == 1 ) {
+            ops_.template matmul_accum<Config::hidden_dim, Config::dim>( cx, chb, w.w2, rows, next_norm ? cxb : nullptr, next_norm );
+          } else {
+            ops_.template matmul<Config::hidden_dim, Config::dim>( cxb, chb, w.w2, rows );
+            ops_.template accum<Config::dim>( cx, cxb, rows );
+            if ( next_norm != nullptr ) {
+              ops_.template rmsnorm<Config::dim>( cxb, cx, reinterpret_cast<float32_t*>( temp_ ), next_norm, rows );
+            }
+          }
+          if ( out_by_run ) {
+            GLINT_GH( gh_event_record( copy_lane_->out[c], ops_.stream() ) );
+            GLINT_GH( gh_stream_wait_event( copy_lane_->stream, copy_lane_->out[c] ) );
+            GLINT_GH( gh_memcpy( acts_out_host + r0 * Config::dim, cx, rows * Config::dim * sizeof( DType ), GH_DEVICE_TO_HOST, 1, copy_lane_->stream ) );
           }
         }
       }
     }
 
     if ( acts_out_host != nullptr ) {
-      ops_.copy( acts_out_host, px, n * Config::dim * sizeof( DType ), CopyType::DeviceToHost );
+      if ( pipelined ) {
+        GLINT_GH( gh_sync( copy_lane_->stream ) ); // the downloads queued behind the last layer
+      } else {
+        ops_.copy( acts_out_host, px, n * Config::dim * sizeof( DType ), CopyType::DeviceToHost );
+      }
     }
     const size_t last = run.back();
     if ( next_tokens != nullptr && last == Config::n_layers - 1 && settings_.hosts( last, InferenceStage::Classification ) ) {
@@ -866,12 +917,44 @@ private:
     pf_attn_ws_ = ops_.device_allocate( std::max<uint64_t>( pf_attn_ws_bytes_, 16 ) );
     pf_capacity_ = n;
   }
+  // the stream and events of the pipelined prefill, created on first use and kept for the life of the model
+  static constexpr size_t N_CHUNKS = 4;
+  struct CopyLane
+  {
+    gh_stream stream { nullptr };
+    gh_event in[N_CHUNKS] {}, out[N_CHUNKS] {};
+    CopyLane()
+    {
+      GLINT_GH( gh_stream_create( &stream ) );
+      for ( size_t c = 0; c < N_CHUNKS; c++ ) {
+        GLINT_GH( gh_event_create( &in[c] ) );
+        GLINT_GH( gh_event_create( &out[c] ) );
+      }
+    }
+    ~CopyLane()
+    {
+      for ( size_t c = 0; c < N_CHUNKS; c++ ) {
+        (void)gh_event_destroy( in[c] );
+        (void)gh_event_destroy( out[c] );
+      }
+      (void)gh_stream_destroy( stream );
+    }
+    CopyLane( const CopyLane& ) = delete;
+    CopyLane& operator=( const CopyLane& ) = delete;
+  };
+  void ensure_copy_stream()
+  {
+    if ( !copy_lane_ ) {
+      copy_lane_ = std::make_unique<CopyLane>();
+    }
+  }
   void** pf_token_rows() const { return reinterpret_cast<void**>( pf_tables_.get() ); }
   uint32_t* pf_pos() const { return reinterpret_cast<uint32_t*>( pf_token_rows() + pf_capacity_ ); }
 
   DevicePtr base_storage_ {}, layer_storage_ {}, scratch_storage_ {}, attn_ws_ {}, tables_dev_ {};
   DevicePtr pf_x_ {}, pf_xb_ {}, pf_q_ {}, pf_hb_ {}, pf_hb2_ {}, pf_xb2_ {}, pf_kv_ {}, pf_tables_ {}, pf_attn_ws_ {};
   uint64_t pf_capacity_ { 0 }, pf_attn_ws_bytes_ { 0 };
+  std::unique_ptr<CopyLane> copy_lane_ {};
   uint64_t attn_ws_bytes_ { 0 };
   uint8_t* tables_host_ { nullptr };
   BaseWeights<DType> base_ {};

@@ -83,6 +83,16 @@ int gh_init( int device );              /* selects the device, checks it is gfx9
 const char* gh_last_error( void );
 int gh_device_name( char* out, size_t len );
 int gh_sync( gh_stream stream );        /* hipStreamSynchronize (NULL: whole device) */
+/* Streams and events for callers that overlap copies with compute (the reference's CUDA target keeps streams of its own,
+ * arch/cuda/common/ops.cuh:78-80,100-108).  A created stream has the default priority and does not synchronise with the
+ * default stream; gh_stream_wait_event makes later work on `stream` wait for what `event` recorded. */
+typedef void* gh_event;
+int gh_stream_create( gh_stream* out );
+int gh_stream_destroy( gh_stream stream );
+int gh_event_create( gh_event* out );
+int gh_event_destroy( gh_event event );
+int gh_event_record( gh_event event, gh_stream stream );
+int gh_stream_wait_event( gh_stream stream, gh_event event );
 
 /* Operations::device_allocate / DeviceUniquePtr deleter (arch/cuda/common/ops.cuh:27-35,748-756) */
 int gh_malloc( void** out, uint64_t bytes );

@@ -678,3 +678,40 @@ def test_vmm_commit_out_of_range_is_refused():
     _lib.check(L.gh_vmm_clear(region))
     assert L.gh_vmm_committed_bytes(region) == 0
     _lib.check(L.gh_vmm_free(region))
+
+
+# ------------------------------------------------------------------ streams and events of the C-ABI
+def test_streams_and_events_order_a_copy_before_a_kernel():
+    import ctypes as C
+    from glinthawk_amd import _lib
+    L = _lib.lib()
+    stream, event = C.c_void_p(), C.c_void_p()
+    _lib.check(L.gh_stream_create(C.byref(stream)))
+    _lib.check(L.gh_event_create(C.byref(event)))
+    assert stream.value and event.value
+    n = 1 << 22
+    src = ops.pinned_empty((n,), np.float16)
+    src[:] = (np.arange(n) % 1000).astype(np.float16)
+    a = torch.zeros(n, dtype=torch.float16, device="cuda")
+    b = torch.ones(n, dtype=torch.float16, device="cuda")
+    # upload on the caller's stream, kernel on the default stream behind the event
+    _lib.check(L.gh_memcpy(a.data_ptr(), src.ctypes.data, 2 * n, _lib.GH_H2D, 1, stream))
+    _lib.check(L.gh_event_record(event, stream))
+    _lib.check(L.gh_stream_wait_event(None, event))
+    _lib.check(L.gh_accum(b.data_ptr(), a.data_ptr(), n, 1, _lib.GH_F16, None))
+    _lib.check(L.gh_sync(None))
+    assert torch.equal(b.cpu(), torch.from_numpy(src.copy()) + 1)
+    # and the other way round: the download on the caller's stream waits for the kernel on the default stream
+    out = ops.pinned_empty((n,), np.float16)
+    out[:] = 0
+    _lib.check(L.gh_accum(b.data_ptr(), a.data_ptr(), n, 1, _lib.GH_F16, None))
+    _lib.check(L.gh_event_record(event, None))
+    _lib.check(L.gh_stream_wait_event(stream, event))
+    _lib.check(L.gh_memcpy(out.ctypes.data, b.data_ptr(), 2 * n, _lib.GH_D2H, 1, stream))
+    _lib.check(L.gh_sync(stream))
+    assert np.array_equal(out, (src.astype(np.float32) * 2 + 1).astype(np.float16))
+    for call in (lambda: L.gh_event_record(None, stream), lambda: L.gh_stream_wait_event(stream, None), lambda: L.gh_stream_destroy(None),
+                 lambda: L.gh_event_destroy(None), lambda: L.gh_stream_create(None)):
+        assert call() == -1
+    _lib.check(L.gh_event_destroy(event))
+    _lib.check(L.gh_stream_destroy(stream))
