@@ -95,6 +95,7 @@ SIGNATURES = {
     "gh_matmul_fuses_many_rows": (_i, [_u64, _u64, _u64, _i]),
     "gh_gemm_stream_plan": (_i, [_u64, _u64, _u64, _vp, _vp, _vp]),
     "gh_matmul": (_i, [_vp, _vp, _vp, _u64, _u64, _u64, _i, _vp]),
+    "gh_matmul_pair": (_i, [_vp, _vp, _vp, _vp, _u64, _u64, _u64, _u64, _i, _vp]),
     "gh_matmul_accum": (_i, [_vp, _vp, _vp, _u64, _u64, _u64, _vp, _vp, _i, _vp]),
     "gh_matmul_silu_gate": (_i, [_vp, _vp, _vp, _u64, _u64, _u64, _i, _vp]),
     "gh_matmul_qkv_rope_append": (_i, [_vp, _vp, _vp, _vp, _u64, _u64, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _i, _vp]),

@@ -26,7 +26,7 @@ int gemm_stream_gate_launch( __half* hb, const __half* x, const __half* w13, uin
 // 256 x 256 tile kernel for products with enough tiles (gh_gemm_tile256.hip)
 bool gemm_tile256_applicable( uint64_t s, uint64_t r, uint64_t b, const void* x, const void* w, const void* xout );
 int gemm_tile256_launch( __half* xout, float* partial, const __half* x, const __half* w, uint64_t s, uint64_t r, uint64_t b, int epilogue, hipStream_t st,
-                         uint32_t splits, uint32_t k_len );
+                         uint32_t splits, uint32_t k_len, __half* xout2 = nullptr, uint64_t r_first = 0 );
 uint64_t gemm_tile256_token_split( uint64_t s, uint64_t r, uint64_t b );
 void gemm_tile256_split_plan( uint64_t s, uint64_t r, uint64_t b, const void* x, const void* w, uint32_t* splits, uint32_t* k_len );
 void gemm_tile256_tuning( int rows );
@@ -413,6 +413,42 @@ int gh_gemm_stream_plan( uint64_t s, uint64_t r, uint64_t b, uint32_t* splits, u
   GH_REQUIRE( s >= 256 && s % 256 == 0 && r > 0 && b > 0, "gh_gemm_stream_plan: the streaming kernel takes s %% 256 == 0, r > 0, b > 0" );
   gemm_stream_plan( s, r, b, splits, k_per_split, rows_per_workgroup );
   return GH_OK;
+}
+
+int gh_matmul_pair( void* xout_a, void* xout_b, const void* x, const void* w, uint64_t s, uint64_t r_a, uint64_t r_b, uint64_t b, gh_dtype dt,
+                    gh_stream stream )
+{
+  if ( int rc = ensure_init() ) {
+    return rc;
+  }
+  if ( b == 0 ) {
+    return GH_OK;
+  }
+  GH_REQUIRE( xout_a && xout_b && x && w, "gh_matmul_pair: NULL pointer" );
+  GH_REQUIRE( dt == GH_F16 || dt == GH_F32, "gh_matmul_pair: unsupported dtype %d", (int)dt );
+  const uint64_t elem = dt == GH_F16 ? 2 : 4;
+  const uint64_t r = r_a + r_b;
+  GH_REQUIRE( s > 0 && s <= 0x7fffffffull && r <= 0x7fffffffull && b <= 0x7fffffffull, "gh_matmul_pair: bad shape" );
+  // many rows: one launch of the large tile kernel whose work-groups store to the matrix their rows belong to, so that the two
+  // products fill their rounds together (a product of 2048 rows alone leaves most of the chip idle)
+  if ( dt == GH_F16 && g_force_kernel == 0 && r_a > 0 && r_b > 0 && r_a % 8 == 0 && r_b % 8 == 0 && gemm_tile256_applicable( s, r, b, x, w, xout_a )
+       && ( reinterpret_cast<uintptr_t>( xout_b ) & 15u ) == 0 ) {
+    if ( const uint64_t b1 = gemm_token_split( s, r, b, dt, x, w, xout_a ) ) {
+      if ( ( b1 * r_a * elem ) % 16 == 0 && ( b1 * r_b * elem ) % 16 == 0 ) {
+        if ( int rc = gh_matmul_pair( xout_a, xout_b, x, w, s, r_a, r_b, b1, dt, stream ) ) {
+          return rc;
+        }
+        return gh_matmul_pair( static_cast<char*>( xout_a ) + b1 * r_a * elem, static_cast<char*>( xout_b ) + b1 * r_b * elem,
+                               static_cast<const char*>( x ) + b1 * s * elem, w, s, r_a, r_b, b - b1, dt, stream );
+      }
+    }
+    return gemm_tile256_launch( static_cast<__half*>( xout_a ), nullptr, static_cast<const __half*>( x ), static_cast<const __half*>( w ), s, r, b, 0,
+                                as_stream( stream ), 1, 0, static_cast<__half*>( xout_b ), r_a );
+  }
+  if ( int rc = gh_matmul( xout_a, x, w, s, r_a, b, dt, stream ) ) {
+    return rc;
+  }
+  return gh_matmul( xout_b, x, static_cast<const char*>( w ) + r_a * s * elem, s, r_b, b, dt, stream );
 }
 
 int gh_matmul( void* xout, const void* x, const void* w, uint64_t s, uint64_t r, uint64_t b, gh_dtype dt, gh_stream stream )

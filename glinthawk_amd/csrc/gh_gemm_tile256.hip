@@ -99,6 +99,8 @@ __global__ __launch_bounds__( T256_THREADS, 1 ) void gemm_tile256_kernel( __half
                                                                         uint32_t r,
                                                                         uint32_t b,
                                                                         uint32_t k_len, // k per split
+                                                                        __half* __restrict__ xout2, // rows from r_first on go here, as rows 0.. of a (b, r - r_first) matrix
+                                                                        uint32_t r_first, // rows [0, r_first) go to xout, a (b, r_first) matrix; == r: one output
                                                                         TileOrder ord )
 {
   // Four separate arrays, not [2][...]: the compiler orders an LDS read behind an outstanding
@@ -306,7 +308,9 @@ __global__ __launch_bounds__( T256_THREADS, 1 ) void gemm_tile256_kernel( __half
       const uint32_t chunk = slot ^ ( token & SWZ_MASK );
       const uint32_t col = tile_col0 + first_token + token, row = tile_row0 + 8 * chunk;
       if ( col < b && row < r ) {
-        uint4* dst = reinterpret_cast<uint4*>( xout + (uint64_t)col * r + row );
+        // two products that share their activations in one launch (r_first % 8 == 0: a 16-byte chunk never straddles the two)
+        const bool second = row >= r_first;
+        uint4* dst = reinterpret_cast<uint4*>( second ? xout2 + (uint64_t)col * ( r - r_first ) + ( row - r_first ) : xout + (uint64_t)col * r_first + row );
         union
         {
           uint4 raw;
@@ -379,7 +383,7 @@ __global__ __launch_bounds__( T256_THREADS, 1 ) void gemm_tile256_kernel( __half
             }
           }
         } else {
-          __half* dst = xout + (uint64_t)col * r + row;
+          __half* dst = xout + (uint64_t)col * r + row; // (one output only: the launch refuses two with r % 8 != 0)
           if ( whole ) {
             union
             {
@@ -505,8 +509,13 @@ void gemm_tile256_split_plan( uint64_t s, uint64_t r, uint64_t b, const void* x,
 // `partial` != nullptr: fp32 sums (splits, b, r) instead of xout; else `epilogue` 0 stores, 1 accumulates into xout (needs r % 8 == 0).
 // splits > 1 (from gemm_tile256_split_plan, with its k_len) needs `partial`.
 int gemm_tile256_launch( __half* xout, float* partial, const __half* x, const __half* w, uint64_t s, uint64_t r, uint64_t b, int epilogue, hipStream_t st,
-                         uint32_t splits, uint32_t k_len )
+                         uint32_t splits, uint32_t k_len, __half* xout2 = nullptr, uint64_t r_first = 0 )
 {
+  if ( xout2 == nullptr ) {
+    r_first = r;
+  }
+  GH_REQUIRE( xout2 == nullptr || ( partial == nullptr && epilogue == EPI_STORE && splits == 1 && r % 8 == 0 && r_first % 8 == 0 && r_first > 0 && r_first < r ),
+              "gh_matmul: two outputs need plain stores, no K split and row counts that are multiples of 8" );
   TileOrder ord;
   GH_REQUIRE( splits >= 1 && ( splits == 1 || ( partial != nullptr && k_len % TKS == 0 && (uint64_t)k_len * splits >= s && (uint64_t)k_len * ( splits - 1 ) < s ) ),
               "gh_matmul: bad K split for the 256-token tile kernel" );
@@ -533,7 +542,7 @@ int gemm_tile256_launch( __half* xout, float* partial, const __half* x, const __
   const int epi = partial != nullptr ? EPI_PARTIAL : epilogue;
   GH_REQUIRE( epi == EPI_STORE || epi == EPI_ACCUM || epi == EPI_PARTIAL, "gh_matmul: unknown tile epilogue %d", epi );
   GH_REQUIRE( epi != EPI_ACCUM || r % 8 == 0, "gh_matmul: the accumulating tile epilogue needs r %% 8 == 0" );
-#define GH_TILE256_LAUNCH( E, N ) gemm_tile256_kernel<E, N><<<grid, block, 0, st>>>( xout, partial, x, w, s32, r32, b32, k_len, ord )
+#define GH_TILE256_LAUNCH( E, N ) gemm_tile256_kernel<E, N><<<grid, block, 0, st>>>( xout, partial, x, w, s32, r32, b32, k_len, xout2, (uint32_t)r_first, ord )
 #define GH_TILE256_ROWS( E ) ( tile_rows == 384 ? GH_TILE256_LAUNCH( E, 3 ) : GH_TILE256_LAUNCH( E, 2 ) )
   switch ( epi ) {
     case EPI_STORE: GH_TILE256_ROWS( EPI_STORE ); break;

@@ -327,6 +327,12 @@ public:
   {
     GLINT_GH( gh_matmul_accum( x, xb, w, s, r, batch_size, norm_out, norm_weight, gh_type<DType>(), this->stream_ ) );
   }
+  // two products that share their activations, their weights one behind the other (wq then wkv): xa = xb . w[0:ra]^T, xo_b = xb . w[ra:]^T
+  template<uint64_t s, uint64_t ra, uint64_t rb>
+  void matmul_pair( DType* xo_a, DType* xo_b, const DType* xb, const DType* w, const uint64_t batch_size ) const
+  {
+    GLINT_GH( gh_matmul_pair( xo_a, xo_b, xb, w, s, ra, rb, batch_size, gh_type<DType>(), this->stream_ ) );
+  }
   // w1, w3, silu: hb = silu(xb . w1^T) * (xb . w3^T); w13 holds the rows of w1 followed by those of w3
   void matmul_silu_gate( DType* hb, const DType* xb, const DType* w13, const uint64_t batch_size ) const
   {

@@ -456,8 +456,13 @@ public:
             GLINT_GH( gh_stream_wait_event( ops_.stream(), copy_lane_->in[c] ) );
             ops_.template rmsnorm<Config::dim>( pxb + r0 * Config::dim, px + r0 * Config::dim, reinterpret_cast<float32_t*>( temp_ ), w.rms_att_weight, rows );
           }
-          ops_.template matmul<Config::dim, Config::dim>( pq + r0 * Config::dim, pxb + r0 * Config::dim, w.wq, rows );
-          ops_.template matmul<Config::dim, Config::kv_dim * 2>( pkv + r0 * Config::kv_dim * 2, pxb + r0 * Config::dim, w.wkv, rows );
+          if ( w.wkv == w.wq + (uint64_t)Config::dim * Config::dim ) { // wkv lies behind wq: one launch for the two products
+            ops_.template matmul_pair<Config::dim, Config::dim, Config::kv_dim * 2>( pq + r0 * Config::dim, pkv + r0 * Config::kv_dim * 2, pxb + r0 * Config::dim,
+                                                                                      w.wq, rows );
+          } else {
+            ops_.template matmul<Config::dim, Config::dim>( pq + r0 * Config::dim, pxb + r0 * Config::dim, w.wq, rows );
+            ops_.template matmul<Config::dim, Config::kv_dim * 2>( pkv + r0 * Config::kv_dim * 2, pxb + r0 * Config::dim, w.wkv, rows );
+          }
           GLINT_GH( gh_kv_append( pf_token_rows() + r0, pkv + r0 * Config::kv_dim * 2, rows, Config::kv_dim, hip::gh_type<DType>(), ops_.stream() ) );
           GLINT_GH( gh_rope( rows, pf_pos() + r0, base_.freq_cis_real, base_.freq_cis_imag, pq + r0 * Config::dim, pf_token_rows() + r0, Config::n_kv_heads,
                              Config::gqa_size, Config::head_size, hip::gh_type<DType>(), ops_.stream() ) );

@@ -99,6 +99,18 @@ def matmul(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None)
     return out
 
 
+def matmul_pair(x: torch.Tensor, w: torch.Tensor, rows_first: int):
+    """(x @ w[:rows_first].T, x @ w[rows_first:].T): two products that share their activations."""
+    b, s = x.shape
+    r, s2 = w.shape
+    assert s == s2 and 0 < rows_first < r and w.is_contiguous()
+    out_a = torch.empty((b, rows_first), dtype=x.dtype, device=x.device)
+    out_b = torch.empty((b, r - rows_first), dtype=x.dtype, device=x.device)
+    check(lib().gh_matmul_pair(_p(out_a), _p(out_b), _p(x), _p(w), s, rows_first, r - rows_first, b, _dt(x), _stream()),
+          "gh_matmul_pair")
+    return out_a, out_b
+
+
 def matmul_accum(residual: torch.Tensor, x: torch.Tensor, w: torch.Tensor, norm_weight: Optional[torch.Tensor] = None):
     """residual += x @ w.T; returns rmsnorm(residual) * norm_weight when a weight is given."""
     b, s = x.shape

@@ -153,6 +153,11 @@ int gh_matmul_fuses_many_rows( uint64_t s, uint64_t r, uint64_t b, gh_dtype dt )
  * units before initialisation): number of K ranges, k per range (a multiple of 256), weight rows per work-group */
 int gh_gemm_stream_plan( uint64_t s, uint64_t r, uint64_t b, uint32_t* splits, uint32_t* k_per_split, uint32_t* rows_per_workgroup );
 int gh_matmul( void* xout, const void* x, const void* w, uint64_t s, uint64_t r, uint64_t b, gh_dtype dt, gh_stream stream );
+/* Two products that share their activations, their weights one behind the other ((r_a + r_b, s) row-major, as the reference lays out
+ * wq and wkv, models/llama2/base.hh:410-433): xout_a = x . w[0:r_a]^T (b, r_a), xout_b = x . w[r_a:]^T (b, r_b).  The same results as
+ * two gh_matmul calls; with many rows one launch serves both, so that a narrow product does not leave the chip idle. */
+int gh_matmul_pair( void* xout_a, void* xout_b, const void* x, const void* w, uint64_t s, uint64_t r_a, uint64_t r_b, uint64_t b, gh_dtype dt,
+                    gh_stream stream );
 /* A projection fused with the ops that follow it in the reference's layer; same arithmetic and the
  * same rounding points as the separate calls (every matmul result is rounded to DType first).
  *

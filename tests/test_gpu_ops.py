@@ -285,6 +285,32 @@ def test_matmul_token_split_one_hot(b, s, r):
     assert torch.equal(got, w[:, cols].t().contiguous())
 
 
+# two products that share their activations (wq and wkv): few rows take the two-call route, many rows one launch of the large tile
+# kernel whose work-groups store to the matrix their rows belong to, also cut along the tokens; one-hot activations, bit for bit
+@pytest.mark.parametrize("dt", ["f16", "f32"])
+@pytest.mark.parametrize("b,s,ra,rb", [(3, 256, 64, 32), (300, 512, 512, 200), (2048, 256, 8192, 2048), (2300, 256, 8192, 2048),
+                                       (1500, 320, 5120, 10240), (1024, 256, 8200, 2056), (1024, 256, 8196, 2052)])
+def test_matmul_pair(dt, b, s, ra, rb):
+    if dt == "f32" and b > 300:
+        pytest.skip("the fp32 route is the same two calls at every size")
+    tdt = torch.float16 if dt == "f16" else torch.float32
+    w = torch.arange((ra + rb) * s, dtype=torch.float32, device="cuda").reshape(ra + rb, s).remainder(1000).to(tdt)
+    x = torch.zeros((b, s), dtype=tdt, device="cuda")
+    cols = torch.tensor([(7919 * i + 3) % s for i in range(b)], device="cuda")
+    x[torch.arange(b, device="cuda"), cols] = 1
+    got_a, got_b = ops.matmul_pair(x, w, ra)
+    assert got_a.shape == (b, ra) and got_b.shape == (b, rb)
+    assert torch.equal(got_a, w[:ra, cols].t().contiguous())
+    assert torch.equal(got_b, w[ra:, cols].t().contiguous())
+    g = torch.Generator(device="cuda").manual_seed(b + ra)
+    xr = torch.randn((b, s), generator=g, device="cuda").to(tdt)
+    wr = (torch.randn((ra + rb, s), generator=g, device="cuda") / s ** 0.5).to(tdt)
+    got_a, got_b = ops.matmul_pair(xr, wr, ra)
+    want = xr.float() @ wr.float().t()
+    err = (torch.cat([got_a, got_b], dim=1).float() - want).abs()
+    assert err.max().item() < 2e-2 and (err.mean() / want.abs().mean()).item() < 1e-3
+
+
 def test_matmul_layout_one_hot():
     s, r = 256, 192
     w = torch.arange(r * s, dtype=torch.float32).reshape(r, s).remainder(1000).half().cuda()
