@@ -88,7 +88,7 @@ public:
 // ---- library-owned device scratch ---------------------------------------------------------------
 // Grow-only buffer for purpose `which`, private to `stream`: work queued on different streams never
 // shares one.  Growing waits for that stream only.  `min_bytes` is the size of the first allocation.
-enum { SCRATCH_GEMM_PARTIALS = 0, SCRATCH_CONVERT = 1, SCRATCH_ATTN_PV = 2 };
+enum { SCRATCH_GEMM_PARTIALS = 0, SCRATCH_CONVERT = 1, SCRATCH_ATTN_PV = 2, SCRATCH_GATE_FACTOR = 3 };
 int stream_scratch( hipStream_t stream, int which, uint64_t bytes, uint64_t min_bytes, void** out );
 
 // Three events per sampled attention call when the benchmark's timer is enabled (slot == -1: off):

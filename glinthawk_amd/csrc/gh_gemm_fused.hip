@@ -12,6 +12,7 @@ int gemm_partials( void* xout, const void* x, const void* w, uint64_t s, uint64_
                    float** partial_out, uint32_t* splits_out );
 int gemm_gate_one_launch( void* hb, const void* x, const void* w13, uint64_t s, uint64_t hidden, uint64_t b, gh_dtype dt, hipStream_t st, bool* done );
 uint64_t gemm_token_split( uint64_t s, uint64_t r, uint64_t b, gh_dtype dt, const void* x, const void* w, const void* xout );
+bool gemm_tile_epilogue_applicable( uint64_t s, uint64_t r, uint64_t b, gh_dtype dt, const void* x, const void* w, const void* xout );
 int gemm_tile_epilogue_launch( void* xout, const void* x, const void* w, uint64_t s, uint64_t r, uint64_t b, gh_dtype dt, int epilogue, hipStream_t st,
                                bool* done );
 
@@ -361,6 +362,21 @@ int gh_matmul_silu_gate( void* hb, const void* x, const void* w13, uint64_t s, u
   }
   if ( done ) {
     return GH_OK;
+  }
+  // Some hundred rows and more with enough tiles for the large tile kernel: both factors in one launch of it, stored as DType whole
+  // row segments (the second factor into a scratch buffer), then the gate as the element-wise kernel.  The fp32 sums that the
+  // route below leaves for its gate kernel are stored from the accumulator registers, 16 bytes to each of 32 lines per
+  // instruction, and are twice the bytes: at 256 rows of the 70B shape 277 + 19 us against 257 + 12.  Same roundings either way
+  // (each factor to DType, then the gate).
+  if ( dt == GH_F16 && hidden_dim % 8 == 0 && gemm_tile_epilogue_applicable( s, 2 * hidden_dim, b, dt, x, w13, hb ) ) {
+    void* factor = nullptr;
+    if ( int rc = stream_scratch( st, SCRATCH_GATE_FACTOR, b * hidden_dim * sizeof( __half ), 16ull << 20, &factor ) ) {
+      return rc;
+    }
+    if ( int rc = gh_matmul_pair( hb, factor, x, w13, s, hidden_dim, hidden_dim, b, dt, stream ) ) {
+      return rc;
+    }
+    return gh_silu( hb, factor, hidden_dim, b, dt, stream );
   }
   float* partial = nullptr;
   uint32_t splits = 0;
