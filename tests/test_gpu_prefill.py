@@ -238,39 +238,46 @@ def test_stage_prefill_middle_stage_and_chunks():
 
 
 def test_stage_prefill_copies_overlapped_with_compute_equal_plain_call():
-    """From 8192 tokens on, a prefill that takes activations from the host and returns them cuts the rows into four runs whose
-    copies overlap the first and the last row-wise products.  Same contexts in one such call (4 x 2048 tokens) and in two plain
-    calls (2 x 2048 each): the outputs and the cache rows agree (the products of the runs may be split differently, so to rounding)."""
+    """From 8192 tokens on, a prefill that takes activations from the host cuts the rows into four runs whose copies overlap the
+    first and the last row-wise products.  Same contexts in one such call (4 x 2048 tokens) and in two plain calls (2 x 2048
+    each): the outputs and the cache rows agree (the products of the runs may be split differently, so to rounding).  Then a
+    second chunk of 2048 tokens per context from position 2048 on, without activations out (only the upload is cut into runs)."""
     first, hosted, batch, T = 8, 2, 4, 2048
-    a = S.Stage("llama2-7b", "f16", first, hosted, batch, batch, seed=3, weight_std=0.02)
-    b = S.Stage("llama2-7b", "f16", first, hosted, batch, batch, seed=3, weight_std=0.02)
-    dim, kv_dim = 4096, 4096
+    a = S.Stage("llama2-13b-4k", "f16", first, hosted, batch, batch, seed=3, weight_std=0.02)
+    b = S.Stage("llama2-13b-4k", "f16", first, hosted, batch, batch, seed=3, weight_std=0.02)
+    dim, kv_dim = 5120, 5120
     rng = np.random.default_rng(5)
-    x = ops.pinned_empty((batch * T, dim), np.float16)
-    x[:] = rng.standard_normal(x.shape).astype(np.float16)
     ids = [40 + i for i in range(batch)]
+    x = ops.pinned_empty((batch * T, dim), np.float16)
     ya = ops.pinned_empty((batch * T, dim), np.float16)
-    ya[:] = 0
-    res = a.prefill(ids, [0] * batch, T, first, activations=x, out=ya)
-    assert res is not None and res[0] is ya
-    yb = np.zeros((batch * T, dim), np.float16)
-    for half in range(2):
-        rows = slice(half * 2 * T, (half + 1) * 2 * T)
-        res = b.prefill(ids[2 * half:2 * half + 2], [0, 0], T, first, activations=x[rows], out=yb[rows])
-        assert res is not None
+
+    def both(start, want_out):
+        x[:] = rng.standard_normal(x.shape).astype(np.float16)
+        ya[:] = 0
+        res = a.prefill(ids, [start] * batch, T, first, activations=x, out=ya if want_out else None, want_activations=want_out)
+        assert res is not None and (res[0] is ya) == want_out
+        yb = np.zeros((batch * T, dim), np.float16)
+        for half in range(2):
+            rows = slice(half * 2 * T, (half + 1) * 2 * T)
+            res = b.prefill(ids[2 * half:2 * half + 2], [start, start], T, first, activations=x[rows], out=yb[rows])
+            assert res is not None
+        return yb
+
+    yb = both(0, True)
     assert np.all(np.isfinite(ya.astype(np.float32)))
-    fa, fb = ya.astype(np.float32), yb.astype(np.float32)
     assert (ya.view(np.uint16) != yb.view(np.uint16)).mean() < 0.05
-    np.testing.assert_allclose(fa, fb, rtol=4e-3, atol=4e-3)
+    np.testing.assert_allclose(ya.astype(np.float32), yb.astype(np.float32), rtol=4e-3, atol=4e-3)
+    both(T, False)
     # the caches: decoding can continue from either
     for st in (a, b):
         st.new_state(batch, next_layer=first)
-        st.set_prompts(ids, [1] * batch, [T] * batch)
+        st.set_prompts(ids, [1] * batch, [2 * T] * batch)
         assert st.acquire_contexts()
     for i in (0, 3):
         for l in (first, first + hosted - 1):
-            ka = d2h(a.context_layer_ptr(i, l), (T, 2 * kv_dim), np.float16)
-            kb = d2h(b.context_layer_ptr(i, l), (T, 2 * kv_dim), np.float16)
+            ka = d2h(a.context_layer_ptr(i, l), (2 * T, 2 * kv_dim), np.float16)
+            kb = d2h(b.context_layer_ptr(i, l), (2 * T, 2 * kv_dim), np.float16)
+            assert np.all(np.isfinite(ka.astype(np.float32)))
             assert (ka.view(np.uint16) != kb.view(np.uint16)).mean() < 0.05
             np.testing.assert_allclose(ka.astype(np.float32), kb.astype(np.float32), rtol=4e-3, atol=4e-3)
     a.close()
