@@ -654,6 +654,43 @@ def test_fused_properties_uniform_values_and_single_key():
         assert torch.allclose(xb.float(), want.expand(batch, -1), atol=2e-3, rtol=2e-3)
 
 
+@pytest.mark.parametrize("variant", [GH_ATTN_MFMA, GH_ATTN_VALU, GH_ATTN_GENERIC], ids=["mfma", "valu", "generic"])
+def test_fused_max_pos_below_the_true_maximum_truncates(variant):
+    """`max_pos` is the caller's upper bound of the positions; the split plan and the workspace follow from it.  A bound below
+    the true maximum must not take a kernel outside the workspace or into another head's partial sums: the result is the
+    attention over the first max_splits * tokens_per_split keys, and the bytes behind the workspace stay as they were."""
+    import ctypes as C
+    from glinthawk_amd import _lib
+    shape = GQA8
+    batch, bound = 5, 199
+    arena = Arena(shape, batch, torch.float16, seed=77)
+    rows = ops.row_table([arena.layer_ptr(i) for i in range(batch)])
+    q = torch.randn((batch, shape.dim), dtype=torch.float16, device="cuda")
+    true_pos = [650, 10, 699, 199, 400]
+    s = shape.c()
+    chunk, splits, need = C.c_uint32(), C.c_uint32(), C.c_uint64()
+    ops.attn_set_chunk(64)                       # several splits even at this small bound
+    try:
+        _lib.check(_lib.lib().gh_attn_decode_plan(batch, bound, C.byref(s), _lib.GH_F16, variant, C.byref(chunk), C.byref(splits), C.byref(need)))
+        covered = chunk.value * splits.value
+        assert splits.value > 1 and bound < covered < max(true_pos)
+        ws_bytes = ops.attn_decode_workspace(batch, bound, shape)
+        guard = 1 << 16
+        buf = torch.full((ws_bytes + guard,), 0x5A, dtype=torch.uint8, device="cuda")
+        got = torch.zeros_like(q)
+        ops.attn_decode(q, rows, torch.tensor(true_pos, dtype=torch.int32, device="cuda"), got, bound, shape,
+                        workspace=buf[:ws_bytes], variant=variant)
+        torch.cuda.synchronize()
+        assert torch.all(buf[ws_bytes:] == 0x5A)
+        assert torch.isfinite(got).all()
+        want = torch.zeros_like(q)
+        clamped = [min(p, covered - 1) for p in true_pos]
+        ops.attn_decode(q, rows, torch.tensor(clamped, dtype=torch.int32, device="cuda"), want, max(clamped), shape, variant=variant)
+    finally:
+        ops.attn_set_chunk(0)
+    assert torch.allclose(got.float(), want.float(), atol=2e-3, rtol=2e-3)
+
+
 def test_fused_rejects_bad_arguments():
     shape = GQA8
     q = torch.zeros((1, shape.dim), dtype=torch.float16, device="cuda")
