@@ -325,15 +325,21 @@ __global__ __launch_bounds__( 256, NQT == 1 ? 2 : 1 ) void attn_prefill_mfma_ker
     float ms[NQT];
 #pragma unroll
     for ( int qt = 0; qt < NQT; qt++ ) {
-      float mx = st[qt][0][0];
+      // four independent chains (one long chain of dependent maxima costs its latency sixteen times), then the other half of the
+      // column's keys from the lane 32 further on: v_permlane32_swap exchanges the two half-waves in the vector ALU, without the
+      // trip through LDS that a shuffle takes
+      float m4[4];
 #pragma unroll
-      for ( int sub = 0; sub < 2; sub++ ) {
+      for ( int c = 0; c < 4; c++ ) {
+        m4[c] = st[qt][c >> 1][8 * ( c & 1 )];
 #pragma unroll
-        for ( int v = 0; v < 16; v++ ) {
-          mx = fmaxf( mx, st[qt][sub][v] );
+        for ( int e = 1; e < 8; e++ ) {
+          m4[c] = fmaxf( m4[c], st[qt][c >> 1][8 * ( c & 1 ) + e] );
         }
       }
-      mx = fmaxf( mx, __shfl_xor( mx, 32, WAVE ) ) * scale_log2e; // log2 domain from here on
+      float mx = fmaxf( fmaxf( m4[0], m4[1] ), fmaxf( m4[2], m4[3] ) );
+      const auto halves = __builtin_amdgcn_permlane32_swap( __builtin_bit_cast( unsigned, mx ), __builtin_bit_cast( unsigned, mx ), false, false );
+      mx = fmaxf( __builtin_bit_cast( float, halves[0] ), __builtin_bit_cast( float, halves[1] ) ) * scale_log2e; // log2 domain from here on
       // The reference point of the exponentials only moves when the maximum has grown by more than 2^LAZY since it was set:
       // weights stay below 2^LAZY (fine for fp32 sums and fp16 operands) and the 64 accumulators are rescaled rarely.  The
       // result does not depend on the reference point.  -inf: a column that has seen no key yet (padding, or hidden so far).
