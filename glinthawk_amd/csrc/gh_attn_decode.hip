@@ -161,27 +161,53 @@ __global__ __launch_bounds__( 256 ) void attn_merge_kernel( Partials part,
 {
   const uint32_t head = blockIdx.x;
   const uint32_t ctx = blockIdx.y;
-  if ( layer_rows[ctx] == nullptr ) {
+  const void* const rows = layer_rows[ctx];
+  const uint32_t last = pos[ctx]; // read before the branch on `rows`: one round trip for the two
+  if ( rows == nullptr ) {
     return;
   }
   // ceil((pos + 1) / chunk); a position beyond the host's bound must not walk into the partials of the next head
-  const uint32_t n_splits = min( ( pos[ctx] + chunk ) / chunk, max_splits );
+  const uint32_t n_splits = min( ( last + chunk ) / chunk, max_splits );
   const uint64_t slot0 = ( (uint64_t)ctx * n_heads + head ) * max_splits;
-  float m = -INFINITY;
-  for ( uint32_t s = 0; s < n_splits; s++ ) {
-    m = fmaxf( m, part.ml[( slot0 + s ) * 2] );
-  }
-  float l = 0.0f;
-  for ( uint32_t s = 0; s < n_splits; s++ ) {
-    l += part.ml[( slot0 + s ) * 2 + 1] * fast_exp2( part.ml[( slot0 + s ) * 2] - m );
-  }
-  const float inv = 1.0f / l;
-  for ( uint32_t d = threadIdx.x; d < head_size; d += blockDim.x ) {
-    float acc = 0.0f;
-    for ( uint32_t s = 0; s < n_splits; s++ ) {
-      acc += part.out[( slot0 + s ) * head_size + d] * fast_exp2( part.ml[( slot0 + s ) * 2] - m );
+  const float2* ml = reinterpret_cast<const float2*>( part.ml ) + slot0; // (maximum, sum) of a split
+  // The first MERGE_BATCH splits, nearly always all of them: every load issued before the first use (a split past the last reads
+  // the last again and gets weight zero), so the kernel is one memory round trip deep.  Splits beyond that, one at a time.
+  constexpr uint32_t MERGE_BATCH = 8;
+  for ( uint32_t d0 = 0; d0 < head_size; d0 += blockDim.x ) {
+    const uint32_t d = d0 + threadIdx.x;
+    const uint32_t dl = min( d, head_size - 1 );
+    float2 st[MERGE_BATCH];
+    float o[MERGE_BATCH];
+#pragma unroll
+    for ( uint32_t u = 0; u < MERGE_BATCH; u++ ) {
+      const uint32_t sp = min( u, n_splits - 1 );
+      st[u] = ml[sp];
+      o[u] = part.out[( slot0 + sp ) * head_size + dl];
     }
-    xb[( (uint64_t)ctx * n_heads + head ) * head_size + d] = from_f32<T>( acc * inv );
+    float m = -INFINITY;
+#pragma unroll
+    for ( uint32_t u = 0; u < MERGE_BATCH; u++ ) {
+      m = fmaxf( m, st[u].x ); // a repeated split repeats a value that is in the set already
+    }
+    for ( uint32_t sp = MERGE_BATCH; sp < n_splits; sp++ ) {
+      m = fmaxf( m, ml[sp].x );
+    }
+    float l = 0.0f, acc = 0.0f;
+#pragma unroll
+    for ( uint32_t u = 0; u < MERGE_BATCH; u++ ) {
+      const float wgt = u < n_splits ? fast_exp2( st[u].x - m ) : 0.0f;
+      l += st[u].y * wgt;
+      acc += o[u] * wgt;
+    }
+    for ( uint32_t sp = MERGE_BATCH; sp < n_splits; sp++ ) {
+      const float2 e = ml[sp];
+      const float wgt = fast_exp2( e.x - m );
+      l += e.y * wgt;
+      acc += part.out[( slot0 + sp ) * head_size + dl] * wgt;
+    }
+    if ( d < head_size ) {
+      xb[( (uint64_t)ctx * n_heads + head ) * head_size + d] = from_f32<T>( acc * ( 1.0f / l ) );
+    }
   }
 }
 

@@ -50,32 +50,6 @@ __device__ __forceinline__ WaveJob wave_job( const __half* const* layer_rows,
   return j;
 }
 
-__device__ __forceinline__ float dpp_quad_xor1( float v )
-{
-  return __builtin_bit_cast( float, __builtin_amdgcn_update_dpp( 0, __builtin_bit_cast( int, v ), 0xB1, 0xF, 0xF, true ) );
-}
-__device__ __forceinline__ float dpp_quad_xor2( float v )
-{
-  return __builtin_bit_cast( float, __builtin_amdgcn_update_dpp( 0, __builtin_bit_cast( int, v ), 0x4E, 0xF, 0xF, true ) );
-}
-__device__ __forceinline__ float dpp_half_mirror( float v )
-{
-  return __builtin_bit_cast( float, __builtin_amdgcn_update_dpp( 0, __builtin_bit_cast( int, v ), 0x141, 0xF, 0xF, true ) );
-}
-__device__ __forceinline__ float dpp_row_mirror( float v )
-{
-  return __builtin_bit_cast( float, __builtin_amdgcn_update_dpp( 0, __builtin_bit_cast( int, v ), 0x140, 0xF, 0xF, true ) );
-}
-// sum over the 16 lanes of a DPP row; every lane of the row gets the total
-__device__ __forceinline__ float row16_sum( float v )
-{
-  v += dpp_quad_xor1( v );
-  v += dpp_quad_xor2( v );
-  v += dpp_half_mirror( v );
-  v += dpp_row_mirror( v );
-  return v;
-}
-
 // Cache rows are reached through pointers that come out of a table, so the compiler cannot tell that they are global memory
 // and would use flat loads.  Those count against the LDS wait counter as well: a wait for an LDS read would then also wait for
 // the rows of the next tile, which are meant to stay in flight.  The casts below name the address space.

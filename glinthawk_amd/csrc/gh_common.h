@@ -101,22 +101,58 @@ constexpr uint64_t MAX_BATCH = 1024;           // models/llama2/base.hh:26
 // ---- device helpers ---------------------------------------------------------------------------
 constexpr int WAVE = 64;
 
+__device__ __forceinline__ float dpp_quad_xor1( float v )
+{
+  return __builtin_bit_cast( float, __builtin_amdgcn_update_dpp( 0, __builtin_bit_cast( int, v ), 0xB1, 0xF, 0xF, true ) );
+}
+__device__ __forceinline__ float dpp_quad_xor2( float v )
+{
+  return __builtin_bit_cast( float, __builtin_amdgcn_update_dpp( 0, __builtin_bit_cast( int, v ), 0x4E, 0xF, 0xF, true ) );
+}
+__device__ __forceinline__ float dpp_half_mirror( float v )
+{
+  return __builtin_bit_cast( float, __builtin_amdgcn_update_dpp( 0, __builtin_bit_cast( int, v ), 0x141, 0xF, 0xF, true ) );
+}
+__device__ __forceinline__ float dpp_row_mirror( float v )
+{
+  return __builtin_bit_cast( float, __builtin_amdgcn_update_dpp( 0, __builtin_bit_cast( int, v ), 0x140, 0xF, 0xF, true ) );
+}
+// sum over the 16 lanes of a DPP row; every lane of the row gets the total
+__device__ __forceinline__ float row16_sum( float v )
+{
+  v += dpp_quad_xor1( v );
+  v += dpp_quad_xor2( v );
+  v += dpp_half_mirror( v );
+  v += dpp_row_mirror( v );
+  return v;
+}
+
+__device__ __forceinline__ float row16_max( float v )
+{
+  v = fmaxf( v, dpp_quad_xor1( v ) );
+  v = fmaxf( v, dpp_quad_xor2( v ) );
+  v = fmaxf( v, dpp_half_mirror( v ) );
+  v = fmaxf( v, dpp_row_mirror( v ) );
+  return v;
+}
+__device__ __forceinline__ float lane_value( float v, int lane )
+{
+  return __builtin_bit_cast( float, __builtin_amdgcn_readlane( __builtin_bit_cast( int, v ), lane ) );
+}
+
+// Reductions over the wave, the result in every lane: within each row of 16 lanes by DPP, whose operand arrives with the
+// instruction, then the four rows by lane reads.  A butterfly of lane exchanges goes through the LDS crossbar six times, a round
+// trip each.
 __device__ __forceinline__ float wave_sum( float v )
 {
-#pragma unroll
-  for ( int off = 32; off > 0; off >>= 1 ) {
-    v += __shfl_xor( v, off, WAVE );
-  }
-  return v;
+  v = row16_sum( v );
+  return ( lane_value( v, 0 ) + lane_value( v, 16 ) ) + ( lane_value( v, 32 ) + lane_value( v, 48 ) );
 }
 
 __device__ __forceinline__ float wave_max( float v )
 {
-#pragma unroll
-  for ( int off = 32; off > 0; off >>= 1 ) {
-    v = fmaxf( v, __shfl_xor( v, off, WAVE ) );
-  }
-  return v;
+  v = row16_max( v );
+  return fmaxf( fmaxf( lane_value( v, 0 ), lane_value( v, 16 ) ), fmaxf( lane_value( v, 32 ), lane_value( v, 48 ) ) );
 }
 
 template<typename T>

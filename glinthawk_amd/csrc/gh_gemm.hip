@@ -192,9 +192,18 @@ __global__ __launch_bounds__( 256 ) void gemm_reduce_kernel( __half* __restrict_
 {
   const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
   for ( uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride ) {
+    // ascending order of the split, four loads in flight: a split past the last reads the last again and is not added
     float sum = 0.0f;
-    for ( uint32_t k = 0; k < splits; k++ ) {
-      sum += partial[(uint64_t)k * n + i];
+    for ( uint32_t k0 = 0; k0 < splits; k0 += 4 ) {
+      float p[4];
+#pragma unroll
+      for ( uint32_t u = 0; u < 4; u++ ) {
+        p[u] = partial[(uint64_t)min( k0 + u, splits - 1 ) * n + i];
+      }
+#pragma unroll
+      for ( uint32_t u = 0; u < 4; u++ ) {
+        sum += k0 + u < splits ? p[u] : 0.0f;
+      }
     }
     xout[i] = __float2half_rn( sum );
   }

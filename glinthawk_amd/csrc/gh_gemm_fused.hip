@@ -18,11 +18,40 @@ int gemm_tile_epilogue_launch( void* xout, const void* x, const void* w, uint64_
 
 namespace {
 
+// Sum over the splits in ascending order, four loads in flight at a time: a split past the last reads the last again and is not
+// added, so no load sits under a branch (a load under a branch is waited for before the next is issued).
+constexpr uint32_t SPLIT_BATCH = 4;
 __device__ __forceinline__ float sum_splits( const float* __restrict__ partial, uint64_t idx, uint64_t n, uint32_t splits )
 {
   float acc = 0.0f;
-  for ( uint32_t k = 0; k < splits; k++ ) {
-    acc += partial[(uint64_t)k * n + idx];
+  for ( uint32_t k0 = 0; k0 < splits; k0 += SPLIT_BATCH ) {
+    float p[SPLIT_BATCH];
+#pragma unroll
+    for ( uint32_t u = 0; u < SPLIT_BATCH; u++ ) {
+      p[u] = partial[(uint64_t)min( k0 + u, splits - 1 ) * n + idx];
+    }
+#pragma unroll
+    for ( uint32_t u = 0; u < SPLIT_BATCH; u++ ) {
+      acc += k0 + u < splits ? p[u] : 0.0f;
+    }
+  }
+  return acc;
+}
+// two neighbouring columns, idx even and the partials 8-byte aligned
+__device__ __forceinline__ float2 sum_splits2( const float* __restrict__ partial, uint64_t idx, uint64_t n, uint32_t splits )
+{
+  float2 acc = make_float2( 0.0f, 0.0f );
+  for ( uint32_t k0 = 0; k0 < splits; k0 += SPLIT_BATCH ) {
+    float2 p[SPLIT_BATCH];
+#pragma unroll
+    for ( uint32_t u = 0; u < SPLIT_BATCH; u++ ) {
+      p[u] = *reinterpret_cast<const float2*>( partial + (uint64_t)min( k0 + u, splits - 1 ) * n + idx );
+    }
+#pragma unroll
+    for ( uint32_t u = 0; u < SPLIT_BATCH; u++ ) {
+      acc.x += k0 + u < splits ? p[u].x : 0.0f;
+      acc.y += k0 + u < splits ? p[u].y : 0.0f;
+    }
   }
   return acc;
 }
@@ -131,29 +160,40 @@ __global__ __launch_bounds__( EPI_THREADS ) void epi_accum_norm_row8k_kernel( __
   float4 acc[2];
   H4 old[2], nw[2];
   bool live[2];
+  uint32_t col[2];
+  // A column group past the row's end reads group 0 instead and stores nothing: loads without a branch around them can all be in
+  // flight together, loads under a branch are waited for one by one.
 #pragma unroll
   for ( int it = 0; it < 2; it++ ) {
     const uint32_t j = ( it * EPI_THREADS + threadIdx.x ) * 4;
     live[it] = j < r;
+    col[it] = live[it] ? j : 0;
     acc[it] = make_float4( 0.0f, 0.0f, 0.0f, 0.0f );
-    old[it].raw = make_uint2( 0, 0 );
-    nw[it].raw = make_uint2( 0, 0 );
-    if ( live[it] ) {
-      old[it].raw = *reinterpret_cast<const uint2*>( res + j );
-      if ( norm_out != nullptr ) {
-        nw[it].raw = *reinterpret_cast<const uint2*>( norm_weight + j );
+    old[it].raw = *reinterpret_cast<const uint2*>( res + col[it] );
+    nw[it].raw = *reinterpret_cast<const uint2*>( ( norm_out != nullptr ? norm_weight : res ) + col[it] );
+  }
+  // Partial sums four splits at a time, eight loads in flight; a split past the last reads the last again and is not added.  Added in
+  // ascending order of the split, as one at a time would.
+  constexpr uint32_t BATCH = 4;
+  for ( uint32_t k0 = 0; k0 < splits; k0 += BATCH ) {
+    float4 p[BATCH][2];
+#pragma unroll
+    for ( uint32_t u = 0; u < BATCH; u++ ) {
+      const uint32_t k = min( k0 + u, splits - 1 );
+#pragma unroll
+      for ( int it = 0; it < 2; it++ ) {
+        p[u][it] = *reinterpret_cast<const float4*>( prow + (uint64_t)k * n + col[it] );
       }
     }
-  }
-  for ( uint32_t k = 0; k < splits; k++ ) {
 #pragma unroll
-    for ( int it = 0; it < 2; it++ ) {
-      if ( live[it] ) {
-        const float4 p = *reinterpret_cast<const float4*>( prow + (uint64_t)k * n + ( it * EPI_THREADS + threadIdx.x ) * 4 );
-        acc[it].x += p.x;
-        acc[it].y += p.y;
-        acc[it].z += p.z;
-        acc[it].w += p.w;
+    for ( uint32_t u = 0; u < BATCH; u++ ) {
+      const bool use = k0 + u < splits;
+#pragma unroll
+      for ( int it = 0; it < 2; it++ ) {
+        acc[it].x += use ? p[u][it].x : 0.0f;
+        acc[it].y += use ? p[u][it].y : 0.0f;
+        acc[it].z += use ? p[u][it].z : 0.0f;
+        acc[it].w += use ? p[u][it].w : 0.0f;
       }
     }
   }
@@ -166,7 +206,7 @@ __global__ __launch_bounds__( EPI_THREADS ) void epi_accum_norm_row8k_kernel( __
 #pragma unroll
     for ( int e = 0; e < 4; e++ ) {
       o.h[e] = __float2half_rn( __half2float( old[it].h[e] ) + __half2float( __float2half_rn( y[e] ) ) ); // xb2 = DType(matmul), then accum
-      v[it][e] = __half2float( o.h[e] );
+      v[it][e] = live[it] ? __half2float( o.h[e] ) : 0.0f; // a group past the row's end holds group 0's values: not part of the norm
       ss += v[it][e] * v[it][e];
     }
     if ( live[it] ) {
@@ -240,8 +280,9 @@ __global__ __launch_bounds__( 256 ) void epi_qkv_kernel( T* __restrict__ q,
     return;
   }
   const uint32_t col = 2 * pair;
-  const T y0 = from_f32<T>( sum_splits( partial, (uint64_t)ctx * r + col, n, splits ) );
-  const T y1 = from_f32<T>( sum_splits( partial, (uint64_t)ctx * r + col + 1, n, splits ) );
+  const float2 y = sum_splits2( partial, (uint64_t)ctx * r + col, n, splits ); // r and n are even: 8-byte aligned
+  const T y0 = from_f32<T>( y.x );
+  const T y1 = from_f32<T>( y.y );
   T* row = static_cast<T*>( token_rows[ctx] );
 
   if ( kv_out != nullptr && col >= dim ) {
