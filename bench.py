@@ -14,6 +14,9 @@ Prints ONE JSON line:
   stage_*      whole stage step: tokens/s and the fraction of the bandwidth roofline, timed over K
                steps with no event between the kernels (ms_per_step); the K steps that carry the
                events run right after them and are reported as ms_per_step_with_attn_events
+  *_resident   the same step between two events, after its activations and tables are queued and before the copy
+               back: what the stage costs with its inputs resident in HBM (ms_per_step goes through the host
+               state buffers on both sides, as the reference's forward() does)
   cpu_baseline the CPU oracle (a port of the reference's fp32 OpenMP path) timed on a bounded sample:
                one hosted layer on the very weights, cache rows and activations the GPU stage ran on
   concept_path the same stage driven through the reference's own op sequence only (unfused attention
@@ -260,6 +263,14 @@ def decode_bench(workload, steps, warmup, fused=True, cpu=True, events=True):
         res.update(ms_per_step_with_events=(t3 - t2) * 1e3 / steps, attn_kernel_ms=k_ms.value / launches,
                    attn_merge_ms=m_ms.value / launches, attn_launches=int(n.value))
 
+    # pass 3: the same steps once more with two events per step, after the activations and tables are queued and before
+    # the copy back: the stage step with its inputs resident in HBM, without the host boundary on either side
+    st.time_device_spans(True)
+    for _ in range(steps):
+        one_step()
+    span_ms, spans = st.device_spans()
+    st.time_device_spans(False)
+    res.update(ms_per_step_resident=span_ms / max(1, spans))
     out = st.activations().astype(np.float32)
     assert np.all(np.isfinite(out)), "stage output is not finite"
 
@@ -320,6 +331,9 @@ def decode_line(workload, steps, warmup, attn_variant="auto", cpu=True):
         "stage_tokens_per_s": round(tokens_per_s, 1),
         "stage_roofline_frac": round(stage_roofline_ms / g["ms_per_step"], 4),
         "stage_bytes_per_step": g["stage_bytes"],
+        "ms_per_step_resident": round(g["ms_per_step_resident"], 4),
+        "stage_tokens_per_s_resident": round(batch / (g["ms_per_step_resident"] * 1e-3), 1),
+        "stage_roofline_frac_resident": round(stage_roofline_ms / g["ms_per_step_resident"], 4),
         "n_gpus": 1,
         "steps": steps,
         "warmup": warmup,

@@ -67,6 +67,8 @@ SIGNATURES = {
     "gh_stream_destroy": (_i, [_vp]),
     "gh_event_create": (_i, [C.POINTER(_vp)]),
     "gh_event_destroy": (_i, [_vp]),
+    "gh_event_create_timed": (_i, [C.POINTER(_vp)]),
+    "gh_event_elapsed_ms": (_i, [_vp, _vp, C.POINTER(C.c_float)]),
     "gh_event_record": (_i, [_vp, _vp]),
     "gh_stream_wait_event": (_i, [_vp, _vp]),
     "gh_malloc": (_i, [C.POINTER(_vp), _u64]),

@@ -331,6 +331,26 @@ int gh_event_create( gh_event* out )
   return GH_OK;
 }
 
+int gh_event_create_timed( gh_event* out )
+{
+  if ( int rc = ensure_init() ) {
+    return rc;
+  }
+  GH_REQUIRE( out != nullptr, "gh_event_create_timed: NULL output" );
+  hipEvent_t e = nullptr;
+  GH_HIP( hipEventCreate( &e ) );
+  *out = e;
+  return GH_OK;
+}
+
+int gh_event_elapsed_ms( gh_event begin, gh_event end, float* ms )
+{
+  GH_REQUIRE( begin != nullptr && end != nullptr && ms != nullptr, "gh_event_elapsed_ms: NULL argument" );
+  GH_HIP( hipEventSynchronize( static_cast<hipEvent_t>( end ) ) );
+  GH_HIP( hipEventElapsedTime( ms, static_cast<hipEvent_t>( begin ), static_cast<hipEvent_t>( end ) ) );
+  return GH_OK;
+}
+
 int gh_event_destroy( gh_event event )
 {
   GH_REQUIRE( event != nullptr, "gh_event_destroy: NULL event" );

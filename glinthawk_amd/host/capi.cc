@@ -47,6 +47,8 @@ struct StageBase
   virtual int release_context( uint32_t id ) = 0;
   virtual void paging_info( size_t row, size_t layer, uint64_t out[3] ) = 0;
   virtual void sync() = 0;
+  virtual void time_device_spans( bool on ) = 0;
+  virtual void device_spans( double* ms, uint64_t* spans ) = 0;
   virtual int prefill( uint32_t batch, const uint32_t* context_ids, const uint32_t* start_pos, uint32_t n_tokens, uint32_t first_layer,
                        const uint32_t* token_ids, const void* acts_in, void* acts_out, uint32_t* next_tokens ) = 0;
 };
@@ -232,6 +234,13 @@ struct StageImpl : StageBase
     }
   }
   void sync() override { model.ops().synchronize(); }
+  void time_device_spans( bool on ) override { model.time_device_spans( on ); }
+  void device_spans( double* ms, uint64_t* spans ) override
+  {
+    const auto [total, n] = model.device_spans();
+    *ms = total;
+    *spans = n;
+  }
 
   int prefill( uint32_t batch, const uint32_t* context_ids, const uint32_t* start_pos, uint32_t n_tokens, uint32_t first_layer, const uint32_t* token_ids,
                const void* acts_in, void* acts_out, uint32_t* next_tokens ) override
@@ -550,6 +559,9 @@ int glint_stage_release_context( void* h, uint32_t id ) { return static_cast<Sta
 void glint_stage_paging_info( void* h, uint32_t row, uint32_t layer, uint64_t out[3] ) { static_cast<StageBase*>( h )->paging_info( row, layer, out ); }
 void* glint_stage_scratch( void* h, int which ) { return static_cast<StageBase*>( h )->scratch( which ); }
 void glint_stage_sync( void* h ) { static_cast<StageBase*>( h )->sync(); }
+// device time of forward() without the copies over the host boundary: on / off, then total milliseconds and steps since the last read
+void glint_stage_time_device_spans( void* h, int on ) { static_cast<StageBase*>( h )->time_device_spans( on != 0 ); }
+void glint_stage_device_spans( void* h, double* ms, uint64_t* spans ) { static_cast<StageBase*>( h )->device_spans( ms, spans ); }
 // batched prefill of n_tokens tokens per context; -1 when the contexts cannot be served
 int glint_stage_prefill( void* h, uint32_t batch, const uint32_t* context_ids, const uint32_t* start_pos, uint32_t n_tokens, uint32_t first_layer,
                          const uint32_t* token_ids, const void* acts_in, void* acts_out, uint32_t* next_tokens )

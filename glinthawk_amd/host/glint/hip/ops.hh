@@ -87,7 +87,14 @@ public:
   // all work is queued on this stream (NULL = the default stream)
   void set_stream( gh_stream s ) { stream_ = s; }
   gh_stream stream() const { return stream_; }
-  void synchronize() const { GLINT_GH( gh_sync( stream_ ) ); }
+  void synchronize() const
+  {
+    GLINT_GH( gh_sync( stream_ ) );
+    drains_++;
+  }
+  // how often the stream has been waited for until it was empty (synchronize(), blocking copies): work queued before the last
+  // of them has finished
+  uint64_t drain_count() const { return drains_; }
 
   template<uint64_t size>
   void accum( DType* a, const DType* b, const uint64_t batch_size ) const
@@ -146,6 +153,9 @@ public:
   void copy( DType* dst, const DType* src, const uint64_t len_bytes, const CopyType type, const bool async = false ) const
   {
     GLINT_GH( gh_memcpy( dst, src, len_bytes, gh_kind( type ), async ? 1 : 0, stream_ ) );
+    if ( !async ) {
+      drains_++;
+    }
   }
 
   void print( const DType* x, const uint64_t b, const std::string base ) const
@@ -161,6 +171,7 @@ public:
 
 protected:
   gh_stream stream_ { nullptr };
+  mutable uint64_t drains_ { 0 };
   mutable uint64_t sample_seed_ { 0x5eed };
   mutable uint64_t fill_seed_ { 0xf111 };
 };

@@ -173,6 +173,25 @@ public:
 
   const SettingsType& settings() const { return settings_; }
   LlamaOperations& ops() { return ops_; }
+  // device time of forward() (see SpanTimer): switch it on or off, read the accumulated milliseconds and steps, which a read resets
+  void time_device_spans( const bool on )
+  {
+    if ( on && !span_timer_ ) {
+      span_timer_ = std::make_unique<SpanTimer>();
+    } else if ( !on ) {
+      span_timer_.reset();
+    }
+  }
+  std::pair<double, uint64_t> device_spans()
+  {
+    std::pair<double, uint64_t> out { 0.0, 0 };
+    if ( span_timer_ ) {
+      out = { span_timer_->total_ms, span_timer_->spans };
+      span_timer_->total_ms = 0;
+      span_timer_->spans = 0;
+    }
+    return out;
+  }
   const BaseWeights<DType>& base_weights() const { return base_; }
   const LayerWeights<DType>& layer_weights( size_t l ) const { return layers_[l]; }
 
@@ -227,6 +246,7 @@ public:
       upload_tables( contexts, run );
     }
 
+    mark_device_span( 0 ); // the activations and the tables are queued: from here to the copy back it is kernels only
     const bool fused_layers = options_.fused_attention && options_.fused_projections;
     if ( fused_layers && !run.empty() ) {
       // the first attention norm stands alone; every later one rides on the epilogue of the previous w2
@@ -253,10 +273,13 @@ public:
 
     if ( last == Config::n_layers - 1 && settings_.hosts( last, InferenceStage::Classification ) ) {
       classify_ops();
+      mark_device_span( 1 );
       postlude( states, last, true );
     } else {
+      mark_device_span( 1 );
       postlude( states, last, false );
     }
+    close_device_span();
   }
 
   // ------------------------------------------------------------------------------------------
@@ -728,9 +751,12 @@ private:
 
   void upload_tables( const ContextVector& contexts, const std::vector<size_t>& run )
   {
-    // the previous step's upload was consumed by kernels queued before this point on the same
-    // stream; wait for them before the pinned buffer is rewritten
-    ops_.synchronize();
+    // The previous upload reads the pinned buffer asynchronously: it has to be over before the buffer is rewritten.  A step
+    // ends with a blocking copy of its results, which is such a wait already; only without one since the last upload is
+    // the stream waited for here (that wait would also sit out the copy of this step's activations, queued just before).
+    if ( tables_uploaded_ && ops_.drain_count() == tables_drain_count_ ) {
+      ops_.synchronize();
+    }
     auto* pos = reinterpret_cast<uint32_t*>( tables_host_ );
     auto** ptrs = reinterpret_cast<void**>( ptr_tables( tables_host_ ) );
     max_pos_ = 0;
@@ -750,6 +776,8 @@ private:
     }
     const size_t bytes = ( ptr_tables( tables_host_ ) - tables_host_ ) + run.size() * 2 * table_stride() * sizeof( void* );
     GLINT_GH( gh_memcpy( tables_dev_.get(), tables_host_, bytes, GH_HOST_TO_DEVICE, 1, ops_.stream() ) );
+    tables_uploaded_ = true;
+    tables_drain_count_ = ops_.drain_count();
   }
 
   // ---- allocation ----------------------------------------------------------------------------
@@ -947,6 +975,44 @@ private:
     CopyLane( const CopyLane& ) = delete;
     CopyLane& operator=( const CopyLane& ) = delete;
   };
+  // Device time of forward(): the span on the stream from the first kernel of a step to its last, without the copies of the
+  // state over the host boundary on either side.  Off by default; two event records per step when on.
+  struct SpanTimer
+  {
+    gh_event mark[2] {};
+    double total_ms { 0 };
+    uint64_t spans { 0 };
+    bool open { false };
+    SpanTimer()
+    {
+      GLINT_GH( gh_event_create_timed( &mark[0] ) );
+      GLINT_GH( gh_event_create_timed( &mark[1] ) );
+    }
+    ~SpanTimer()
+    {
+      (void)gh_event_destroy( mark[0] );
+      (void)gh_event_destroy( mark[1] );
+    }
+    SpanTimer( const SpanTimer& ) = delete;
+    SpanTimer& operator=( const SpanTimer& ) = delete;
+  };
+  void mark_device_span( const int which )
+  {
+    if ( span_timer_ ) {
+      GLINT_GH( gh_event_record( span_timer_->mark[which], ops_.stream() ) );
+      span_timer_->open = which == 1;
+    }
+  }
+  void close_device_span()
+  {
+    if ( span_timer_ && span_timer_->open ) {
+      float ms = 0;
+      GLINT_GH( gh_event_elapsed_ms( span_timer_->mark[0], span_timer_->mark[1], &ms ) );
+      span_timer_->total_ms += ms;
+      span_timer_->spans++;
+      span_timer_->open = false;
+    }
+  }
   void ensure_copy_stream()
   {
     if ( !copy_lane_ ) {
@@ -960,8 +1026,11 @@ private:
   DevicePtr pf_x_ {}, pf_xb_ {}, pf_q_ {}, pf_hb_ {}, pf_hb2_ {}, pf_xb2_ {}, pf_kv_ {}, pf_tables_ {}, pf_attn_ws_ {};
   uint64_t pf_capacity_ { 0 }, pf_attn_ws_bytes_ { 0 };
   std::unique_ptr<CopyLane> copy_lane_ {};
+  std::unique_ptr<SpanTimer> span_timer_ {};
   uint64_t attn_ws_bytes_ { 0 };
   uint8_t* tables_host_ { nullptr };
+  bool tables_uploaded_ { false };
+  uint64_t tables_drain_count_ { 0 };
   BaseWeights<DType> base_ {};
   std::vector<LayerWeights<DType>> layers_ {};
 

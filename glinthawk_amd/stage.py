@@ -61,6 +61,8 @@ def host_lib() -> C.CDLL:
             "glint_stage_paging_info": (None, [vp, u32, u32, C.POINTER(u64)]),
             "glint_stage_scratch": (vp, [vp, C.c_int]),
             "glint_stage_sync": (None, [vp]),
+            "glint_stage_time_device_spans": (None, [vp, C.c_int]),
+            "glint_stage_device_spans": (None, [vp, C.POINTER(C.c_double), C.POINTER(u64)]),
             "glint_stage_prefill": (C.c_int, [vp, u32, vp, vp, u32, u32, vp, vp, vp, vp]),
             "glint_stage_load": (C.c_int, [vp, C.c_char_p]),
             "glint_last_error": (C.c_char_p, []),
@@ -250,6 +252,16 @@ class Stage:
 
     def sync(self) -> None:
         host_lib().glint_stage_sync(self._h)
+
+    def time_device_spans(self, on: bool) -> None:
+        """Times forward() on the device, first kernel to last, without the copies of the state over the host boundary."""
+        host_lib().glint_stage_time_device_spans(self._h, int(on))
+
+    def device_spans(self):
+        """(milliseconds, steps) accumulated since the last read."""
+        ms, n = C.c_double(0), C.c_uint64(0)
+        host_lib().glint_stage_device_spans(self._h, C.byref(ms), C.byref(n))
+        return ms.value, int(n.value)
 
     def prefill(self, context_ids, start_pos, n_tokens: int, first_layer: int = 0, token_ids=None, activations=None,
                 want_activations: bool = True, want_next_tokens: bool = False, out=None):

@@ -93,6 +93,11 @@ int gh_event_create( gh_event* out );
 int gh_event_destroy( gh_event event );
 int gh_event_record( gh_event event, gh_stream stream );
 int gh_stream_wait_event( gh_stream stream, gh_event event );
+/* Measurement support (the reference times whole calls with steady_clock, profiler.hh:153-192; on a device whose calls are
+ * asynchronous the span between two points of a stream takes events): an event that keeps its time stamp, and the milliseconds
+ * between two such events.  gh_event_elapsed_ms waits for `end`. */
+int gh_event_create_timed( gh_event* out );
+int gh_event_elapsed_ms( gh_event begin, gh_event end, float* ms );
 
 /* Operations::device_allocate / DeviceUniquePtr deleter (arch/cuda/common/ops.cuh:27-35,748-756) */
 int gh_malloc( void** out, uint64_t bytes );
