@@ -778,3 +778,34 @@ def test_streams_and_events_order_a_copy_before_a_kernel():
         assert call() == -1
     _lib.check(L.gh_event_destroy(event))
     _lib.check(L.gh_stream_destroy(stream))
+
+
+@pytest.mark.gpu
+def test_timed_events_bracket_the_work_between_them():
+    import ctypes as C
+    import time
+    from glinthawk_amd import _lib
+    L = _lib.lib()
+    e0, e1 = C.c_void_p(), C.c_void_p()
+    _lib.check(L.gh_event_create_timed(C.byref(e0)))
+    _lib.check(L.gh_event_create_timed(C.byref(e1)))
+    n = 1 << 26
+    a = torch.zeros(n, dtype=torch.float16, device="cuda")
+    b = torch.ones(n, dtype=torch.float16, device="cuda")
+    _lib.check(L.gh_sync(None))
+    t0 = time.perf_counter()
+    _lib.check(L.gh_event_record(e0, None))
+    for _ in range(20):
+        _lib.check(L.gh_accum(a.data_ptr(), b.data_ptr(), n, 1, _lib.GH_F16, None))
+    _lib.check(L.gh_event_record(e1, None))
+    ms = C.c_float(-1)
+    _lib.check(L.gh_event_elapsed_ms(e0, e1, C.byref(ms)))  # waits for the second event
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    assert torch.all(a.cpu() == 20)
+    # 20 passes over 384 MiB each: above what 8 TB/s allows (1 ms), within the wall time around the same work
+    assert 1.0 < ms.value <= wall_ms, (ms.value, wall_ms)
+    for call in (lambda: L.gh_event_elapsed_ms(None, e1, C.byref(ms)), lambda: L.gh_event_elapsed_ms(e0, e1, None),
+                 lambda: L.gh_event_create_timed(None)):
+        assert call() == -1
+    _lib.check(L.gh_event_destroy(e0))
+    _lib.check(L.gh_event_destroy(e1))

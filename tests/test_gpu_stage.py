@@ -322,3 +322,41 @@ def test_set_prompts_equals_row_by_row():
         b.set_prompts(ids, tokens[:4], pos)
     a.close()
     b.close()
+
+
+def test_device_span_timing_counts_steps_and_leaves_results_alone():
+    # the span timer records two events per forward(): same outputs with it on, one span per step, a read resets it
+    import time
+    name, dtype = "test-gqa4", "f16"
+    cfg = SHAPES[name]
+    layers, base = make_weights(cfg, np.float16, seed=8, wcls=True)
+    batch = 5
+    rng = np.random.default_rng(10)
+    xs = [rng.standard_normal((batch, cfg.dim)).astype(np.float16) for _ in range(4)]
+
+    def run(timed):
+        st = S.Stage(name, dtype, 1, 2, batch, batch, with_cls=False)
+        load_weights(st, cfg, layers, base, True, layer_range=[1, 2], with_embedding=False, with_cls=False)
+        st.time_device_spans(timed)
+        outs, wall = [], 0.0
+        for step, x in enumerate(xs):
+            st.new_state(batch, next_layer=1)
+            for i in range(batch):
+                st.set_prompt(i, 20 + i, 1, step)
+            st.activations(allocate=True)[:] = x.reshape(-1)
+            t0 = time.perf_counter()
+            assert st.forward()
+            wall += time.perf_counter() - t0
+            outs.append(st.activations().copy())
+        spans = st.device_spans()
+        again = st.device_spans()
+        st.close()
+        return outs, spans, again, wall * 1e3
+
+    plain, spans_off, _, _ = run(False)
+    timed, spans_on, again, wall_ms = run(True)
+    assert spans_off == (0.0, 0)
+    assert spans_on[1] == len(xs) and again == (0.0, 0)
+    assert 0.0 < spans_on[0] <= wall_ms, (spans_on, wall_ms)
+    for a, b in zip(plain, timed):
+        assert np.array_equal(a, b)
