@@ -120,6 +120,9 @@ SIGNATURES = {
     "gh_attn_decode_static_limit": (_u64, []),
     "gh_attn_decode_static": (_i, [_vp, _vp, _vp, _vp, _u64, _u32, _shp, _i, _i, _vp]),
     "gh_attn_decode_host": (_i, [_vp, _vp, _vp, _vp, _u64, _shp, _i, _vp, _u64, _i, _vp]),
+    "gh_attn_balanced_workspace": (_u64, [_u64, _shp]),
+    "gh_attn_balance": (_i, [_vp, _vp, _u64, _u32, _shp, _vp, _u64, _vp]),
+    "gh_attn_decode_balanced": (_i, [_vp, _vp, _vp, _u64, _u32, _shp, _i, _vp, _u64, _vp]),
     "gh_prefill_tables": (_i, [_vp, _vp, _u64, _u32, _u64, _vp, _vp, _vp, _vp]),
     "gh_attn_set_prefill_tiles": (_i, [_i]),
     "gh_attn_prefill_workspace": (_u64, [_u64, _u32, _shp]),

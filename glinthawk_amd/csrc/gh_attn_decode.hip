@@ -396,36 +396,35 @@ __global__ __launch_bounds__( 256 ) void attn_decode_valu_kernel( const __half* 
 //   V fragments B[k = token 4*g4+i][n = c] for output column (dim 8*c + nn) are byte-permuted out of
 //     the four 16-byte registers; acc[nn][i] = O[head 4*g4+i][dim 8*c+nn]
 // =================================================================================================
+// One (context, kv head) stream over the tokens [t_begin, t_end), t_begin < t_end: the running maximum `m` (log2 domain) and this
+// lane's share `l` of the running sum of head c, and the unnormalised output acc[nn][i] = O[head 4*g4+i][dim 8*c+nn].
+// `rot` moves the tile the walk starts at (see below).
 template<int G>
-__global__ __launch_bounds__( 256 ) void attn_decode_mfma_kernel( const __half* __restrict__ q,
-                                                                  const __half* const* __restrict__ layer_rows,
-                                                                  const uint32_t* __restrict__ pos,
-                                                                  Partials part,
-                                                                  __half* __restrict__ xb,
-                                                                  uint32_t n_kv_heads,
-                                                                  uint32_t chunk,
-                                                                  uint32_t max_splits,
-                                                                  float scale_log2e )
+__device__ __forceinline__ void mfma_stream_range( const __half* __restrict__ q,
+                                                   const __half* base,
+                                                   const uint32_t ctx,
+                                                   const uint32_t h,
+                                                   const uint32_t t_begin,
+                                                   const uint32_t t_end,
+                                                   const uint32_t rot,
+                                                   const uint32_t n_kv_heads,
+                                                   const float scale_log2e,
+                                                   uint4* tile,
+                                                   f32x4 ( &acc )[8],
+                                                   float& m,
+                                                   float& l )
 {
-  __shared__ uint4 s_k[4][16 * 16]; // per wave: 16 tokens x 16 chunks of 16 bytes
-
-  const WaveJob job = wave_job( layer_rows, pos, n_kv_heads, chunk, max_splits );
-  if ( !job.valid ) {
-    return; // wave-uniform; only wave-private LDS is used, no block barrier
-  }
-  const uint32_t wave = threadIdx.x >> 6;
   const uint32_t lane = threadIdx.x & 63;
   const uint32_t c = lane & 15;
   const uint32_t g4 = lane >> 4;
   const uint32_t n_heads = n_kv_heads * G;
   const uint64_t row_elems = 2ull * n_kv_heads * HS;
   const uint32_t v_off = n_kv_heads * HS;
-  uint4* tile = s_k[wave];
 
   // B fragments of Q^T: head c (zero for the padding heads), dims of chunk 4*kk + g4
   f16x8 qb[4];
   {
-    const __half* qp = q + ( (uint64_t)job.ctx * n_heads + (uint64_t)job.h * G + ( c < G ? c : 0 ) ) * HS;
+    const __half* qp = q + ( (uint64_t)ctx * n_heads + (uint64_t)h * G + ( c < G ? c : 0 ) ) * HS;
 #pragma unroll
     for ( int kk = 0; kk < 4; kk++ ) {
       uint4 v = load16( qp + 8 * ( 4 * kk + g4 ) );
@@ -436,30 +435,29 @@ __global__ __launch_bounds__( 256 ) void attn_decode_mfma_kernel( const __half* 
     }
   }
 
-  f32x4 acc[8];
 #pragma unroll
   for ( int nn = 0; nn < 8; nn++ ) {
     acc[nn] = f32x4 { 0.0f, 0.0f, 0.0f, 0.0f };
   }
-  float m = -INFINITY; // running max of head c (log2 domain), identical in the 4 lanes that share c
-  float l = 0.0f;      // this lane's share of the running sum of head c
+  m = -INFINITY; // running max of head c (log2 domain), identical in the 4 lanes that share c
+  l = 0.0f;      // this lane's share of the running sum of head c
 
-  const __half* kp = job.base + (uint64_t)job.h * HS + 8 * c;
+  const __half* kp = base + (uint64_t)h * HS + 8 * c;
   const uint4 zero4 = make_uint4( 0, 0, 0, 0 );
 
   // The 16-token tiles of the range are visited from a starting tile that differs between blocks,
   // wrapping around (the online softmax does not care about the order).  Blocks launched together
   // otherwise walk their ranges in lock step, and ranges of different contexts and splits lie
   // large power-of-two distances apart: such addresses share few HBM channels.
-  const uint32_t n_tiles = ( job.t_end - job.t_begin + 15 ) / 16;
-  uint32_t tile_i = ( ( job.ctx * 5u + job.split * 3u ) * 7u ) % n_tiles;
-  uint32_t t0 = job.t_begin + 16 * tile_i;
+  const uint32_t n_tiles = ( t_end - t_begin + 15 ) / 16;
+  uint32_t tile_i = ( ( ctx * 5u + rot * 3u ) * 7u ) % n_tiles;
+  uint32_t t0 = t_begin + 16 * tile_i;
 
   uint4 kn[4], vn[4];
 #pragma unroll
   for ( int i = 0; i < 4; i++ ) {
     const uint32_t tok = t0 + 4 * g4 + i;
-    const bool ok = tok < job.t_end;
+    const bool ok = tok < t_end;
     const __half* row = kp + (uint64_t)tok * row_elems;
     kn[i] = ok ? load16_stream( row ) : zero4;
     vn[i] = ok ? load16_stream( row + v_off ) : zero4;
@@ -467,7 +465,7 @@ __global__ __launch_bounds__( 256 ) void attn_decode_mfma_kernel( const __half* 
 
   for ( uint32_t it = 0; it < n_tiles; it++ ) {
     tile_i = tile_i + 1 == n_tiles ? 0 : tile_i + 1;
-    const uint32_t t_next = job.t_begin + 16 * tile_i;
+    const uint32_t t_next = t_begin + 16 * tile_i;
     const bool more = it + 1 < n_tiles;
     uint4 vc[4];
     // K tile into LDS: token 4*g4+i, chunk c, stored at chunk position c ^ token
@@ -481,7 +479,7 @@ __global__ __launch_bounds__( 256 ) void attn_decode_mfma_kernel( const __half* 
 #pragma unroll
     for ( int i = 0; i < 4; i++ ) {
       const uint32_t tok = t_next + 4 * g4 + i;
-      const bool ok = more && tok < job.t_end;
+      const bool ok = more && tok < t_end;
       const __half* row = kp + (uint64_t)tok * row_elems;
       kn[i] = ok ? load16_stream( row ) : zero4;
       vn[i] = ok ? load16_stream( row + v_off ) : zero4;
@@ -505,7 +503,7 @@ __global__ __launch_bounds__( 256 ) void attn_decode_mfma_kernel( const __half* 
     float mt = -INFINITY;
 #pragma unroll
     for ( int i = 0; i < 4; i++ ) {
-      const bool ok = t0 + 4 * g4 + i < job.t_end;
+      const bool ok = t0 + 4 * g4 + i < t_end;
       s[i] = ok ? st[i] * scale_log2e : -INFINITY;
       mt = fmaxf( mt, s[i] );
     }
@@ -554,6 +552,36 @@ __global__ __launch_bounds__( 256 ) void attn_decode_mfma_kernel( const __half* 
     t0 = t_next;
   }
 
+}
+
+template<int G>
+__global__ __launch_bounds__( 256 ) void attn_decode_mfma_kernel( const __half* __restrict__ q,
+                                                                  const __half* const* __restrict__ layer_rows,
+                                                                  const uint32_t* __restrict__ pos,
+                                                                  Partials part,
+                                                                  __half* __restrict__ xb,
+                                                                  uint32_t n_kv_heads,
+                                                                  uint32_t chunk,
+                                                                  uint32_t max_splits,
+                                                                  float scale_log2e )
+{
+  __shared__ uint4 s_k[4][16 * 16]; // per wave: 16 tokens x 16 chunks of 16 bytes
+
+  const WaveJob job = wave_job( layer_rows, pos, n_kv_heads, chunk, max_splits );
+  if ( !job.valid ) {
+    return; // wave-uniform; only wave-private LDS is used, no block barrier
+  }
+  const uint32_t wave = threadIdx.x >> 6;
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t c = lane & 15;
+  const uint32_t g4 = lane >> 4;
+  const uint32_t n_heads = n_kv_heads * G;
+  uint4* tile = s_k[wave];
+
+  f32x4 acc[8];
+  float m, l;
+  mfma_stream_range<G>( q, job.base, job.ctx, job.h, job.t_begin, job.t_end, job.split, n_kv_heads, scale_log2e, tile, acc, m, l );
+
   // total sum of head c over the four lane groups
   l += __shfl_xor( l, 16, WAVE );
   l += __shfl_xor( l, 32, WAVE );
@@ -590,6 +618,227 @@ __global__ __launch_bounds__( 256 ) void attn_decode_mfma_kernel( const __half* 
       }
     }
   }
+}
+
+// =================================================================================================
+// balanced variant of the mfma kernel for batches whose contexts differ in length
+//
+// With one work-group per (context, group of 4 kv heads) and every work-group resident at once, a launch lasts as long as
+// the CU that drew the longest contexts.  Here the keys of all contexts are laid end to end in chunks of BAL_CHUNK tokens
+// and the list is cut into equal runs, one per resident work-group (two per CU): a work-group walks its run through as
+// many contexts as it spans.  A piece that is a whole context is finished on the spot; the pieces of a context that a cut
+// divides leave partials, at slot (context + work-group) -- along the list either of the two grows by one from piece to
+// piece, so the sum numbers the pieces -- and the merge kernel combines them.  The cuts depend on the positions only, not
+// on the layer: attn_balance_kernel makes them once per step.
+//   plan (u32): header[8] (0: chunks per work-group, 1: chunks in all) | prefix[batch + 1] chunks before context c |
+//               length[batch] keys of context c (0: none) | first[work-groups per head group] context a work-group starts in
+// =================================================================================================
+constexpr uint32_t BAL_CHUNK = 64;
+constexpr uint32_t BAL_MIN_RUN = 4; // chunks: a shorter run costs more in start-up than it evens out (measured at 16 contexts)
+constexpr uint32_t BAL_HEADER = 8;
+constexpr int BAL_PLAN_THREADS = 1024;
+
+struct BalancedPlan
+{
+  uint32_t* header;
+  uint32_t* prefix;
+  uint32_t* length;
+  uint32_t* first;
+};
+
+__global__ __launch_bounds__( BAL_PLAN_THREADS ) void attn_balance_kernel( const void* const* __restrict__ layer_rows,
+                                                                         const uint32_t* __restrict__ pos,
+                                                                         uint32_t batch,
+                                                                         uint32_t max_len,
+                                                                         uint32_t wgs,
+                                                                         BalancedPlan plan )
+{
+  __shared__ uint32_t s_scan[BAL_PLAN_THREADS];
+  const uint32_t t = threadIdx.x;
+  const uint32_t per = ( batch + BAL_PLAN_THREADS - 1 ) / BAL_PLAN_THREADS; // contexts per thread, consecutive
+  const uint32_t c_begin = min( batch, t * per ), c_end = min( batch, c_begin + per );
+  uint32_t own = 0;
+  for ( uint32_t c = c_begin; c < c_end; c++ ) {
+    const uint32_t len = layer_rows[c] != nullptr ? min( pos[c] + 1, max_len ) : 0u; // never beyond what the host sized the call for
+    plan.length[c] = len;
+    own += ( len + BAL_CHUNK - 1 ) / BAL_CHUNK;
+  }
+  s_scan[t] = own;
+  __syncthreads();
+  for ( uint32_t d = 1; d < BAL_PLAN_THREADS; d <<= 1 ) { // inclusive scan
+    const uint32_t add = t >= d ? s_scan[t - d] : 0u;
+    __syncthreads();
+    s_scan[t] += add;
+    __syncthreads();
+  }
+  const uint32_t total = s_scan[BAL_PLAN_THREADS - 1];
+  const uint32_t run = max( BAL_MIN_RUN, ( total + wgs - 1 ) / wgs );
+  if ( t == 0 ) {
+    plan.header[0] = run;
+    plan.header[1] = total;
+    plan.prefix[batch] = total;
+  }
+  for ( uint32_t w = t; w < wgs; w += BAL_PLAN_THREADS ) {
+    plan.first[w] = batch; // a work-group whose run starts behind the list has nothing to do
+  }
+  __syncthreads(); // first[] is initialised before any thread overwrites an entry (global memory, same block)
+  uint32_t before = s_scan[t] - own;
+  for ( uint32_t c = c_begin; c < c_end; c++ ) {
+    const uint32_t n = ( plan.length[c] + BAL_CHUNK - 1 ) / BAL_CHUNK;
+    plan.prefix[c] = before;
+    // the work-groups whose run starts inside this context
+    for ( uint32_t w = ( before + run - 1 ) / run; w < wgs && w * run < before + n; w++ ) {
+      plan.first[w] = c;
+    }
+    before += n;
+  }
+}
+
+// slot of the piece (context c, work-group w of head group g) for the query head (kv head `h_local` of the group, head `hd` of it)
+__device__ __forceinline__ uint64_t balanced_slot( uint32_t g, uint32_t pieces, uint32_t c, uint32_t w, uint32_t h_local, uint32_t G, uint32_t hd )
+{
+  return ( ( (uint64_t)g * pieces + c + w ) * 4 + h_local ) * G + hd;
+}
+
+// grid: work-groups per head group x head groups; wave <-> kv head of the group
+template<int G>
+__global__ __launch_bounds__( 256 ) void attn_decode_balanced_kernel( const __half* __restrict__ q,
+                                                                      const __half* const* __restrict__ layer_rows,
+                                                                      BalancedPlan plan,
+                                                                      Partials part,
+                                                                      __half* __restrict__ xb,
+                                                                      uint32_t n_kv_heads,
+                                                                      uint32_t batch,
+                                                                      uint32_t wgs,
+                                                                      float scale_log2e )
+{
+  __shared__ uint4 s_k[4][16 * 16];
+  const uint32_t wave = threadIdx.x >> 6;
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t c16 = lane & 15;
+  const uint32_t g4 = lane >> 4;
+  const uint32_t head_groups = ( n_kv_heads + 3 ) / 4;
+  const uint32_t w = blockIdx.x / head_groups; // the head groups of a run of keys start next to each other in time: whole cache rows are read together
+  const uint32_t g = blockIdx.x % head_groups;
+  const uint32_t h = g * 4 + wave;
+  if ( h >= n_kv_heads ) {
+    return; // wave-uniform; only wave-private LDS is used, no block barrier
+  }
+  const uint32_t n_heads = n_kv_heads * G;
+  const uint32_t run = plan.header[0], total = plan.header[1];
+  const uint32_t pieces = batch + wgs;
+  uint32_t at = w * run; // position in the list of chunks
+  const uint32_t end = min( total, at + run );
+  uint32_t c = plan.first[w];
+  // every turn either moves `at` forward or steps over a context without keys; at < end <= prefix[batch] keeps c < batch
+  while ( at < end && c < batch ) {
+    const uint32_t p0 = plan.prefix[c], p1 = plan.prefix[c + 1];
+    if ( p1 <= at ) {
+      c++;
+      continue;
+    }
+    const uint32_t piece_end = min( p1, end );
+    const __half* base = layer_rows[c];
+    const uint32_t t_begin = ( at - p0 ) * BAL_CHUNK;
+    const uint32_t t_end = min( plan.length[c], ( piece_end - p0 ) * BAL_CHUNK );
+    const bool whole = at == p0 && piece_end == p1;
+    if ( base != nullptr && t_begin < t_end ) {
+      f32x4 acc[8];
+      float m, l;
+      mfma_stream_range<G>( q, base, c, h, t_begin, t_end, w, n_kv_heads, scale_log2e, s_k[wave], acc, m, l );
+      l += __shfl_xor( l, 16, WAVE );
+      l += __shfl_xor( l, 32, WAVE );
+#pragma unroll
+      for ( int i = 0; i < 4; i++ ) {
+        const uint32_t hd = 4 * g4 + i;
+        const float mh = __shfl( m, (int)hd, WAVE );
+        const float lh = __shfl( l, (int)hd, WAVE );
+        if ( hd < G ) {
+          if ( whole ) {
+            const uint64_t head = (uint64_t)c * n_heads + (uint64_t)h * G + hd;
+            const float inv = 1.0f / lh;
+            union
+            {
+              uint4 raw;
+              __half h[8];
+            } o;
+#pragma unroll
+            for ( int nn = 0; nn < 8; nn++ ) {
+              o.h[nn] = __float2half_rn( acc[nn][i] * inv );
+            }
+            *reinterpret_cast<uint4*>( xb + head * HS + 8 * c16 ) = o.raw;
+          } else {
+            const uint64_t slot = balanced_slot( g, pieces, c, w, wave, G, hd );
+            float4* o = reinterpret_cast<float4*>( part.out + slot * HS + 8 * c16 );
+            o[0] = make_float4( acc[0][i], acc[1][i], acc[2][i], acc[3][i] );
+            o[1] = make_float4( acc[4][i], acc[5][i], acc[6][i], acc[7][i] );
+            if ( c16 == 0 ) {
+              part.ml[slot * 2] = mh;
+              part.ml[slot * 2 + 1] = lh;
+            }
+          }
+        }
+      }
+    }
+    at = piece_end;
+    if ( piece_end == p1 ) {
+      c++;
+    }
+  }
+}
+
+// block <-> (query head, context), thread <-> output dim: combines the pieces of a context that the cuts divided
+template<int G>
+__global__ __launch_bounds__( 128 ) void attn_merge_balanced_kernel( BalancedPlan plan, Partials part, __half* __restrict__ xb, uint32_t n_heads, uint32_t batch, uint32_t wgs )
+{
+  const uint32_t head = blockIdx.x;
+  const uint32_t ctx = blockIdx.y;
+  const uint32_t p0 = plan.prefix[ctx], p1 = plan.prefix[ctx + 1], run = plan.header[0];
+  if ( p1 == p0 ) {
+    return; // no keys: the output row stays as it is, as in the other kernels
+  }
+  const uint32_t w0 = p0 / run, w1 = ( p1 - 1 ) / run;
+  if ( w0 == w1 ) {
+    return; // one piece: written by the work-group that ran it
+  }
+  const uint32_t kv = head / G, hd = head % G;
+  const uint64_t slot0 = balanced_slot( kv / 4, batch + wgs, ctx, w0, kv % 4, G, hd );
+  const uint64_t step = 4ull * G; // slots from one work-group's piece to the next one's
+  const uint32_t n = w1 - w0 + 1;
+  const float2* ml = reinterpret_cast<const float2*>( part.ml );
+  const uint32_t d = threadIdx.x; // head size 128 = block size
+  constexpr uint32_t MERGE_BATCH = 4;
+  float2 st[MERGE_BATCH];
+  float o[MERGE_BATCH];
+#pragma unroll
+  for ( uint32_t u = 0; u < MERGE_BATCH; u++ ) {
+    const uint64_t slot = slot0 + min( u, n - 1 ) * step;
+    st[u] = ml[slot];
+    o[u] = part.out[slot * HS + d];
+  }
+  float m = -INFINITY;
+#pragma unroll
+  for ( uint32_t u = 0; u < MERGE_BATCH; u++ ) {
+    m = fmaxf( m, st[u].x );
+  }
+  for ( uint32_t k = MERGE_BATCH; k < n; k++ ) {
+    m = fmaxf( m, ml[slot0 + k * step].x );
+  }
+  float l = 0.0f, acc = 0.0f;
+#pragma unroll
+  for ( uint32_t u = 0; u < MERGE_BATCH; u++ ) {
+    const float wgt = u < n ? fast_exp2( st[u].x - m ) : 0.0f;
+    l += st[u].y * wgt;
+    acc += o[u] * wgt;
+  }
+  for ( uint32_t k = MERGE_BATCH; k < n; k++ ) {
+    const uint64_t slot = slot0 + k * step;
+    const float2 e = ml[slot];
+    const float wgt = fast_exp2( e.x - m );
+    l += e.y * wgt;
+    acc += part.out[slot * HS + d] * wgt;
+  }
+  xb[( (uint64_t)ctx * n_heads + head ) * HS + d] = __float2half_rn( acc * ( 1.0f / l ) );
 }
 
 // =================================================================================================
@@ -673,6 +922,65 @@ void launch_mfma( dim3 grid, hipStream_t st, const void* q, const void* const* r
 {
   attn_decode_mfma_kernel<G><<<grid, 256, 0, st>>>( static_cast<const __half*>( q ), reinterpret_cast<const __half* const*>( rows ), pos, part,
                                                    static_cast<__half*>( xb ), s->n_kv_heads, p.chunk, p.max_splits, scale );
+}
+
+// where the plan and the partials of the balanced variant lie in its workspace
+struct BalancedLayout
+{
+  uint32_t head_groups, wgs; // groups of 4 kv heads; work-groups per head group
+  uint64_t plan_bytes, out_floats, ml_floats, total_bytes;
+};
+
+BalancedLayout balanced_layout( uint64_t batch, const gh_shape* s )
+{
+  BalancedLayout y;
+  y.head_groups = ( s->n_kv_heads + 3 ) / 4;
+  // two work-groups of four waves are resident per CU
+  y.wgs = std::max<uint32_t>( 1, 2u * (uint32_t)cu_count() / y.head_groups );
+  const uint64_t pieces = batch + y.wgs;
+  const uint64_t heads = 4ull * s->gqa_size; // per (head group, piece)
+  y.out_floats = y.head_groups * pieces * heads * HS;
+  y.ml_floats = y.head_groups * pieces * heads * 2;
+  y.plan_bytes = ( ( BAL_HEADER + ( batch + 1 ) + batch + y.wgs ) * sizeof( uint32_t ) + 255 ) / 256 * 256;
+  y.total_bytes = y.plan_bytes + ( y.out_floats + y.ml_floats ) * sizeof( float );
+  return y;
+}
+
+BalancedPlan balanced_plan( void* workspace, uint64_t batch )
+{
+  BalancedPlan p;
+  p.header = static_cast<uint32_t*>( workspace );
+  p.prefix = p.header + BAL_HEADER;
+  p.length = p.prefix + batch + 1;
+  p.first = p.length + batch;
+  return p;
+}
+
+int balanced_check( const char* who, uint64_t batch, uint32_t max_pos, const gh_shape* shape, const void* workspace, uint64_t workspace_bytes )
+{
+  GH_REQUIRE( shape != nullptr, "%s: NULL shape", who );
+  GH_REQUIRE( shape->n_kv_heads > 0 && shape->gqa_size > 0 && shape->seq_len > 0, "%s: zero dimension", who );
+  GH_REQUIRE( shape->n_heads == shape->n_kv_heads * shape->gqa_size, "%s: n_heads != n_kv_heads * gqa_size", who );
+  GH_REQUIRE( shape->kv_dim == shape->n_kv_heads * shape->head_size, "%s: kv_dim != n_kv_heads * head_size", who );
+  GH_REQUIRE( shape->head_size == HS && mfma_gqa_ok( shape->gqa_size ), "%s: needs head_size 128 and gqa in {2,4,8,16}", who );
+  GH_REQUIRE( max_pos < shape->seq_len, "%s: max_pos %u outside seq_len %u", who, max_pos, shape->seq_len );
+  GH_REQUIRE( batch > 0 && batch <= 65535, "%s: bad batch", who );
+  GH_REQUIRE( workspace != nullptr && ( reinterpret_cast<uintptr_t>( workspace ) & 15u ) == 0, "%s: workspace missing or not 16-byte aligned", who );
+  const uint64_t need = balanced_layout( batch, shape ).total_bytes;
+  if ( workspace_bytes < need ) {
+    return fail( GH_ERR_WORKSPACE, "%s: %llu bytes of workspace needed, %llu available", who, (unsigned long long)need, (unsigned long long)workspace_bytes );
+  }
+  return GH_OK;
+}
+
+template<int G>
+void launch_balanced( const BalancedLayout& y, hipStream_t st, const void* q, const void* const* rows, const BalancedPlan& plan, Partials part, void* xb,
+                      const gh_shape* s, uint64_t batch, float scale )
+{
+  attn_decode_balanced_kernel<G><<<y.head_groups * y.wgs, 256, 0, st>>>( static_cast<const __half*>( q ), reinterpret_cast<const __half* const*>( rows ), plan,
+                                                                        part, static_cast<__half*>( xb ), s->n_kv_heads, (uint32_t)batch, y.wgs, scale );
+  attn_merge_balanced_kernel<G><<<dim3( s->n_heads, (unsigned)batch ), 128, 0, st>>>( plan, part, static_cast<__half*>( xb ), s->n_heads, (uint32_t)batch,
+                                                                                      y.wgs );
 }
 
 } // namespace
@@ -874,6 +1182,67 @@ int gh_attn_decode_static( const void* q, const void* const* layer_rows_dev, con
   // a plan that needs more partials than the array holds is refused by the size check of the shared path (GH_ERR_WORKSPACE)
   return attn_decode_run( "gh_attn_decode_static", q, layer_rows_dev, pos_dev, xb, batch, max_pos, shape, dt, g_static_scratch[device],
                           STATIC_SCRATCH_BYTES, variant, stream, false );
+}
+
+uint64_t gh_attn_balanced_workspace( uint64_t batch, const gh_shape* shape )
+{
+  if ( shape == nullptr || batch == 0 || shape->n_kv_heads == 0 || ensure_init() != GH_OK ) {
+    return 0;
+  }
+  return balanced_layout( batch, shape ).total_bytes;
+}
+
+int gh_attn_balance( const void* const* layer_rows_dev, const uint32_t* pos_dev, uint64_t batch, uint32_t max_pos, const gh_shape* shape, void* workspace,
+                     uint64_t workspace_bytes, gh_stream stream )
+{
+  if ( int rc = ensure_init() ) {
+    return rc;
+  }
+  if ( batch == 0 ) {
+    return GH_OK;
+  }
+  GH_REQUIRE( layer_rows_dev && pos_dev, "gh_attn_balance: NULL pointer" );
+  if ( int rc = balanced_check( "gh_attn_balance", batch, max_pos, shape, workspace, workspace_bytes ) ) {
+    return rc;
+  }
+  const BalancedLayout y = balanced_layout( batch, shape );
+  attn_balance_kernel<<<1, BAL_PLAN_THREADS, 0, as_stream( stream )>>>( layer_rows_dev, pos_dev, (uint32_t)batch, max_pos + 1, y.wgs,
+                                                                        balanced_plan( workspace, batch ) );
+  GH_LAUNCH_CHECK();
+  return GH_OK;
+}
+
+int gh_attn_decode_balanced( const void* q, const void* const* layer_rows_dev, void* xb, uint64_t batch, uint32_t max_pos, const gh_shape* shape, gh_dtype dt,
+                             void* workspace, uint64_t workspace_bytes, gh_stream stream )
+{
+  if ( int rc = ensure_init() ) {
+    return rc;
+  }
+  if ( batch == 0 ) {
+    return GH_OK;
+  }
+  GH_REQUIRE( q && layer_rows_dev && xb, "gh_attn_decode_balanced: NULL pointer" );
+  GH_REQUIRE( dt == GH_F16, "gh_attn_decode_balanced: f16 only" );
+  GH_REQUIRE( ( reinterpret_cast<uintptr_t>( q ) & 15u ) == 0 && ( reinterpret_cast<uintptr_t>( xb ) & 15u ) == 0,
+              "gh_attn_decode_balanced: q and xb must be 16-byte aligned" );
+  if ( int rc = balanced_check( "gh_attn_decode_balanced", batch, max_pos, shape, workspace, workspace_bytes ) ) {
+    return rc;
+  }
+  const BalancedLayout y = balanced_layout( batch, shape );
+  const BalancedPlan plan = balanced_plan( workspace, batch );
+  Partials part;
+  part.out = reinterpret_cast<float*>( static_cast<char*>( workspace ) + y.plan_bytes );
+  part.ml = part.out + y.out_floats;
+  const float scale = LOG2E / sqrtf( (float)shape->head_size );
+  hipStream_t st = as_stream( stream );
+  switch ( shape->gqa_size ) {
+    case 2: launch_balanced<2>( y, st, q, layer_rows_dev, plan, part, xb, shape, batch, scale ); break;
+    case 4: launch_balanced<4>( y, st, q, layer_rows_dev, plan, part, xb, shape, batch, scale ); break;
+    case 8: launch_balanced<8>( y, st, q, layer_rows_dev, plan, part, xb, shape, batch, scale ); break;
+    default: launch_balanced<16>( y, st, q, layer_rows_dev, plan, part, xb, shape, batch, scale ); break;
+  }
+  GH_LAUNCH_CHECK();
+  return GH_OK;
 }
 
 int gh_attn_decode_host( const void* q, const void* const* layer_rows_host, const uint32_t* pos_host, void* xb, uint64_t batch,

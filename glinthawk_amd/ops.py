@@ -232,6 +232,24 @@ def attn_decode(q, layer_rows: torch.Tensor, pos: torch.Tensor, xb, max_pos: int
           "gh_attn_decode")
 
 
+def attn_balanced_workspace(batch: int, shape: Shape) -> int:
+    s = shape.c()
+    return int(lib().gh_attn_balanced_workspace(batch, C.byref(s)))
+
+
+def attn_balance(layer_rows: torch.Tensor, pos: torch.Tensor, max_pos: int, shape: Shape, workspace: torch.Tensor) -> None:
+    """Cuts the keys of a batch into equal runs (once per step); `workspace` then serves attn_decode_balanced for every layer."""
+    s = shape.c()
+    check(lib().gh_attn_balance(_p(layer_rows), _p(pos), layer_rows.numel(), max_pos, C.byref(s), _p(workspace),
+                                workspace.numel() * workspace.element_size(), _stream()), "gh_attn_balance")
+
+
+def attn_decode_balanced(q, layer_rows: torch.Tensor, xb, max_pos: int, shape: Shape, workspace: torch.Tensor) -> None:
+    s = shape.c()
+    check(lib().gh_attn_decode_balanced(_p(q), _p(layer_rows), _p(xb), layer_rows.numel(), max_pos, C.byref(s), _dt(q), _p(workspace),
+                                        workspace.numel() * workspace.element_size(), _stream()), "gh_attn_decode_balanced")
+
+
 def attn_decode_host(q, layer_rows: Sequence[int], pos: Sequence[int], xb, shape: Shape,
                      workspace: Optional[torch.Tensor] = None, variant: int = GH_ATTN_AUTO) -> None:
     s = shape.c()

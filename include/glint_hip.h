@@ -255,6 +255,20 @@ int gh_attn_decode( const void* q, const void* const* layer_rows_dev, const uint
 uint64_t gh_attn_decode_static_limit( void );
 int gh_attn_decode_static( const void* q, const void* const* layer_rows_dev, const uint32_t* pos_dev, void* xb, uint64_t batch, uint32_t max_pos,
                            const gh_shape* shape, gh_dtype dt, int variant, gh_stream stream );
+/* Decode attention for batches whose contexts differ in length (the same result as gh_attn_decode: attention_0_gemm, attention_softmax
+ * and attention_2_gemm of arch/amd64/llama2/ops.hh:170-298 in one pass; the reference runs one task per (context, kv head),
+ * ops.hh:192-193, whatever their lengths).  The keys of all contexts are cut into equal runs, one per resident work-group, so that
+ * no CU is left with the longest contexts while others idle.  f16, head size 128, gqa in {2, 4, 8, 16}.
+ *   gh_attn_balanced_workspace  bytes for the cuts and the partial results of `batch` contexts (needs the device: 0 on failure)
+ *   gh_attn_balance             makes the cuts from the positions (pos_dev[i] = position of the current token, keys [0, pos_i];
+ *                               contexts with a NULL row in layer_rows_dev have none); once per step: the cuts do not depend on the layer
+ *   gh_attn_decode_balanced     one layer, with the cuts gh_attn_balance left in `workspace`; layer_rows_dev must have its NULL
+ *                               rows where that call's table had them.  Calls on one workspace must not overlap in time. */
+uint64_t gh_attn_balanced_workspace( uint64_t batch, const gh_shape* shape );
+int gh_attn_balance( const void* const* layer_rows_dev, const uint32_t* pos_dev, uint64_t batch, uint32_t max_pos, const gh_shape* shape, void* workspace,
+                     uint64_t workspace_bytes, gh_stream stream );
+int gh_attn_decode_balanced( const void* q, const void* const* layer_rows_dev, void* xb, uint64_t batch, uint32_t max_pos, const gh_shape* shape, gh_dtype dt,
+                             void* workspace, uint64_t workspace_bytes, gh_stream stream );
 int gh_attn_decode_host( const void* q, const void* const* layer_rows_host, const uint32_t* pos_host, void* xb, uint64_t batch,
                          const gh_shape* shape, gh_dtype dt, void* workspace, uint64_t workspace_bytes, int variant, gh_stream stream );
 

@@ -546,7 +546,7 @@ def test_unfused_attention_ops_streaming_kernels(name, shape, pos, host_tables):
 
 
 # ------------------------------------------------------------------ fused decode attention
-def run_fused_case(shape, dt, variant, pos, present, chunk, seed=13, host_tables=False, std=1.0):
+def run_fused_case(shape, dt, variant, pos, present, chunk, seed=13, host_tables=False, std=1.0, balanced=False):
     batch = len(pos)
     cfg = oracle_cfg(shape)
     arena = Arena(shape, batch, tdt(dt), seed=seed, std=std)
@@ -557,7 +557,13 @@ def run_fused_case(shape, dt, variant, pos, present, chunk, seed=13, host_tables
     dxb = torch.full((batch, shape.dim), 5.0, dtype=tdt(dt), device="cuda")
     ops.attn_set_chunk(chunk)
     try:
-        if host_tables:
+        if balanced:
+            max_pos = max([p for p, ok in zip(pos, present) if ok] + [0])
+            ws = torch.empty(ops.attn_balanced_workspace(batch, shape), dtype=torch.uint8, device="cuda")
+            table = ops.row_table(layers)
+            ops.attn_balance(table, torch.tensor(pos, dtype=torch.int32, device="cuda"), max_pos, shape, ws)
+            ops.attn_decode_balanced(dq, table, dxb, max_pos, shape, ws)
+        elif host_tables:
             ops.attn_decode_host(dq, layers, pos, dxb, shape, variant=variant)
         else:
             max_pos = max([p for p, ok in zip(pos, present) if ok] + [0])
@@ -618,6 +624,90 @@ def test_fused_auto_and_host_tables(shape):
     pos = [0, 5, shape.seq_len - 1, shape.seq_len // 2]
     run_fused_case(shape, "f16", GH_ATTN_AUTO, pos, [True, True, True, True], 0, host_tables=True)
     run_fused_case(shape, "f16", GH_ATTN_AUTO, pos, [True, False, True, True], 32, host_tables=True)
+
+
+@pytest.mark.parametrize("shape", [GQA2, GQA4, GQA8, GQA16], ids=["gqa2", "gqa4", "gqa8", "gqa16"])
+def test_fused_balanced_ragged(shape):
+    # keys cut into equal runs over the work-groups: contexts shorter than a run share one, longer ones are divided
+    # (a run is at least 256 keys), an empty context in the middle and at the end
+    pos = [p for p in RAGGED if p < shape.seq_len] + [shape.seq_len - 1, 2, shape.seq_len - 1, 100, 2]
+    present = [True] * len(pos)
+    present[3] = False
+    present[-1] = False
+    run_fused_case(shape, "f16", GH_ATTN_MFMA, pos, present, 0, balanced=True)
+
+
+def test_fused_balanced_cases():
+    shape = GQA8
+    # one context; one long context among short ones; every context equal; only empty contexts but one
+    run_fused_case(shape, "f16", GH_ATTN_MFMA, [699], [True], 0, balanced=True, seed=51)
+    run_fused_case(shape, "f16", GH_ATTN_MFMA, [0], [True], 0, balanced=True, seed=52)
+    run_fused_case(shape, "f16", GH_ATTN_MFMA, [3] * 5 + [699] + [7] * 6, [True] * 12, 0, balanced=True, seed=53)
+    run_fused_case(shape, "f16", GH_ATTN_MFMA, [511] * 9, [True] * 9, 0, balanced=True, seed=54)
+    run_fused_case(shape, "f16", GH_ATTN_MFMA, [10, 20, 300, 40], [False, False, True, False], 0, balanced=True, seed=55)
+    run_fused_case(shape, "f16", GH_ATTN_MFMA, [10, 20], [False, False], 0, balanced=True, seed=56)
+    # large scores
+    run_fused_case(shape, "f16", GH_ATTN_MFMA, [699, 256, 30], [True] * 3, 0, balanced=True, seed=57, std=6.0)
+
+
+def test_fused_balanced_many_contexts_equal_plain_kernel():
+    # more contexts than the planning kernel has threads (it then takes several per thread), against the plain kernel
+    shape = Shape(dim=256, n_layers=1, n_heads=2, n_kv_heads=1, hidden_dim=64, seq_len=96)
+    batch = 2500
+    rng = np.random.default_rng(61)
+    pos = rng.integers(0, shape.seq_len, batch)
+    pos[::97] = shape.seq_len - 1
+    arena = Arena(shape, batch, torch.float16, seed=62)
+    ptrs = [arena.layer_ptr(i) for i in range(batch)]
+    for i in range(5, batch, 41):
+        ptrs[i] = 0
+    table = ops.row_table(ptrs)
+    dpos = torch.tensor(pos, dtype=torch.int32, device="cuda")
+    q = torch.randn((batch, shape.dim), dtype=torch.float16, device="cuda")
+    plain = torch.full((batch, shape.dim), 5.0, dtype=torch.float16, device="cuda")
+    bal = torch.full((batch, shape.dim), 5.0, dtype=torch.float16, device="cuda")
+    max_pos = int(pos.max())
+    ops.attn_decode(q, table, dpos, plain, max_pos, shape, variant=GH_ATTN_MFMA)
+    ws = torch.empty(ops.attn_balanced_workspace(batch, shape), dtype=torch.uint8, device="cuda")
+    ops.attn_balance(table, dpos, max_pos, shape, ws)
+    for _ in range(2):  # the cuts serve every layer of a step: a second call on the same workspace gives the same
+        bal.fill_(5.0)
+        ops.attn_decode_balanced(q, table, bal, max_pos, shape, ws)
+        a, r = errors(bal.cpu().numpy(), plain.cpu().numpy())
+        assert a < 4e-3 and r < 1e-3, (a, r)
+    assert torch.all(bal[5] == 5.0) and torch.all(bal[46] == 5.0)
+
+
+def test_fused_balanced_bound_below_the_true_maximum_truncates_and_bad_arguments():
+    shape = GQA8
+    batch = 3
+    arena = Arena(shape, batch, torch.float16, seed=71)
+    table = ops.row_table([arena.layer_ptr(i) for i in range(batch)])
+    q = torch.randn((batch, shape.dim), dtype=torch.float16, device="cuda")
+    ws = torch.empty(ops.attn_balanced_workspace(batch, shape), dtype=torch.uint8, device="cuda")
+    true_pos = torch.tensor([699, 500, 90], dtype=torch.int32, device="cuda")
+    cut_pos = torch.tensor([299, 299, 90], dtype=torch.int32, device="cuda")
+    a = torch.zeros((batch, shape.dim), dtype=torch.float16, device="cuda")
+    b = torch.zeros_like(a)
+    ops.attn_balance(table, true_pos, 299, shape, ws)   # positions above the bound count as the bound
+    ops.attn_decode_balanced(q, table, a, 299, shape, ws)
+    ops.attn_balance(table, cut_pos, 299, shape, ws)
+    ops.attn_decode_balanced(q, table, b, 299, shape, ws)
+    assert torch.equal(a, b)
+    import ctypes as C
+    from glinthawk_amd import _lib
+    from glinthawk_amd._lib import GH_F16, GH_F32
+    GH_ERR_INVALID, GH_ERR_WORKSPACE = -1, -5
+    L = _lib.lib()
+    s = shape.c()
+    small = torch.empty(1024, dtype=torch.uint8, device="cuda")
+    assert L.gh_attn_balance(table.data_ptr(), true_pos.data_ptr(), batch, 299, C.byref(s), small.data_ptr(), 1024, None) == GH_ERR_WORKSPACE
+    assert L.gh_attn_decode_balanced(q.data_ptr(), table.data_ptr(), a.data_ptr(), batch, 299, C.byref(s), GH_F16, small.data_ptr(), 1024, None) == GH_ERR_WORKSPACE
+    assert L.gh_attn_balance(table.data_ptr(), true_pos.data_ptr(), batch, shape.seq_len, C.byref(s), ws.data_ptr(), ws.numel(), None) == GH_ERR_INVALID
+    mha = MHA128.c()
+    assert L.gh_attn_balance(table.data_ptr(), true_pos.data_ptr(), batch, 10, C.byref(mha), ws.data_ptr(), ws.numel(), None) == GH_ERR_INVALID
+    assert L.gh_attn_decode_balanced(q.data_ptr(), table.data_ptr(), a.data_ptr(), batch, 299, C.byref(s), GH_F32, ws.data_ptr(), ws.numel(), None) == GH_ERR_INVALID
+    assert L.gh_attn_decode_balanced(None, table.data_ptr(), a.data_ptr(), batch, 299, C.byref(s), GH_F16, ws.data_ptr(), ws.numel(), None) == GH_ERR_INVALID
 
 
 def test_fused_variants_agree():
