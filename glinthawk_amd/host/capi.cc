@@ -282,6 +282,7 @@ StageBase* make_stage( int dtype, uint32_t first_layer, uint32_t n_hosted, uint3
   ModelOptions o;
   o.fused_attention = flags & 1u;
   o.fused_projections = !( flags & 8u );
+  o.balanced_attention = ( flags & 16u ) ? 1 : ( ( flags & 32u ) ? -1 : 0 );
   o.seed = seed;
   o.weight_std = std;
   return make_for_config<Config>( dtype, flags & 4u, s, o );
@@ -456,7 +457,8 @@ struct EchoModel
 extern "C" {
 
 // ---- stage harness --------------------------------------------------------------------------
-// flags: 1 fused attention, 2 host the classifier, 4 paged (virtual-memory) contexts, 8 keep the projections unfused
+// flags: 1 fused attention, 2 host the classifier, 4 paged (virtual-memory) contexts, 8 keep the projections unfused,
+// 16 / 32 decode attention over equal runs of keys always / never (neither: where a step's lengths call for it)
 void* glint_stage_create( const char* config, int dtype, uint32_t first_layer, uint32_t n_hosted, uint32_t concurrency, uint32_t max_contexts,
                           uint32_t flags, uint64_t seed, float weight_std )
 {
@@ -761,6 +763,7 @@ void* glint_kernel_create( const char* config, int dtype, uint32_t first_layer, 
   ModelOptions o;
   o.fused_attention = flags & 1u;
   o.fused_projections = !( flags & 8u );
+  o.balanced_attention = ( flags & 16u ) ? 1 : ( ( flags & 32u ) ? -1 : 0 );
   o.seed = seed;
   o.weight_std = weight_std;
   const bool with_cls = flags & 2u;

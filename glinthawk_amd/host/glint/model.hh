@@ -16,6 +16,7 @@
 #include <cstdio>
 #include <filesystem>
 #include <memory>
+#include <type_traits>
 #include <vector>
 
 #include "glint/concepts.hh"
@@ -114,6 +115,7 @@ struct ModelOptions
 {
   bool fused_attention { true };  // false: the reference's three unfused ops + score buffer
   bool fused_projections { true }; // with fused_attention: projections fused with the ops that follow them
+  int balanced_attention { 0 };   // fused decode attention over equal runs of keys: 0 where the step's lengths call for it, 1 always (shapes that have it), -1 never
   bool allocate_logits { true };  // only needed when the classifier is hosted
   uint64_t seed { 1 };            // random initialisation of weights
   float weight_std { 0.02f };     // N(0, std) for every tensor, as the benchmark configurations say
@@ -406,7 +408,7 @@ public:
                                            k == 0 && start_pos[i] == 0 && settings_.first_layer_served == first_layer ) );
       }
     }
-    upload_tables( contexts, run ); // per-context tables: pos = start positions, layer bases per layer
+    upload_tables( contexts, run, false ); // per-context tables: pos = start positions, layer bases per layer
 
     DType* px = pf_x_.get();
     DType* pxb = pf_xb_.get();
@@ -580,12 +582,25 @@ private:
     }
   }
 
+  // the fused decode attention of one layer: over equal runs of keys where upload_tables() found the lengths of this
+  // step's contexts far apart (the cuts are made there, once for all layers), else one wave per (context, kv head, split)
+  void fused_attention( const size_t table_index )
+  {
+    if ( balanced_step_ ) {
+      const gh_shape s = LlamaOperations::shape();
+      GLINT_GH( gh_attn_decode_balanced( q_, layer_rows_dev( table_index ), xb_, batch_, max_pos_, &s, hip::gh_type<DType>(), attn_bal_ws_.get(),
+                                         attn_bal_ws_bytes_, ops_.stream() ) );
+    } else {
+      ops_.attention_fused( q_, layer_rows_dev( table_index ), pos_dev(), xb_, batch_, max_pos_, attn_ws_.get(), attn_ws_bytes_ );
+    }
+  }
+
   void attention_ops( const size_t table_index )
   {
     if ( options_.fused_attention ) {
       GLINT_GH( gh_rope( batch_, pos_dev(), base_.freq_cis_real, base_.freq_cis_imag, q_, token_rows_dev( table_index ), Config::n_kv_heads, Config::gqa_size,
                          Config::head_size, hip::gh_type<DType>(), ops_.stream() ) );
-      ops_.attention_fused( q_, layer_rows_dev( table_index ), pos_dev(), xb_, batch_, max_pos_, attn_ws_.get(), attn_ws_bytes_ );
+      fused_attention( table_index );
     } else {
       ops_.apply_rope( batch_, token_positions_, base_.freq_cis_real, base_.freq_cis_imag, q_, token_contexts_ );
       ops_.attention_0_gemm( q_, layer_contexts_, att_, batch_, token_positions_ );
@@ -621,7 +636,7 @@ private:
   {
     const auto& w = layers_[layer];
     ops_.matmul_qkv_rope_append( q_, xb_, w.wq, batch_, pos_dev(), base_.freq_cis_real, base_.freq_cis_imag, token_rows_dev( table_index ) );
-    ops_.attention_fused( q_, layer_rows_dev( table_index ), pos_dev(), xb_, batch_, max_pos_, attn_ws_.get(), attn_ws_bytes_ );
+    fused_attention( table_index );
     ops_.template matmul_accum<Config::dim, Config::dim>( x_, xb_, w.wo, batch_, xb_, w.rms_ffn_weight );
     ops_.matmul_silu_gate( hb_, xb_, w.w1, batch_ );
     ops_.template matmul_accum<Config::hidden_dim, Config::dim>( x_, hb_, w.w2, batch_, next_att_norm ? xb_ : nullptr, next_att_norm );
@@ -749,7 +764,8 @@ private:
     return reinterpret_cast<void* const*>( ptr_tables( reinterpret_cast<uint8_t*>( tables_dev_.get() ) ) ) + ( 2 * k + 1 ) * table_stride();
   }
 
-  void upload_tables( const ContextVector& contexts, const std::vector<size_t>& run )
+  // `decode`: the positions are those of one new token per context (a batched prefill attends from many)
+  void upload_tables( const ContextVector& contexts, const std::vector<size_t>& run, const bool decode = true )
   {
     // The previous upload reads the pinned buffer asynchronously: it has to be over before the buffer is rewritten.  A step
     // ends with a blocking copy of its results, which is such a wait already; only without one since the last upload is
@@ -760,13 +776,18 @@ private:
     auto* pos = reinterpret_cast<uint32_t*>( tables_host_ );
     auto** ptrs = reinterpret_cast<void**>( ptr_tables( tables_host_ ) );
     max_pos_ = 0;
+    uint64_t keys = 0, live = 0;
     for ( size_t i = 0; i < batch_; i++ ) {
       pos[i] = token_positions_[i];
       if ( !contexts[i]->empty() ) {
         GLINT_CHECK( token_positions_[i] < Config::seq_len );
         max_pos_ = std::max( max_pos_, token_positions_[i] );
+        keys += token_positions_[i] + 1;
+        live++;
       }
     }
+    balanced_step_ = decode && attn_bal_ws_bytes_ > 0 && !run.empty() && options_.balanced_attention >= 0
+                     && ( options_.balanced_attention > 0 || lengths_far_apart( keys, live, max_pos_ + 1 ) );
     for ( size_t k = 0; k < run.size(); k++ ) {
       for ( size_t i = 0; i < batch_; i++ ) {
         const auto layer = contexts[i]->layer( run[k] );
@@ -778,6 +799,26 @@ private:
     GLINT_GH( gh_memcpy( tables_dev_.get(), tables_host_, bytes, GH_HOST_TO_DEVICE, 1, ops_.stream() ) );
     tables_uploaded_ = true;
     tables_drain_count_ = ops_.drain_count();
+    if ( balanced_step_ ) {
+      const gh_shape s = LlamaOperations::shape();
+      GLINT_GH( gh_attn_balance( layer_rows_dev( 0 ), pos_dev(), batch_, max_pos_, &s, attn_bal_ws_.get(), attn_bal_ws_bytes_, ops_.stream() ) );
+    }
+  }
+
+  // Whether the attention over equal runs of keys pays for this step: measured on the 70B shape, it costs 2 % where the
+  // contexts are equally long and start-up where there is little to even out, and gains 10-25 % for lengths spread over
+  // 16..4096 (a launch of the plain kernel lasts as long as the CU that drew the longest contexts), several times for one
+  // long context among many short ones (with 1024 and more (context, kv head) pairs the plain kernel does not split).
+  static bool lengths_far_apart( const uint64_t keys, const uint64_t live, const uint64_t longest )
+  {
+    if ( live == 0 || keys * 100 >= 85 * live * longest ) {
+      return false; // mean length within 15 % of the longest
+    }
+    const uint64_t head_groups = ( Config::n_kv_heads + 3 ) / 4;
+    if ( keys * head_groups >= 131072 ) {
+      return true; // enough keys for runs of 256 and more on every CU
+    }
+    return live * Config::n_kv_heads >= 1024 && longest >= 1024 && longest * live >= 4 * keys;
   }
 
   // ---- allocation ----------------------------------------------------------------------------
@@ -870,6 +911,11 @@ private:
       const gh_shape s = LlamaOperations::shape();
       attn_ws_bytes_ = gh_attn_decode_workspace( cap, Config::seq_len - 1, &s );
       attn_ws_ = ops_.device_allocate( std::max<uint64_t>( attn_ws_bytes_, 16 ) );
+      if ( std::is_same_v<DType, glint::float16_t> && Config::head_size == 128
+           && ( Config::gqa_size == 2 || Config::gqa_size == 4 || Config::gqa_size == 8 || Config::gqa_size == 16 ) ) {
+        attn_bal_ws_bytes_ = gh_attn_balanced_workspace( cap, &s ); // the shapes gh_attn_decode_balanced takes
+        attn_bal_ws_ = ops_.device_allocate( std::max<uint64_t>( attn_bal_ws_bytes_, 16 ) );
+      }
       const size_t n_run = std::max<size_t>( 1, settings_.num_attention_layers_hosted() );
       const size_t bytes = ( cap * sizeof( uint32_t ) + 15 ) / 16 * 16 + n_run * 2 * cap * sizeof( void* );
       tables_dev_ = ops_.device_allocate( bytes );
@@ -1028,6 +1074,9 @@ private:
   std::unique_ptr<CopyLane> copy_lane_ {};
   std::unique_ptr<SpanTimer> span_timer_ {};
   uint64_t attn_ws_bytes_ { 0 };
+  DevicePtr attn_bal_ws_ {};
+  uint64_t attn_bal_ws_bytes_ { 0 };
+  bool balanced_step_ { false };
   uint8_t* tables_host_ { nullptr };
   bool tables_uploaded_ { false };
   uint64_t tables_drain_count_ { 0 };

@@ -17,7 +17,7 @@ _HOST_LIB_PATH = os.environ.get("GLINT_HOST_LIB") or os.path.join(_PKG, "lib", "
 
 STAGE_PRE, STAGE_ATT, STAGE_POST, STAGE_CLS = 0, 1, 2, 3
 FWD_ALL, FWD_PRE, FWD_ATT, FWD_POST, FWD_CLS = 0, 1, 2, 3, 4
-FLAG_FUSED, FLAG_CLS, FLAG_PAGED, FLAG_UNFUSED_PROJ = 1, 2, 4, 8
+FLAG_FUSED, FLAG_CLS, FLAG_PAGED, FLAG_UNFUSED_PROJ, FLAG_BALANCED, FLAG_NOT_BALANCED = 1, 2, 4, 8, 16, 32
 
 # layer tensors in file order (rms_att_weight, wq, wkv, wo, rms_ffn_weight, w1, w2, w3)
 LAYER_TENSORS = ("rms_att_weight", "wq", "wkv", "wo", "rms_ffn_weight", "w1", "w2", "w3")
@@ -95,10 +95,12 @@ class Stage:
 
     def __init__(self, config: str, dtype: str, first_layer: int, n_hosted: int, concurrency: int,
                  max_contexts: int, fused: bool = True, with_cls: bool = False, paged: bool = False,
-                 seed: int = 1, weight_std: float = 0.02, fused_projections: bool = True):
+                 seed: int = 1, weight_std: float = 0.02, fused_projections: bool = True, balanced=None):
+        # balanced: decode attention over equal runs of keys always (True) / never (False); None: where a step's lengths call for it
         self.np_dtype = np.float16 if dtype == "f16" else np.float32
         flags = ((FLAG_FUSED if fused else 0) | (FLAG_CLS if with_cls else 0) | (FLAG_PAGED if paged else 0)
-                 | (0 if fused_projections else FLAG_UNFUSED_PROJ))
+                 | (0 if fused_projections else FLAG_UNFUSED_PROJ)
+                 | (0 if balanced is None else FLAG_BALANCED if balanced else FLAG_NOT_BALANCED))
         self._h = host_lib().glint_stage_create(config.encode(), 0 if dtype == "f16" else 1, first_layer, n_hosted,
                                                 concurrency, max_contexts, flags, seed, weight_std)
         if not self._h:
