@@ -787,11 +787,17 @@ __global__ __launch_bounds__( 256 ) void attn_decode_balanced_kernel( const __ha
   }
 }
 
-// block <-> (query head, context), thread <-> output dim: combines the pieces of a context that the cuts divided
+// block <-> (kv head, context), thread <-> (query head of the kv head, output dim): combines the pieces of a context that the
+// cuts divided.  Most blocks of a launch find their context in one piece and leave at once, so there are few and large ones.
 template<int G>
-__global__ __launch_bounds__( 128 ) void attn_merge_balanced_kernel( BalancedPlan plan, Partials part, __half* __restrict__ xb, uint32_t n_heads, uint32_t batch, uint32_t wgs )
+__global__ __launch_bounds__( ( G < 8 ? G : 8 ) * 128 ) void attn_merge_balanced_kernel( BalancedPlan plan,
+                                                                                       Partials part,
+                                                                                       __half* __restrict__ xb,
+                                                                                       uint32_t n_heads,
+                                                                                       uint32_t batch,
+                                                                                       uint32_t wgs )
 {
-  const uint32_t head = blockIdx.x;
+  const uint32_t kv = blockIdx.x;
   const uint32_t ctx = blockIdx.y;
   const uint32_t p0 = plan.prefix[ctx], p1 = plan.prefix[ctx + 1], run = plan.header[0];
   if ( p1 == p0 ) {
@@ -801,44 +807,45 @@ __global__ __launch_bounds__( 128 ) void attn_merge_balanced_kernel( BalancedPla
   if ( w0 == w1 ) {
     return; // one piece: written by the work-group that ran it
   }
-  const uint32_t kv = head / G, hd = head % G;
-  const uint64_t slot0 = balanced_slot( kv / 4, batch + wgs, ctx, w0, kv % 4, G, hd );
-  const uint64_t step = 4ull * G; // slots from one work-group's piece to the next one's
   const uint32_t n = w1 - w0 + 1;
+  const uint64_t step = 4ull * G; // slots from one work-group's piece to the next one's
   const float2* ml = reinterpret_cast<const float2*>( part.ml );
-  const uint32_t d = threadIdx.x; // head size 128 = block size
+  const uint32_t d = threadIdx.x % HS;
   constexpr uint32_t MERGE_BATCH = 4;
-  float2 st[MERGE_BATCH];
-  float o[MERGE_BATCH];
+  for ( uint32_t hd = threadIdx.x / HS; hd < G; hd += blockDim.x / HS ) { // one turn except at gqa 16
+    const uint64_t slot0 = balanced_slot( kv / 4, batch + wgs, ctx, w0, kv % 4, G, hd );
+    float2 st[MERGE_BATCH];
+    float o[MERGE_BATCH];
 #pragma unroll
-  for ( uint32_t u = 0; u < MERGE_BATCH; u++ ) {
-    const uint64_t slot = slot0 + min( u, n - 1 ) * step;
-    st[u] = ml[slot];
-    o[u] = part.out[slot * HS + d];
-  }
-  float m = -INFINITY;
+    for ( uint32_t u = 0; u < MERGE_BATCH; u++ ) { // a piece past the last reads the last again and gets weight zero
+      const uint64_t slot = slot0 + min( u, n - 1 ) * step;
+      st[u] = ml[slot];
+      o[u] = part.out[slot * HS + d];
+    }
+    float m = -INFINITY;
 #pragma unroll
-  for ( uint32_t u = 0; u < MERGE_BATCH; u++ ) {
-    m = fmaxf( m, st[u].x );
-  }
-  for ( uint32_t k = MERGE_BATCH; k < n; k++ ) {
-    m = fmaxf( m, ml[slot0 + k * step].x );
-  }
-  float l = 0.0f, acc = 0.0f;
+    for ( uint32_t u = 0; u < MERGE_BATCH; u++ ) {
+      m = fmaxf( m, st[u].x );
+    }
+    for ( uint32_t k = MERGE_BATCH; k < n; k++ ) {
+      m = fmaxf( m, ml[slot0 + k * step].x );
+    }
+    float l = 0.0f, acc = 0.0f;
 #pragma unroll
-  for ( uint32_t u = 0; u < MERGE_BATCH; u++ ) {
-    const float wgt = u < n ? fast_exp2( st[u].x - m ) : 0.0f;
-    l += st[u].y * wgt;
-    acc += o[u] * wgt;
+    for ( uint32_t u = 0; u < MERGE_BATCH; u++ ) {
+      const float wgt = u < n ? fast_exp2( st[u].x - m ) : 0.0f;
+      l += st[u].y * wgt;
+      acc += o[u] * wgt;
+    }
+    for ( uint32_t k = MERGE_BATCH; k < n; k++ ) {
+      const uint64_t slot = slot0 + k * step;
+      const float2 e = ml[slot];
+      const float wgt = fast_exp2( e.x - m );
+      l += e.y * wgt;
+      acc += part.out[slot * HS + d] * wgt;
+    }
+    xb[( (uint64_t)ctx * n_heads + (uint64_t)kv * G + hd ) * HS + d] = __float2half_rn( acc * ( 1.0f / l ) );
   }
-  for ( uint32_t k = MERGE_BATCH; k < n; k++ ) {
-    const uint64_t slot = slot0 + k * step;
-    const float2 e = ml[slot];
-    const float wgt = fast_exp2( e.x - m );
-    l += e.y * wgt;
-    acc += part.out[slot * HS + d] * wgt;
-  }
-  xb[( (uint64_t)ctx * n_heads + head ) * HS + d] = __float2half_rn( acc * ( 1.0f / l ) );
 }
 
 // =================================================================================================
@@ -979,8 +986,8 @@ void launch_balanced( const BalancedLayout& y, hipStream_t st, const void* q, co
 {
   attn_decode_balanced_kernel<G><<<y.head_groups * y.wgs, 256, 0, st>>>( static_cast<const __half*>( q ), reinterpret_cast<const __half* const*>( rows ), plan,
                                                                         part, static_cast<__half*>( xb ), s->n_kv_heads, (uint32_t)batch, y.wgs, scale );
-  attn_merge_balanced_kernel<G><<<dim3( s->n_heads, (unsigned)batch ), 128, 0, st>>>( plan, part, static_cast<__half*>( xb ), s->n_heads, (uint32_t)batch,
-                                                                                      y.wgs );
+  attn_merge_balanced_kernel<G><<<dim3( s->n_kv_heads, (unsigned)batch ), ( G < 8 ? G : 8 ) * 128, 0, st>>>( plan, part, static_cast<__half*>( xb ), s->n_heads,
+                                                                                                             (uint32_t)batch, y.wgs );
 }
 
 } // namespace
