@@ -593,6 +593,8 @@ def main():
     ap.add_argument("--concept-path", action="store_true", help="time the named decode workload through the reference's op sequence only")
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="also run a plain D2D copy of this many MiB (reference point for profiler byte counters)")
+    ap.add_argument("--library-rows", type=int, default=-1,
+                    help="measurement hook: rows from which plain products go to the vendor's GEMM library (0: never; default: the library's own setting)")
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -605,6 +607,10 @@ def main():
         from glinthawk_amd import ops
         ops.init(0)
         calibration_copy(args.calibration_copy_mib << 20)
+    if args.library_rows >= 0:
+        from glinthawk_amd import _lib, ops
+        ops.init(0)
+        _lib.check(_lib.lib().gh_gemm_set_library_rows(args.library_rows))
     if args.attn_variant != "auto":
         from glinthawk_amd import _lib, ops
         ops.init(0)

@@ -94,6 +94,7 @@ SIGNATURES = {
     "gh_silu": (_i, [_vp, _vp, _u64, _u64, _i, _vp]),
     "gh_argmax": (_i, [_vp, _vp, _vp, _u64, _u64, _i, _vp]),
     "gh_gemm_set_tuning": (_i, [_i, _i, _i]),
+    "gh_gemm_set_library_rows": (_i, [_u64]),
     "gh_matmul_fuses_many_rows": (_i, [_u64, _u64, _u64, _i]),
     "gh_gemm_stream_plan": (_i, [_u64, _u64, _u64, _vp, _vp, _vp]),
     "gh_matmul": (_i, [_vp, _vp, _vp, _u64, _u64, _u64, _i, _vp]),

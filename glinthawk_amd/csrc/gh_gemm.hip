@@ -39,6 +39,7 @@ int gemm_tile_launch( __half* xout, float* partial, const __half* x, const __hal
 namespace {
 
 int g_force_kernel = 0; // 0 auto, 1 small tiled kernel of this file, 2 streaming kernel, 3 large tile kernel
+uint64_t g_library_rows = 768; // plain products of this many rows and more go to the vendor's GEMM library (measurement hook: gh_gemm_set_library_rows)
 
 typedef _Float16 f16x8 __attribute__( ( ext_vector_type( 8 ) ) );
 typedef float f32x4 __attribute__( ( ext_vector_type( 4 ) ) );
@@ -398,6 +399,15 @@ int gemm_partials( void* xout, const void* x, const void* w, uint64_t s, uint64_
 
 } // namespace gh
 
+namespace gh {
+// whether a plain product goes to the vendor's library (gh_gemm_lib.hip)
+bool gemm_library_wanted( uint64_t s, uint64_t r, uint64_t b, gh_dtype dt, const void* x, const void* w, const void* xout )
+{
+  const bool aligned = ( ( reinterpret_cast<uintptr_t>( x ) | reinterpret_cast<uintptr_t>( w ) | reinterpret_cast<uintptr_t>( xout ) ) & 15u ) == 0;
+  return dt == GH_F16 && g_force_kernel == 0 && g_library_rows > 0 && b >= g_library_rows && s % 8 == 0 && r % 8 == 0 && aligned;
+}
+} // namespace gh
+
 using namespace gh;
 
 extern "C" {
@@ -407,6 +417,12 @@ int gh_gemm_set_tuning( int kernel, int target_workgroups, int tile_rows )
   g_force_kernel = kernel;
   gemm_stream_tuning( target_workgroups, 0 );
   gemm_tile256_tuning( tile_rows );
+  return GH_OK;
+}
+
+int gh_gemm_set_library_rows( uint64_t rows )
+{
+  g_library_rows = rows;
   return GH_OK;
 }
 
@@ -438,6 +454,12 @@ int gh_matmul_pair( void* xout_a, void* xout_b, const void* x, const void* w, ui
   const uint64_t elem = dt == GH_F16 ? 2 : 4;
   const uint64_t r = r_a + r_b;
   GH_REQUIRE( s > 0 && s <= 0x7fffffffull && r <= 0x7fffffffull && b <= 0x7fffffffull, "gh_matmul_pair: bad shape" );
+  if ( r_a > 0 && r_b > 0 && gemm_library_wanted( s, r_a, b, dt, x, w, xout_a ) && gemm_library_wanted( s, r_b, b, dt, x, w, xout_b ) ) {
+    if ( int rc = gh_matmul( xout_a, x, w, s, r_a, b, dt, stream ) ) { // the library's kernels cut their work finer than whole tiles
+      return rc;
+    }
+    return gh_matmul( xout_b, x, static_cast<const char*>( w ) + r_a * s * elem, s, r_b, b, dt, stream );
+  }
   // many rows: one launch of the large tile kernel whose work-groups store to the matrix their rows belong to, so that the two
   // products fill their rounds together (a product of 2048 rows alone leaves most of the chip idle)
   if ( dt == GH_F16 && g_force_kernel == 0 && r_a > 0 && r_b > 0 && r_a % 8 == 0 && r_b % 8 == 0 && gemm_tile256_applicable( s, r, b, x, w, xout_a )
@@ -471,6 +493,15 @@ int gh_matmul( void* xout, const void* x, const void* w, uint64_t s, uint64_t r,
   GH_REQUIRE( xout && x && w, "gh_matmul: NULL pointer" );
   GH_REQUIRE( s > 0 && s <= 0x7fffffffull && r <= 0x7fffffffull && b <= 0x7fffffffull, "gh_matmul: bad shape" );
   hipStream_t st = as_stream( stream );
+  if ( gemm_library_wanted( s, r, b, dt, x, w, xout ) ) { // a plain product of many rows
+    bool done = false;
+    if ( int rc = gemm_library( xout, x, w, s, r, b, st, &done ) ) {
+      return rc;
+    }
+    if ( done ) {
+      return GH_OK;
+    }
+  }
   if ( const uint64_t b1 = gemm_token_split( s, r, b, dt, x, w, xout ) ) { // two products along the tokens
     const uint64_t elem = 2;
     if ( int rc = gh_matmul( xout, x, w, s, r, b1, dt, stream ) ) {

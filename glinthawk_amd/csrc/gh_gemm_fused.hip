@@ -347,6 +347,24 @@ int gh_matmul_accum( void* residual, const void* x, const void* w, uint64_t s, u
   GH_REQUIRE( residual != nullptr, "gh_matmul_accum: NULL residual" );
   GH_REQUIRE( ( norm_out == nullptr ) == ( norm_weight == nullptr ), "gh_matmul_accum: norm_out and norm_weight go together" );
   hipStream_t st = as_stream( stream );
+  bool done = false;
+  // many rows (prompt tokens), the product by the vendor's library where the dispatcher sends plain products there: the rounded
+  // product, then the reference's own next ops on it (accum, rmsnorm) -- the same roundings as fused
+  if ( gemm_library_wanted( s, r, b, dt, x, w, residual ) ) {
+    void* product = nullptr;
+    if ( int rc = stream_scratch( st, SCRATCH_PRODUCT, b * r * sizeof( __half ), 64ull << 20, &product ) ) {
+      return rc;
+    }
+    if ( int rc = gemm_library( product, x, w, s, r, b, st, &done ) ) {
+      return rc;
+    }
+    if ( done ) {
+      if ( int rc = gh_accum( residual, product, r, b, dt, stream ) ) {
+        return rc;
+      }
+      return norm_out != nullptr ? gh_rmsnorm( norm_out, residual, norm_weight, r, b, dt, stream ) : GH_OK;
+    }
+  }
   if ( const uint64_t b1 = gemm_token_split( s, r, b, dt, x, w, residual ) ) { // two products along the tokens (rows are independent)
     const uint64_t elem = 2;
     if ( int rc = gh_matmul_accum( residual, x, w, s, r, b1, norm_out, norm_weight, dt, stream ) ) {
@@ -355,9 +373,9 @@ int gh_matmul_accum( void* residual, const void* x, const void* w, uint64_t s, u
     return gh_matmul_accum( static_cast<char*>( residual ) + b1 * r * elem, static_cast<const char*>( x ) + b1 * s * elem, w, s, r, b - b1,
                             norm_out ? static_cast<char*>( norm_out ) + b1 * r * elem : nullptr, norm_weight, dt, stream );
   }
-  // many rows (prompt tokens): the residual is added in the tile kernel's epilogue, no fp32 partials;
+  // many rows: the residual is added in the tile kernel's epilogue, no fp32 partials;
   // the norm of the new residual, when asked for, is the plain row kernel
-  bool done = false;
+  done = false;
   if ( int rc = gemm_tile_epilogue_launch( residual, x, w, s, r, b, dt, 1, st, &done ) ) {
     return rc;
   }

@@ -151,6 +151,12 @@ int gh_argmax( uint32_t* out_host, uint32_t* out_dev, const void* v, uint64_t n,
  * streaming kernel's K split is balanced for (<= 0 keeps the current value; the default is the device's own count); weight rows per work-group of the
  * 256-token tile kernel: 256, 384, or 0 for the library's choice */
 int gh_gemm_set_tuning( int kernel, int target_workgroups, int tile_rows );
+/* Plain f16 products (gh_matmul, the two of gh_matmul_pair, the product inside gh_matmul_accum and gh_matmul_silu_gate where no
+ * kernel of this library fuses it) of `rows` activation rows and more go to the vendor's GEMM library, as every product of the
+ * reference's GPU target does (cublasGemmEx, arch/cuda/common/ops.cuh:666-700); 0: never.  Default 768 (measured: from there on the library's kernels are the faster ones for nearly every shape of the 13B and
+ * 70B models; below, the split-K tile kernel and the fused epilogues of this library are).  A forced kernel
+ * (gh_gemm_set_tuning) also keeps the library out. */
+int gh_gemm_set_library_rows( uint64_t rows );
 /* host-only query: 1 when gh_matmul_accum runs a product of this shape (16-byte aligned operands) in the large tile kernel with the residual added
  * in its epilogue, i.e. without fp32 partial sums of (b, r): the caller's test for taking the fused call on many rows */
 int gh_matmul_fuses_many_rows( uint64_t s, uint64_t r, uint64_t b, gh_dtype dt );
