@@ -48,3 +48,13 @@ def pytest_sessionfinish(session, exitstatus):
             w[0], w[1], w[2], w[3] = max(w[0], r16), max(w[1], r32), max(w[2], rs), w[3] + 1
         for key, (r16, r32, rs, n) in worst.items():
             f.write(f"{key}: max over {n} outputs  {r16:.3e} | {r32:.3e} | {rs:.3e}\n")
+
+
+@pytest.fixture(params=["vendor-library", "own-kernels"])
+def product_route(request):
+    """Plain products of many rows both ways: through the vendor's GEMM library (the default from 768 rows on) and on
+    the tile kernels of this library."""
+    from glinthawk_amd import _lib
+    _lib.check(_lib.lib().gh_gemm_set_library_rows(768 if request.param == "vendor-library" else 0))
+    yield request.param
+    _lib.check(_lib.lib().gh_gemm_set_library_rows(768))

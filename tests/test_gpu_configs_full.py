@@ -96,7 +96,7 @@ def oracle_kv_rows(cfg, w, x_rows, positions):
 
 
 @pytest.mark.timeout(900)
-def test_config3_llama13b_prefill_8x2048_then_decode():
+def test_config3_llama13b_prefill_8x2048_then_decode(product_route):
     cfg = O.Config(dim=5120, n_layers=40, n_heads=40, n_kv_heads=40, hidden_dim=13824, seq_len=4096, attention_rounds=2)
     layer, batch, T = 12, 8, 2048
     ops.init(0)

@@ -24,7 +24,7 @@ def _init():
                                    # enough 256-token tiles: the residual is added in the large tile kernel's epilogue (f16, r % 8 == 0)
                                    (768, 8192, 16384), (2048, 512, 6152), (3000, 1024, 6144), (2300, 512, 8192),
                                    (2048, 512, 6150)])          # r % 8 != 0: fp32 partials and the row kernel
-def test_matmul_accum_and_norm(dt, b, s, r):
+def test_matmul_accum_and_norm(dt, b, s, r, product_route):
     g = torch.Generator(device="cuda").manual_seed(1)
     x = torch.randn((b, s), generator=g, device="cuda").to(dt)
     w = (torch.randn((r, s), generator=g, device="cuda") / s ** 0.5).to(dt)

@@ -276,7 +276,7 @@ def test_matmul_some_hundred_rows(b, s, r):
 # many rows whose 256-token tiles would leave the last round nearly empty: the library runs such a product as two products along
 # the tokens (here 2048 + 252 and 4096 + 404 tokens); one-hot activations, every output is one weight
 @pytest.mark.parametrize("b,s,r", [(2300, 512, 8192), (4500, 256, 8192), (2300, 512, 8200)])
-def test_matmul_token_split_one_hot(b, s, r):
+def test_matmul_token_split_one_hot(b, s, r, product_route):
     w = torch.arange(r * s, dtype=torch.float32, device="cuda").reshape(r, s).remainder(1000).half()
     x = torch.zeros((b, s), dtype=torch.float16, device="cuda")
     cols = torch.tensor([(7919 * i + 3) % s for i in range(b)], device="cuda")
@@ -290,7 +290,7 @@ def test_matmul_token_split_one_hot(b, s, r):
 @pytest.mark.parametrize("dt", ["f16", "f32"])
 @pytest.mark.parametrize("b,s,ra,rb", [(3, 256, 64, 32), (300, 512, 512, 200), (2048, 256, 8192, 2048), (2300, 256, 8192, 2048),
                                        (1500, 320, 5120, 10240), (1024, 256, 8200, 2056), (1024, 256, 8196, 2052)])
-def test_matmul_pair(dt, b, s, ra, rb):
+def test_matmul_pair(dt, b, s, ra, rb, product_route):
     if dt == "f32" and b > 300:
         pytest.skip("the fp32 route is the same two calls at every size")
     tdt = torch.float16 if dt == "f16" else torch.float32
