@@ -427,7 +427,8 @@ int gh_matmul_silu_gate( void* hb, const void* x, const void* w13, uint64_t s, u
   // route below leaves for its gate kernel are stored from the accumulator registers, 16 bytes to each of 32 lines per
   // instruction, and are twice the bytes: at 256 rows of the 70B shape 277 + 19 us against 257 + 12.  Same roundings either way
   // (each factor to DType, then the gate).
-  if ( dt == GH_F16 && hidden_dim % 8 == 0 && gemm_tile_epilogue_applicable( s, 2 * hidden_dim, b, dt, x, w13, hb ) ) {
+  if ( dt == GH_F16 && hidden_dim % 8 == 0
+       && ( gemm_tile_epilogue_applicable( s, 2 * hidden_dim, b, dt, x, w13, hb ) || gemm_library_wanted( s, hidden_dim, b, dt, x, w13, hb ) ) ) {
     void* factor = nullptr;
     if ( int rc = stream_scratch( st, SCRATCH_GATE_FACTOR, b * hidden_dim * sizeof( __half ), 16ull << 20, &factor ) ) {
       return rc;
