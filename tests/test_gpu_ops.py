@@ -311,6 +311,21 @@ def test_matmul_pair(dt, b, s, ra, rb, product_route):
     assert err.max().item() < 2e-2 and (err.mean() / want.abs().mean()).item() < 1e-3
 
 
+def test_matmul_many_rows_repeatable(product_route):
+    # the same product twice, other work in between: bit-identical results on either route (no sums in arrival order)
+    b, s, r = 3328, 1024, 2560
+    g = torch.Generator(device="cuda").manual_seed(77)
+    x = torch.randn((b, s), generator=g, device="cuda").half()
+    w = (torch.randn((r, s), generator=g, device="cuda") / s ** 0.5).half()
+    first = ops.matmul(x, w)
+    ops.matmul(torch.flip(x, dims=[0]).contiguous(), w)
+    again = ops.matmul(x, w)
+    assert torch.equal(first, again)
+    want = x.float() @ w.float().t()
+    err = (first.float() - want).abs()
+    assert err.max().item() < 2e-2 and (err.mean() / want.abs().mean()).item() < 1e-3
+
+
 def test_matmul_layout_one_hot():
     s, r = 256, 192
     w = torch.arange(r * s, dtype=torch.float32).reshape(r, s).remainder(1000).half().cuda()
