@@ -8,7 +8,10 @@
 //                 two waves per SIMD.
 //                 With one wave per SIMD (four waves of 64 x 256, the first version of this kernel)
 //                 every stall of a memory or LDS instruction also holds back that wave's MFMAs:
-//                 0.82-0.97 PFLOP/s however the operands were fetched.
+//                 0.82-0.97 PFLOP/s however the operands were fetched.  Four waves of 128 x 128 (256
+//                 accumulator registers, a third less LDS traffic per flop than 64 x 128, the step's
+//                 barrier in front of the last 16-k group with the next stage's first fragments
+//                 requested behind it): 0.68-0.79.
 //   384 rows    bring 80 KiB per 64 k for 1.5 x the flops of 256 rows (64 KiB) and fill the LDS
 //                 (2 x 80 KiB) and the registers (one set of MFMA operands instead of two); a round
 //                 of them takes 1.24-1.44 x as long, so they win where their rounds fit the shape
