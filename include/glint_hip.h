@@ -302,7 +302,9 @@ int gh_attn_prefill( const void* q, const void* const* layer_rows_dev, const uin
 /* Timing hooks for the benchmark: HIP events recorded on `stream` around the two kernels of
  * gh_attn_decode.  gh_attn_timing_read() synchronises and returns, accumulated since
  * gh_attn_timing_reset(): milliseconds in the split-K attention kernel, milliseconds in the merge
- * kernel (0 when no split was needed) and the number of gh_attn_decode calls sampled. */
+ * kernel (0 when no split was needed) and the number of gh_attn_decode calls sampled.  on = 2: events only in front of and
+ * behind the pair of kernels, nothing between them, as the pair runs in production (an event record holds the next kernel
+ * back by a few microseconds); the whole span is then returned as kernel_ms and merge_ms is 0.  Read before changing the mode. */
 int gh_attn_timing_enable( int on );
 int gh_attn_timing_reset( void );
 int gh_attn_timing_read( double* kernel_ms, double* merge_ms, uint64_t* launches );

@@ -725,6 +725,38 @@ def test_fused_balanced_bound_below_the_true_maximum_truncates_and_bad_arguments
     assert L.gh_attn_decode_balanced(None, table.data_ptr(), a.data_ptr(), batch, 299, C.byref(s), GH_F16, ws.data_ptr(), ws.numel(), None) == GH_ERR_INVALID
 
 
+def test_attention_timing_hooks_count_calls_in_both_modes():
+    import ctypes as C
+    from glinthawk_amd import _lib
+    L = _lib.lib()
+    shape = GQA8
+    batch = 4
+    arena = Arena(shape, batch, torch.float16, seed=81)
+    table = ops.row_table([arena.layer_ptr(i) for i in range(batch)])
+    pos = torch.tensor([699, 650, 600, 512], dtype=torch.int32, device="cuda")
+    q = torch.randn((batch, shape.dim), dtype=torch.float16, device="cuda")
+    xb = torch.zeros_like(q)
+    k_ms, m_ms, n = C.c_double(0), C.c_double(0), C.c_uint64(0)
+    spans = {}
+    try:
+        for mode in (1, 2):
+            _lib.check(L.gh_attn_timing_enable(mode))
+            _lib.check(L.gh_attn_timing_reset())
+            for _ in range(5):
+                ops.attn_decode(q, table, pos, xb, 699, shape, variant=GH_ATTN_MFMA)
+            _lib.check(L.gh_attn_timing_read(C.byref(k_ms), C.byref(m_ms), C.byref(n)))
+            assert n.value == 5 and k_ms.value > 0
+            spans[mode] = (k_ms.value, m_ms.value)
+    finally:
+        _lib.check(L.gh_attn_timing_enable(0))
+    assert spans[1][1] > 0          # split kernel and merge timed apart
+    assert spans[2][1] == 0         # one span over the pair
+    _lib.check(L.gh_attn_timing_reset())
+    ops.attn_decode(q, table, pos, xb, 699, shape, variant=GH_ATTN_MFMA)   # off: nothing recorded
+    _lib.check(L.gh_attn_timing_read(C.byref(k_ms), C.byref(m_ms), C.byref(n)))
+    assert n.value == 0
+
+
 def test_fused_variants_agree():
     # the three kernels on the same input: differences are rounding only
     shape = GQA8
