@@ -214,21 +214,23 @@ __global__ __launch_bounds__( 256 ) void attn_merge_kernel( Partials part,
 // =================================================================================================
 // valu kernel: lane = (r = lane / 16: token within a group of 4, c = lane % 16: 16-byte chunk of the head row)
 // =================================================================================================
+// One (context, kv head) stream over the tokens [t_begin, t_end), t_begin < t_end, for the G query heads of the kv head: running
+// maxima m (log2 domain), sums l and the unnormalised output acc[g][e] = O[head g][dim 8*c + e], the same in the four lanes
+// that share a chunk c.  `rot` moves the tile the walk starts at.
 template<int G>
-__global__ __launch_bounds__( 256 ) void attn_decode_valu_kernel( const __half* __restrict__ q,
-                                                                  const __half* const* __restrict__ layer_rows,
-                                                                  const uint32_t* __restrict__ pos,
-                                                                  Partials part,
-                                                                  __half* __restrict__ xb,
-                                                                  uint32_t n_kv_heads,
-                                                                  uint32_t chunk,
-                                                                  uint32_t max_splits,
-                                                                  float scale_log2e )
+__device__ __forceinline__ void valu_stream_range( const __half* __restrict__ q,
+                                                   const __half* base,
+                                                   const uint32_t ctx,
+                                                   const uint32_t h,
+                                                   const uint32_t t_begin,
+                                                   const uint32_t t_end,
+                                                   const uint32_t rot,
+                                                   const uint32_t n_kv_heads,
+                                                   const float scale_log2e,
+                                                   float ( &m )[G],
+                                                   float ( &l )[G],
+                                                   float ( &acc )[G][8] )
 {
-  const WaveJob job = wave_job( layer_rows, pos, n_kv_heads, chunk, max_splits );
-  if ( !job.valid ) {
-    return; // wave-uniform; the kernel has no block-level barrier
-  }
   const uint32_t lane = threadIdx.x & 63;
   const uint32_t c = lane & 15;
   const uint32_t r = lane >> 4;
@@ -238,14 +240,13 @@ __global__ __launch_bounds__( 256 ) void attn_decode_valu_kernel( const __half* 
 
   uint4 qr[G];
   {
-    const __half* qp = q + ( (uint64_t)job.ctx * n_heads + (uint64_t)job.h * G ) * HS + 8 * c;
+    const __half* qp = q + ( (uint64_t)ctx * n_heads + (uint64_t)h * G ) * HS + 8 * c;
 #pragma unroll
     for ( int g = 0; g < G; g++ ) {
       qr[g] = load16( qp + g * HS );
     }
   }
 
-  float m[G], l[G], acc[G][8];
 #pragma unroll
   for ( int g = 0; g < G; g++ ) {
     m[g] = -INFINITY;
@@ -256,19 +257,19 @@ __global__ __launch_bounds__( 256 ) void attn_decode_valu_kernel( const __half* 
     }
   }
 
-  const __half* kp = job.base + (uint64_t)job.h * HS + 8 * c;
+  const __half* kp = base + (uint64_t)h * HS + 8 * c;
   const uint4 zero4 = make_uint4( 0, 0, 0, 0 );
 
   // 16-token tiles in rotated order, a different starting tile per block (see the mfma kernel)
-  const uint32_t n_tiles = ( job.t_end - job.t_begin + 15 ) / 16;
-  uint32_t tile_i = ( ( job.ctx * 5u + job.split * 3u ) * 7u ) % n_tiles;
-  uint32_t t0 = job.t_begin + 16 * tile_i;
+  const uint32_t n_tiles = ( t_end - t_begin + 15 ) / 16;
+  uint32_t tile_i = ( ( ctx * 5u + rot * 3u ) * 7u ) % n_tiles;
+  uint32_t t0 = t_begin + 16 * tile_i;
 
   uint4 kn[4], vn[4]; // prefetched block
 #pragma unroll
   for ( int j = 0; j < 4; j++ ) {
     const uint32_t tok = t0 + 4 * j + r;
-    const bool ok = tok < job.t_end;
+    const bool ok = tok < t_end;
     const __half* row = kp + (uint64_t)tok * row_elems;
     kn[j] = ok ? load16_stream( row ) : zero4;
     vn[j] = ok ? load16_stream( row + v_off ) : zero4;
@@ -276,7 +277,7 @@ __global__ __launch_bounds__( 256 ) void attn_decode_valu_kernel( const __half* 
 
   for ( uint32_t it = 0; it < n_tiles; it++ ) {
     tile_i = tile_i + 1 == n_tiles ? 0 : tile_i + 1;
-    const uint32_t t_next = job.t_begin + 16 * tile_i;
+    const uint32_t t_next = t_begin + 16 * tile_i;
     const bool more = it + 1 < n_tiles;
     uint4 kc[4], vc[4];
 #pragma unroll
@@ -288,7 +289,7 @@ __global__ __launch_bounds__( 256 ) void attn_decode_valu_kernel( const __half* 
 #pragma unroll
     for ( int j = 0; j < 4; j++ ) {
       const uint32_t tok = t_next + 4 * j + r;
-      const bool ok = more && tok < job.t_end;
+      const bool ok = more && tok < t_end;
       const __half* row = kp + (uint64_t)tok * row_elems;
       kn[j] = ok ? load16_stream( row ) : zero4;
       vn[j] = ok ? load16_stream( row + v_off ) : zero4;
@@ -297,7 +298,7 @@ __global__ __launch_bounds__( 256 ) void attn_decode_valu_kernel( const __half* 
     float s[4][G];
 #pragma unroll
     for ( int j = 0; j < 4; j++ ) {
-      const bool ok = t0 + 4 * j + r < job.t_end;
+      const bool ok = t0 + 4 * j + r < t_end;
 #pragma unroll
       for ( int g = 0; g < G; g++ ) {
         const float d = row16_sum( dot8( kc[j], qr[g], 0.0f ) );
@@ -354,6 +355,31 @@ __global__ __launch_bounds__( 256 ) void attn_decode_valu_kernel( const __half* 
     m[g] = mm;
     l[g] = ll;
   }
+
+}
+
+template<int G>
+__global__ __launch_bounds__( 256 ) void attn_decode_valu_kernel( const __half* __restrict__ q,
+                                                                  const __half* const* __restrict__ layer_rows,
+                                                                  const uint32_t* __restrict__ pos,
+                                                                  Partials part,
+                                                                  __half* __restrict__ xb,
+                                                                  uint32_t n_kv_heads,
+                                                                  uint32_t chunk,
+                                                                  uint32_t max_splits,
+                                                                  float scale_log2e )
+{
+  const WaveJob job = wave_job( layer_rows, pos, n_kv_heads, chunk, max_splits );
+  if ( !job.valid ) {
+    return; // wave-uniform; the kernel has no block-level barrier
+  }
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t c = lane & 15;
+  const uint32_t r = lane >> 4;
+  const uint32_t n_heads = n_kv_heads * G;
+
+  float m[G], l[G], acc[G][8];
+  valu_stream_range<G>( q, job.base, job.ctx, job.h, job.t_begin, job.t_end, job.split, n_kv_heads, scale_log2e, m, l, acc );
 
   if ( r == 0 ) {
 #pragma unroll
@@ -700,8 +726,9 @@ __device__ __forceinline__ uint64_t balanced_slot( uint32_t g, uint32_t pieces, 
   return ( ( (uint64_t)g * pieces + c + w ) * 4 + h_local ) * G + hd;
 }
 
-// grid: work-groups per head group x head groups; wave <-> kv head of the group
-template<int G>
+// grid: work-groups per head group x head groups; wave <-> kv head of the group.  MFMA: the streaming loop of the mfma kernel
+// (gqa 2 and more), else that of the valu kernel (one query head per kv head).
+template<int G, bool MFMA>
 __global__ __launch_bounds__( 256 ) void attn_decode_balanced_kernel( const __half* __restrict__ q,
                                                                       const __half* const* __restrict__ layer_rows,
                                                                       BalancedPlan plan,
@@ -743,38 +770,71 @@ __global__ __launch_bounds__( 256 ) void attn_decode_balanced_kernel( const __ha
     const uint32_t t_end = min( plan.length[c], ( piece_end - p0 ) * BAL_CHUNK );
     const bool whole = at == p0 && piece_end == p1;
     if ( base != nullptr && t_begin < t_end ) {
-      f32x4 acc[8];
-      float m, l;
-      mfma_stream_range<G>( q, base, c, h, t_begin, t_end, w, n_kv_heads, scale_log2e, s_k[wave], acc, m, l );
-      l += __shfl_xor( l, 16, WAVE );
-      l += __shfl_xor( l, 32, WAVE );
+      if constexpr ( MFMA ) {
+        f32x4 acc[8];
+        float m, l;
+        mfma_stream_range<G>( q, base, c, h, t_begin, t_end, w, n_kv_heads, scale_log2e, s_k[wave], acc, m, l );
+        l += __shfl_xor( l, 16, WAVE );
+        l += __shfl_xor( l, 32, WAVE );
 #pragma unroll
-      for ( int i = 0; i < 4; i++ ) {
-        const uint32_t hd = 4 * g4 + i;
-        const float mh = __shfl( m, (int)hd, WAVE );
-        const float lh = __shfl( l, (int)hd, WAVE );
-        if ( hd < G ) {
-          if ( whole ) {
-            const uint64_t head = (uint64_t)c * n_heads + (uint64_t)h * G + hd;
-            const float inv = 1.0f / lh;
-            union
-            {
-              uint4 raw;
-              __half h[8];
-            } o;
+        for ( int i = 0; i < 4; i++ ) {
+          const uint32_t hd = 4 * g4 + i;
+          const float mh = __shfl( m, (int)hd, WAVE );
+          const float lh = __shfl( l, (int)hd, WAVE );
+          if ( hd < G ) {
+            if ( whole ) {
+              const uint64_t head = (uint64_t)c * n_heads + (uint64_t)h * G + hd;
+              const float inv = 1.0f / lh;
+              union
+              {
+                uint4 raw;
+                __half h[8];
+              } o;
 #pragma unroll
-            for ( int nn = 0; nn < 8; nn++ ) {
-              o.h[nn] = __float2half_rn( acc[nn][i] * inv );
+              for ( int nn = 0; nn < 8; nn++ ) {
+                o.h[nn] = __float2half_rn( acc[nn][i] * inv );
+              }
+              *reinterpret_cast<uint4*>( xb + head * HS + 8 * c16 ) = o.raw;
+            } else {
+              const uint64_t slot = balanced_slot( g, pieces, c, w, wave, G, hd );
+              float4* o = reinterpret_cast<float4*>( part.out + slot * HS + 8 * c16 );
+              o[0] = make_float4( acc[0][i], acc[1][i], acc[2][i], acc[3][i] );
+              o[1] = make_float4( acc[4][i], acc[5][i], acc[6][i], acc[7][i] );
+              if ( c16 == 0 ) {
+                part.ml[slot * 2] = mh;
+                part.ml[slot * 2 + 1] = lh;
+              }
             }
-            *reinterpret_cast<uint4*>( xb + head * HS + 8 * c16 ) = o.raw;
-          } else {
-            const uint64_t slot = balanced_slot( g, pieces, c, w, wave, G, hd );
-            float4* o = reinterpret_cast<float4*>( part.out + slot * HS + 8 * c16 );
-            o[0] = make_float4( acc[0][i], acc[1][i], acc[2][i], acc[3][i] );
-            o[1] = make_float4( acc[4][i], acc[5][i], acc[6][i], acc[7][i] );
-            if ( c16 == 0 ) {
-              part.ml[slot * 2] = mh;
-              part.ml[slot * 2 + 1] = lh;
+          }
+        }
+      } else {
+        float m[G], l[G], acc[G][8];
+        valu_stream_range<G>( q, base, c, h, t_begin, t_end, w, n_kv_heads, scale_log2e, m, l, acc );
+        if ( g4 == 0 ) { // the four lanes that share a chunk hold the same sums
+#pragma unroll
+          for ( int hd = 0; hd < G; hd++ ) {
+            if ( whole ) {
+              const uint64_t head = (uint64_t)c * n_heads + (uint64_t)h * G + hd;
+              const float inv = 1.0f / l[hd];
+              union
+              {
+                uint4 raw;
+                __half h[8];
+              } o;
+#pragma unroll
+              for ( int e = 0; e < 8; e++ ) {
+                o.h[e] = __float2half_rn( acc[hd][e] * inv );
+              }
+              *reinterpret_cast<uint4*>( xb + head * HS + 8 * c16 ) = o.raw;
+            } else {
+              const uint64_t slot = balanced_slot( g, pieces, c, w, wave, G, hd );
+              float4* o = reinterpret_cast<float4*>( part.out + slot * HS + 8 * c16 );
+              o[0] = make_float4( acc[hd][0], acc[hd][1], acc[hd][2], acc[hd][3] );
+              o[1] = make_float4( acc[hd][4], acc[hd][5], acc[hd][6], acc[hd][7] );
+              if ( c16 == 0 ) {
+                part.ml[slot * 2] = m[hd];
+                part.ml[slot * 2 + 1] = l[hd];
+              }
             }
           }
         }
@@ -889,11 +949,13 @@ Plan make_plan( uint64_t batch, uint32_t max_pos, const gh_shape* s, gh_dtype dt
     chunk = g_chunk_override;
   } else {
     // One wave per (context, kv head, split).  Measured on MI355X: 8 waves per CU (2048 in all), each
-    // streaming a long range, is the sweet spot; with 1024 or more (context, head) streams no split is
-    // needed at all and the merge kernel disappears.  Splits are never shorter than 256 tokens so
-    // that the partial traffic stays a few percent of the cache traffic.
+    // streaming a long range, is the sweet spot; with 2048 or more (context, head) streams no split is
+    // needed at all and the merge kernel disappears.  Between 1024 and 2048 streams one wave per stream
+    // leaves the CUs with 4-7 waves: ranges of 512 keys, which come in several rounds, are 3-11 % faster
+    // (7B shape, 32 contexts of 1024 keys: 90 -> 87 us; 13B, 32 of 2048: 222 -> 203).  Splits are never
+    // shorter than 256 tokens so that the partial traffic stays a few percent of the cache traffic.
     const uint64_t streams = batch * ( p.variant == GH_ATTN_GENERIC ? s->n_heads : s->n_kv_heads );
-    uint64_t splits = streams >= 1024 ? 1 : ( 2048 + streams - 1 ) / ( streams ? streams : 1 );
+    uint64_t splits = streams >= 2048 ? 1 : streams >= 1024 ? std::max<uint64_t>( 2, n_tok / 512 ) : ( 2048 + streams - 1 ) / ( streams ? streams : 1 );
     chunk = (uint32_t)( ( n_tok + splits - 1 ) / splits );
     if ( chunk < 256 ) {
       chunk = 256;
@@ -969,7 +1031,7 @@ int balanced_check( const char* who, uint64_t batch, uint32_t max_pos, const gh_
   GH_REQUIRE( shape->n_kv_heads > 0 && shape->gqa_size > 0 && shape->seq_len > 0, "%s: zero dimension", who );
   GH_REQUIRE( shape->n_heads == shape->n_kv_heads * shape->gqa_size, "%s: n_heads != n_kv_heads * gqa_size", who );
   GH_REQUIRE( shape->kv_dim == shape->n_kv_heads * shape->head_size, "%s: kv_dim != n_kv_heads * head_size", who );
-  GH_REQUIRE( shape->head_size == HS && mfma_gqa_ok( shape->gqa_size ), "%s: needs head_size 128 and gqa in {2,4,8,16}", who );
+  GH_REQUIRE( shape->head_size == HS && ( shape->gqa_size == 1 || mfma_gqa_ok( shape->gqa_size ) ), "%s: needs head_size 128 and gqa in {1,2,4,8,16}", who );
   GH_REQUIRE( max_pos < shape->seq_len, "%s: max_pos %u outside seq_len %u", who, max_pos, shape->seq_len );
   GH_REQUIRE( batch > 0 && batch <= 65535, "%s: bad batch", who );
   GH_REQUIRE( workspace != nullptr && ( reinterpret_cast<uintptr_t>( workspace ) & 15u ) == 0, "%s: workspace missing or not 16-byte aligned", who );
@@ -980,11 +1042,11 @@ int balanced_check( const char* who, uint64_t batch, uint32_t max_pos, const gh_
   return GH_OK;
 }
 
-template<int G>
+template<int G, bool MFMA>
 void launch_balanced( const BalancedLayout& y, hipStream_t st, const void* q, const void* const* rows, const BalancedPlan& plan, Partials part, void* xb,
                       const gh_shape* s, uint64_t batch, float scale )
 {
-  attn_decode_balanced_kernel<G><<<y.head_groups * y.wgs, 256, 0, st>>>( static_cast<const __half*>( q ), reinterpret_cast<const __half* const*>( rows ), plan,
+  attn_decode_balanced_kernel<G, MFMA><<<y.head_groups * y.wgs, 256, 0, st>>>( static_cast<const __half*>( q ), reinterpret_cast<const __half* const*>( rows ), plan,
                                                                         part, static_cast<__half*>( xb ), s->n_kv_heads, (uint32_t)batch, y.wgs, scale );
   attn_merge_balanced_kernel<G><<<dim3( s->n_kv_heads, (unsigned)batch ), ( G < 8 ? G : 8 ) * 128, 0, st>>>( plan, part, static_cast<__half*>( xb ), s->n_heads,
                                                                                                              (uint32_t)batch, y.wgs );
@@ -1243,10 +1305,11 @@ int gh_attn_decode_balanced( const void* q, const void* const* layer_rows_dev, v
   const float scale = LOG2E / sqrtf( (float)shape->head_size );
   hipStream_t st = as_stream( stream );
   switch ( shape->gqa_size ) {
-    case 2: launch_balanced<2>( y, st, q, layer_rows_dev, plan, part, xb, shape, batch, scale ); break;
-    case 4: launch_balanced<4>( y, st, q, layer_rows_dev, plan, part, xb, shape, batch, scale ); break;
-    case 8: launch_balanced<8>( y, st, q, layer_rows_dev, plan, part, xb, shape, batch, scale ); break;
-    default: launch_balanced<16>( y, st, q, layer_rows_dev, plan, part, xb, shape, batch, scale ); break;
+    case 1: launch_balanced<1, false>( y, st, q, layer_rows_dev, plan, part, xb, shape, batch, scale ); break; // one query head per kv head: dot products
+    case 2: launch_balanced<2, true>( y, st, q, layer_rows_dev, plan, part, xb, shape, batch, scale ); break;
+    case 4: launch_balanced<4, true>( y, st, q, layer_rows_dev, plan, part, xb, shape, batch, scale ); break;
+    case 8: launch_balanced<8, true>( y, st, q, layer_rows_dev, plan, part, xb, shape, batch, scale ); break;
+    default: launch_balanced<16, true>( y, st, q, layer_rows_dev, plan, part, xb, shape, batch, scale ); break;
   }
   GH_LAUNCH_CHECK();
   return GH_OK;

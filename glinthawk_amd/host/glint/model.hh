@@ -912,7 +912,7 @@ private:
       attn_ws_bytes_ = gh_attn_decode_workspace( cap, Config::seq_len - 1, &s );
       attn_ws_ = ops_.device_allocate( std::max<uint64_t>( attn_ws_bytes_, 16 ) );
       if ( std::is_same_v<DType, glint::float16_t> && Config::head_size == 128
-           && ( Config::gqa_size == 2 || Config::gqa_size == 4 || Config::gqa_size == 8 || Config::gqa_size == 16 ) ) {
+           && ( Config::gqa_size == 1 || Config::gqa_size == 2 || Config::gqa_size == 4 || Config::gqa_size == 8 || Config::gqa_size == 16 ) ) {
         attn_bal_ws_bytes_ = gh_attn_balanced_workspace( cap, &s ); // the shapes gh_attn_decode_balanced takes
         attn_bal_ws_ = ops_.device_allocate( std::max<uint64_t>( attn_bal_ws_bytes_, 16 ) );
       }

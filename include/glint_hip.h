@@ -264,7 +264,7 @@ int gh_attn_decode_static( const void* q, const void* const* layer_rows_dev, con
 /* Decode attention for batches whose contexts differ in length (the same result as gh_attn_decode: attention_0_gemm, attention_softmax
  * and attention_2_gemm of arch/amd64/llama2/ops.hh:170-298 in one pass; the reference runs one task per (context, kv head),
  * ops.hh:192-193, whatever their lengths).  The keys of all contexts are cut into equal runs, one per resident work-group, so that
- * no CU is left with the longest contexts while others idle.  f16, head size 128, gqa in {2, 4, 8, 16}.
+ * no CU is left with the longest contexts while others idle.  f16, head size 128, gqa in {1, 2, 4, 8, 16}.
  *   gh_attn_balanced_workspace  bytes for the cuts and the partial results of `batch` contexts (needs the device: 0 on failure)
  *   gh_attn_balance             makes the cuts from the positions (pos_dev[i] = position of the current token, keys [0, pos_i];
  *                               contexts with a NULL row in layer_rows_dev have none); once per step: the cuts do not depend on the layer

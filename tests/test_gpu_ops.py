@@ -641,7 +641,7 @@ def test_fused_auto_and_host_tables(shape):
     run_fused_case(shape, "f16", GH_ATTN_AUTO, pos, [True, False, True, True], 32, host_tables=True)
 
 
-@pytest.mark.parametrize("shape", [GQA2, GQA4, GQA8, GQA16], ids=["gqa2", "gqa4", "gqa8", "gqa16"])
+@pytest.mark.parametrize("shape", [MHA128, MHA128_ODD, GQA2, GQA4, GQA8, GQA16], ids=["mha", "mha6", "gqa2", "gqa4", "gqa8", "gqa16"])
 def test_fused_balanced_ragged(shape):
     # keys cut into equal runs over the work-groups: contexts shorter than a run share one, longer ones are divided
     # (a run is at least 256 keys), an empty context in the middle and at the end
@@ -719,8 +719,8 @@ def test_fused_balanced_bound_below_the_true_maximum_truncates_and_bad_arguments
     assert L.gh_attn_balance(table.data_ptr(), true_pos.data_ptr(), batch, 299, C.byref(s), small.data_ptr(), 1024, None) == GH_ERR_WORKSPACE
     assert L.gh_attn_decode_balanced(q.data_ptr(), table.data_ptr(), a.data_ptr(), batch, 299, C.byref(s), GH_F16, small.data_ptr(), 1024, None) == GH_ERR_WORKSPACE
     assert L.gh_attn_balance(table.data_ptr(), true_pos.data_ptr(), batch, shape.seq_len, C.byref(s), ws.data_ptr(), ws.numel(), None) == GH_ERR_INVALID
-    mha = MHA128.c()
-    assert L.gh_attn_balance(table.data_ptr(), true_pos.data_ptr(), batch, 10, C.byref(mha), ws.data_ptr(), ws.numel(), None) == GH_ERR_INVALID
+    odd = Shape(dim=768, n_layers=1, n_heads=6, n_kv_heads=2, hidden_dim=64, seq_len=300).c()      # gqa 3
+    assert L.gh_attn_balance(table.data_ptr(), true_pos.data_ptr(), batch, 10, C.byref(odd), ws.data_ptr(), ws.numel(), None) == GH_ERR_INVALID
     assert L.gh_attn_decode_balanced(q.data_ptr(), table.data_ptr(), a.data_ptr(), batch, 299, C.byref(s), GH_F32, ws.data_ptr(), ws.numel(), None) == GH_ERR_INVALID
     assert L.gh_attn_decode_balanced(None, table.data_ptr(), a.data_ptr(), batch, 299, C.byref(s), GH_F16, ws.data_ptr(), ws.numel(), None) == GH_ERR_INVALID
 
