@@ -241,6 +241,76 @@ __global__ __launch_bounds__( EPI_THREADS ) void epi_accum_norm_row8k_kernel( __
   }
 }
 
+// residual(b, r) += product(b, r), both f16 (the product already rounded, as a library GEMM leaves it), and the norm of the new
+// residual in the same pass: accum and rmsnorm of the reference in one kernel, one read of each operand.  Rows of at most 8192
+// elements, r % 4 == 0, 8-byte aligned rows.
+__global__ __launch_bounds__( EPI_THREADS ) void accum_norm_row8k_kernel( __half* __restrict__ residual,
+                                                                         const __half* __restrict__ product,
+                                                                         uint32_t r,
+                                                                         __half* __restrict__ norm_out,
+                                                                         const __half* __restrict__ norm_weight )
+{
+  __shared__ float smem[EPI_THREADS / WAVE];
+  const uint32_t row = blockIdx.x;
+  __half* res = residual + (uint64_t)row * r;
+  const __half* prod = product + (uint64_t)row * r;
+  union H4
+  {
+    uint2 raw;
+    __half h[4];
+  };
+  H4 old[2], add[2], nw[2];
+  bool live[2];
+  uint32_t col[2];
+#pragma unroll
+  for ( int it = 0; it < 2; it++ ) { // a column group past the row's end reads group 0 and stores nothing: no load under a branch
+    const uint32_t j = ( it * EPI_THREADS + threadIdx.x ) * 4;
+    live[it] = j < r;
+    col[it] = live[it] ? j : 0;
+    old[it].raw = *reinterpret_cast<const uint2*>( res + col[it] );
+    add[it].raw = *reinterpret_cast<const uint2*>( prod + col[it] );
+    nw[it].raw = *reinterpret_cast<const uint2*>( norm_weight + col[it] );
+  }
+  float ss = 0.0f;
+  float v[2][4];
+#pragma unroll
+  for ( int it = 0; it < 2; it++ ) {
+    H4 o;
+#pragma unroll
+    for ( int e = 0; e < 4; e++ ) {
+      o.h[e] = __float2half_rn( __half2float( old[it].h[e] ) + __half2float( add[it].h[e] ) );
+      v[it][e] = live[it] ? __half2float( o.h[e] ) : 0.0f;
+      ss += v[it][e] * v[it][e];
+    }
+    if ( live[it] ) {
+      *reinterpret_cast<uint2*>( res + col[it] ) = o.raw;
+    }
+  }
+  ss = wave_sum( ss );
+  if ( threadIdx.x % WAVE == 0 ) {
+    smem[threadIdx.x / WAVE] = ss;
+  }
+  __syncthreads();
+  ss = 0.0f;
+  for ( int w = 0; w < EPI_THREADS / WAVE; w++ ) {
+    ss += smem[w];
+  }
+  ss = ss / (float)r + 1e-5f;
+  const float inv = 1.0f / sqrtf( ss );
+  __half* o = norm_out + (uint64_t)row * r;
+#pragma unroll
+  for ( int it = 0; it < 2; it++ ) {
+    if ( live[it] ) {
+      H4 out;
+#pragma unroll
+      for ( int e = 0; e < 4; e++ ) {
+        out.h[e] = __float2half_rn( __half2float( nw[it].h[e] ) * ( inv * v[it][e] ) );
+      }
+      *reinterpret_cast<uint2*>( o + col[it] ) = out.raw;
+    }
+  }
+}
+
 // hb(b, hidden) = DType( silu(DType(y1)) * DType(y3) ), partial rows [0, hidden) = w1, [hidden, 2 hidden) = w3
 template<typename T>
 __global__ __launch_bounds__( 256 ) void epi_silu_gate_kernel( T* __restrict__ hb, const float* __restrict__ partial, uint32_t hidden, uint32_t b, uint32_t splits )
@@ -359,6 +429,14 @@ int gh_matmul_accum( void* residual, const void* x, const void* w, uint64_t s, u
       return rc;
     }
     if ( done ) {
+      const bool rows_8byte
+        = ( ( reinterpret_cast<uintptr_t>( residual ) | reinterpret_cast<uintptr_t>( norm_out ) | reinterpret_cast<uintptr_t>( norm_weight ) ) & 7u ) == 0;
+      if ( norm_out != nullptr && r % 4 == 0 && r <= 2 * 4 * EPI_THREADS && rows_8byte && b <= 0x7fffffffull ) {
+        accum_norm_row8k_kernel<<<(unsigned)b, EPI_THREADS, 0, st>>>( static_cast<__half*>( residual ), static_cast<const __half*>( product ), (uint32_t)r,
+                                                                     static_cast<__half*>( norm_out ), static_cast<const __half*>( norm_weight ) );
+        GH_LAUNCH_CHECK();
+        return GH_OK;
+      }
       if ( int rc = gh_accum( residual, product, r, b, dt, stream ) ) {
         return rc;
       }
