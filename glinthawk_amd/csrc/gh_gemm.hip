@@ -409,6 +409,13 @@ bool gemm_library_wanted( uint64_t s, uint64_t r, uint64_t b, gh_dtype dt, const
   // of 256 slots 10.07 ms against 9.84)
   return dt == GH_F16 && g_force_kernel == 0 && g_library_rows > 0 && b >= g_library_rows && s % 8 == 0 && r % 8 == 0 && aligned;
 }
+// a product with many weight rows (w1 and w3 together) of some hundred activation rows, below gemm_library_wanted()'s row count:
+// measured on the 13B and 70B shapes, the library wins there from 128 rows on (1.1-1.6 x), which it does not for narrower products
+bool gemm_library_wanted_wide( uint64_t s, uint64_t r, uint64_t b, gh_dtype dt, const void* x, const void* w, const void* xout )
+{
+  const bool aligned = ( ( reinterpret_cast<uintptr_t>( x ) | reinterpret_cast<uintptr_t>( w ) | reinterpret_cast<uintptr_t>( xout ) ) & 15u ) == 0;
+  return dt == GH_F16 && g_force_kernel == 0 && g_library_rows > 0 && b >= 128 && b < g_library_rows && r >= 16384 && s % 8 == 0 && r % 8 == 0 && aligned;
+}
 } // namespace gh
 
 using namespace gh;
