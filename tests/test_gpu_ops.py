@@ -693,6 +693,53 @@ def test_fused_balanced_many_contexts_equal_plain_kernel():
     assert torch.all(bal[5] == 5.0) and torch.all(bal[46] == 5.0)
 
 
+def test_fused_balanced_random_batches_equal_plain_kernel():
+    # seeded sweep over shapes (gqa 8, 1, 4 with three kv heads, 16, 2 with five kv heads), batch sizes, length patterns (uniform
+    # random, all short, all full, one long among short ones, lengths at chunk boundaries) and empty contexts; the workspace holds
+    # stale bytes before every call
+    shapes = [GQA8, MHA128, GQA4, GQA16, Shape(dim=1280, n_layers=1, n_heads=10, n_kv_heads=5, hidden_dim=64, seq_len=1100)]
+    rng = np.random.default_rng(123)
+    for it in range(60):
+        shape = shapes[it % len(shapes)]
+        batch = int(rng.choice([1, 2, 3, 7, 16, 33, 64, 130]))
+        kind = it // len(shapes) % 5
+        if kind == 0:
+            p = rng.integers(0, shape.seq_len, batch)
+        elif kind == 1:
+            p = rng.integers(0, 64, batch)
+        elif kind == 2:
+            p = np.full(batch, shape.seq_len - 1)
+        elif kind == 3:
+            p = rng.integers(0, 30, batch)
+            p[rng.integers(0, batch)] = shape.seq_len - 1
+        else:
+            p = (rng.integers(0, shape.seq_len // 64, batch) * 64 + rng.choice([-1, 0, 1, 63], batch)).clip(0, shape.seq_len - 1)
+        row_bytes = 2 * shape.kv_dim * 2
+        cache = torch.randn((batch, shape.seq_len, 2 * shape.kv_dim), dtype=torch.float16, device="cuda")
+        ptrs = [cache.data_ptr() + i * shape.seq_len * row_bytes for i in range(batch)]
+        holes = rng.random(batch) < (0.2 if it % 3 == 0 else 0.0)
+        if holes.all():
+            holes[0] = False
+        for i in np.nonzero(holes)[0]:
+            ptrs[i] = 0
+        table = ops.row_table(ptrs)
+        pos = torch.tensor(p, dtype=torch.int32, device="cuda")
+        max_pos = int(p.max())
+        q = torch.randn((batch, shape.dim), dtype=torch.float16, device="cuda")
+        plain = torch.full((batch, shape.dim), 7.0, dtype=torch.float16, device="cuda")
+        bal = torch.full((batch, shape.dim), 7.0, dtype=torch.float16, device="cuda")
+        ops.attn_decode(q, table, pos, plain, max_pos, shape)
+        ws = torch.empty(ops.attn_balanced_workspace(batch, shape), dtype=torch.uint8, device="cuda")
+        ws.fill_(0xFF)
+        ops.attn_balance(table, pos, max_pos, shape, ws)
+        ops.attn_decode_balanced(q, table, bal, max_pos, shape, ws)
+        what = f"case {it}: kv heads {shape.n_kv_heads}, gqa {shape.gqa_size}, batch {batch}, pattern {kind}, {int(holes.sum())} empty"
+        assert bool(torch.isfinite(bal).all()), what
+        assert (plain.float() - bal.float()).abs().max().item() < 6e-3, what
+        for i in np.nonzero(holes)[0]:
+            assert torch.all(bal[i] == 7.0), what
+
+
 def test_fused_balanced_bound_below_the_true_maximum_truncates_and_bad_arguments():
     shape = GQA8
     batch = 3
