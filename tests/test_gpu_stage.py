@@ -363,20 +363,23 @@ def test_device_span_timing_counts_steps_and_leaves_results_alone():
 
 
 @pytest.mark.parametrize("balanced", [True, False], ids=["equal-runs", "per-context"])
-def test_decode_attention_over_equal_runs_of_keys_in_a_stage(balanced):
+@pytest.mark.parametrize("name,first,n_hosted", [("test-gqa4", 1, 2), ("test-mha", 1, 1)])
+def test_decode_attention_over_equal_runs_of_keys_in_a_stage(name, first, n_hosted, balanced):
     # contexts of very different lengths and an inactive row; cache rows written straight into the slots.  Both attention
-    # routes of the fused path against the oracle on the same rows.
-    name, dtype = "test-gqa4", "f16"
+    # routes of the fused path against the oracle on the same rows, for grouped and for one-to-one query heads.
+    dtype = "f16"
     cfg = SHAPES[name]
-    layers, base = make_weights(cfg, np.float16, seed=12, wcls=True)
-    pos = [0, 5, 319, 64, 100, 255, 256, 300, 17]
+    layers, base = make_weights(cfg, np.float16, seed=12, wcls=WCLS[name])
+    top = cfg.seq_len - 1
+    pos = [0, 5, top, 64, 100, top - 64, top - 63, top - 19, 17]
     batch = len(pos)
     cids = [40 + i for i in range(batch)]
-    st = S.Stage(name, dtype, 1, 2, batch, batch, with_cls=False, balanced=balanced)
-    load_weights(st, cfg, layers, base, True, layer_range=[1, 2], with_embedding=False, with_cls=False)
+    hosted = list(range(first, first + n_hosted))
+    st = S.Stage(name, dtype, first, n_hosted, batch, batch, with_cls=False, balanced=balanced)
+    load_weights(st, cfg, layers, base, WCLS[name], layer_range=hosted, with_embedding=False, with_cls=False)
     ref = OracleModel(cfg, layers, base)
     rng = np.random.default_rng(13)
-    st.new_state(batch, next_layer=1)
+    st.new_state(batch, next_layer=first)
     for i in range(batch):
         st.set_prompt(i, cids[i], 1, pos[i])
     st.discard(4)
@@ -384,7 +387,7 @@ def test_decode_attention_over_equal_runs_of_keys_in_a_stage(balanced):
     for i in range(batch):
         if i == 4:
             continue
-        for l in (1, 2):
+        for l in hosted:
             rows = rng.standard_normal((cfg.seq_len, 2 * cfg.kv_dim)).astype(np.float16)
             _lib.check(_lib.lib().gh_memcpy(st.context_layer_ptr(i, l), rows.ctypes.data, rows.nbytes, _lib.GH_H2D, 0, None), "gh_memcpy")
             ref.ctx(cids[i])[l][:] = rows.astype(np.float32)
@@ -392,11 +395,11 @@ def test_decode_attention_over_equal_runs_of_keys_in_a_stage(balanced):
     st.activations(allocate=True)[:] = x.reshape(-1)
     assert st.forward()
     got = st.activations().reshape(batch, cfg.dim).astype(np.float32)
-    want = ref.run_layers(x.astype(np.float32), [None if i == 4 else c for i, c in enumerate(cids)], pos, [1, 2])
+    want = ref.run_layers(x.astype(np.float32), [None if i == 4 else c for i, c in enumerate(cids)], pos, hosted)
     live = [i for i in range(batch) if i != 4]
     assert_close(got[live], want[live], what="stage step over ragged contexts")
     # the appended rows are where the oracle put them
     for i in (2, 7):
-        row = d2h(st.context_layer_ptr(i, 2) + pos[i] * 2 * cfg.kv_dim * 2, (2 * cfg.kv_dim,), np.float16).astype(np.float32)
-        assert_close(row[None], ref.ctx(cids[i])[2][pos[i]][None], what="appended row")
+        row = d2h(st.context_layer_ptr(i, hosted[-1]) + pos[i] * 2 * cfg.kv_dim * 2, (2 * cfg.kv_dim,), np.float16).astype(np.float32)
+        assert_close(row[None], ref.ctx(cids[i])[hosted[-1]][pos[i]][None], what="appended row")
     st.close()
