@@ -11,6 +11,7 @@
 // f32: plain wave-per-row kernel (only the tiny fp32 configuration uses it).
 #include "gh_common.h"
 
+#include <cstdlib>
 #include <mutex>
 
 namespace gh {
@@ -39,7 +40,13 @@ int gemm_tile_launch( __half* xout, float* partial, const __half* x, const __hal
 namespace {
 
 int g_force_kernel = 0; // 0 auto, 1 small tiled kernel of this file, 2 streaming kernel, 3 large tile kernel
-uint64_t g_library_rows = 768; // plain products of this many rows and more go to the vendor's GEMM library (measurement hook: gh_gemm_set_library_rows)
+// GLINT_LIBRARY_ROWS in the environment overrides the default (for the command-line profilers, which have no other way in)
+uint64_t library_rows_default()
+{
+  const char* env = getenv( "GLINT_LIBRARY_ROWS" );
+  return env != nullptr && *env != '\0' ? strtoull( env, nullptr, 10 ) : 768;
+}
+uint64_t g_library_rows = library_rows_default(); // plain products of this many rows and more go to the vendor's GEMM library (measurement hook: gh_gemm_set_library_rows)
 
 typedef _Float16 f16x8 __attribute__( ( ext_vector_type( 8 ) ) );
 typedef float f32x4 __attribute__( ( ext_vector_type( 4 ) ) );

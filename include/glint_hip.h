@@ -155,7 +155,7 @@ int gh_gemm_set_tuning( int kernel, int target_workgroups, int tile_rows );
  * kernel of this library fuses it) of `rows` activation rows and more go to the vendor's GEMM library, as every product of the
  * reference's GPU target does (cublasGemmEx, arch/cuda/common/ops.cuh:666-700); 0: never.  Default 768 (measured: from there on the library's kernels are the faster ones for nearly every shape of the 13B and
  * 70B models; below, the split-K tile kernel and the fused epilogues of this library are).  A forced kernel
- * (gh_gemm_set_tuning) also keeps the library out. */
+ * (gh_gemm_set_tuning) also keeps the library out.  GLINT_LIBRARY_ROWS in the environment replaces the default. */
 int gh_gemm_set_library_rows( uint64_t rows );
 /* host-only query: 1 when gh_matmul_accum runs a product of this shape (16-byte aligned operands) in the large tile kernel with the residual added
  * in its epilogue, i.e. without fp32 partial sums of (b, r): the caller's test for taking the fused call on many rows */
