@@ -45,6 +45,7 @@ struct Product
 };
 
 constexpr uint64_t LIB_WORKSPACE = 64ull << 20;
+constexpr size_t MAX_PRODUCTS = 4096; // shapes whose descriptors and algorithm are kept
 
 std::mutex g_lib_mutex;
 Api g_api;
@@ -87,6 +88,10 @@ bool open_library()
 
 const Product& product_for( uint64_t s, uint64_t r, uint64_t b )
 {
+  static const Product declined {};
+  if ( g_products.size() >= MAX_PRODUCTS && g_products.find( { s, r, b } ) == g_products.end() ) {
+    return declined; // a caller with ever new shapes: the descriptors kept so far stay, further shapes run on the tile kernels
+  }
   Product& p = g_products[{ s, r, b }];
   if ( p.desc != nullptr || !g_api.ok ) {
     return p; // made before (p.ok says how that went)
