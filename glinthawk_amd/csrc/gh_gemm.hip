@@ -414,7 +414,11 @@ bool gemm_library_wanted( uint64_t s, uint64_t r, uint64_t b, gh_dtype dt, const
   // measured (13B and 70B shapes): from g_library_rows rows on the library's kernels win nearly everywhere; below, the split-K
   // tile kernel and the two-output launch do (w1 and w3 of the 70B shape at 256 rows as two library products: the decode step
   // of 256 slots 10.07 ms against 9.84)
-  return dt == GH_F16 && g_force_kernel == 0 && g_library_rows > 0 && b >= g_library_rows && s % 8 == 0 && r % 8 == 0 && aligned;
+  // from half that row count on as well unless the weight matrix is much wider than tall (w2): measured with the residual add and
+  // the norm behind the product, 384-704 rows, 4-50 % faster for every such product of the 7B, 13B and 70B shapes; for w2 the
+  // split-K tile kernel keeps up
+  const bool rows_enough = b >= g_library_rows || ( 2 * b >= g_library_rows && 2 * r >= s );
+  return dt == GH_F16 && g_force_kernel == 0 && g_library_rows > 0 && rows_enough && s % 8 == 0 && r % 8 == 0 && aligned;
 }
 // a product with many weight rows (w1 and w3 together) of some hundred activation rows, below gemm_library_wanted()'s row count:
 // measured on the 13B and 70B shapes, the library wins there from 128 rows on (1.1-1.6 x), which it does not for narrower products

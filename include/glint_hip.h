@@ -153,7 +153,7 @@ int gh_argmax( uint32_t* out_host, uint32_t* out_dev, const void* v, uint64_t n,
 int gh_gemm_set_tuning( int kernel, int target_workgroups, int tile_rows );
 /* Plain f16 products (gh_matmul, the two of gh_matmul_pair, the product inside gh_matmul_accum and gh_matmul_silu_gate where no
  * kernel of this library fuses it) of `rows` activation rows and more go to the vendor's GEMM library, as every product of the
- * reference's GPU target does (cublasGemmEx, arch/cuda/common/ops.cuh:666-700); 0: never.  Default 768 (measured: from there on the library's kernels are the faster ones for nearly every shape of the 13B and
+ * reference's GPU target does (cublasGemmEx, arch/cuda/common/ops.cuh:666-700); 0: never; from half as many rows on for weight matrices that are not much wider than tall.  Default 768 (measured: from there on the library's kernels are the faster ones for nearly every shape of the 13B and
  * 70B models; below, the split-K tile kernel and the fused epilogues of this library are).  A forced kernel
  * (gh_gemm_set_tuning) also keeps the library out.  GLINT_LIBRARY_ROWS in the environment replaces the default. */
 int gh_gemm_set_library_rows( uint64_t rows );
