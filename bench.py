@@ -52,6 +52,22 @@ TRAFFIC_PROFILE = {
 }
 
 
+def gemm_route(calls_before=0):
+    """Which kernels ran the products of many activation rows: the tile kernels of this library ("own", the default) or,
+    when a row threshold was set (--library-rows, GLINT_LIBRARY_ROWS), the vendor's GEMM library from that many rows on;
+    `vendor_products` counts the products the vendor library really ran since `calls_before` (it declines silently)."""
+    from glinthawk_amd import _lib
+    L = _lib.lib()
+    rows = int(L.gh_gemm_library_rows())
+    calls = int(L.gh_gemm_library_calls()) - calls_before
+    return {"route": "vendor" if rows > 0 and calls > 0 else "own", "vendor_library_from_rows": rows or None, "vendor_products": calls}
+
+
+def library_calls():
+    from glinthawk_amd import _lib
+    return int(_lib.lib().gh_gemm_library_calls())
+
+
 def kernel_source_digest(sources):
     """sha256 over the kernel's source files, in the order given."""
     h = hashlib.sha256()
@@ -196,7 +212,7 @@ def cpu_decode_layer(shape, w, re, im, layers, x, pos, reps=3):
     return float(np.median(layer_times)), float(np.median(att_times)), O.num_threads()
 
 
-def decode_bench(workload, steps, warmup, fused=True, cpu=True, events=True):
+def decode_bench(workload, steps, warmup, fused=True, cpu=True, events=True, advance=False):
     """A decode workload: K stage steps timed plain, K more with events around the attention launches, a plain
     copy as the practical bandwidth ceiling, and (cpu) the oracle on the first hosted layer's own inputs."""
     import numpy as np
@@ -209,6 +225,7 @@ def decode_bench(workload, steps, warmup, fused=True, cpu=True, events=True):
     pos = keys - 1
     ops.init(0)
     L = _lib.lib()
+    calls0 = library_calls()
 
     st = S.Stage(cfg_name, "f16", first, n_hosted, batch, batch, fused=fused, seed=4, weight_std=0.02)
     st.new_state(batch, next_layer=first)
@@ -226,8 +243,15 @@ def decode_bench(workload, steps, warmup, fused=True, cpu=True, events=True):
     rng = np.random.default_rng(0)
     acts = rng.standard_normal((batch, shape["dim"])).astype(np.float16)
 
-    def one_step():
-        st.set_next(first)
+    ids = [1000 + i for i in range(batch)]
+    ones = np.ones(batch, np.uint32)
+
+    def one_step(at=None):
+        if at is None:
+            st.set_next(first)
+        else:                                   # the next token of every context: a new state at the next position
+            st.new_state(batch, next_layer=first)
+            st.set_prompts(ids, ones, np.full(batch, at, np.uint32))
         st.activations(allocate=True)[:] = acts.reshape(-1)
         ok = st.forward()
         assert ok
@@ -238,14 +262,19 @@ def decode_bench(workload, steps, warmup, fused=True, cpu=True, events=True):
     torch.cuda.synchronize()
     # pass 1: the stage step as it runs in production, nothing recorded between its kernels
     t0 = time.perf_counter()
-    for _ in range(steps):
-        one_step()
+    for k in range(steps):
+        one_step(pos + k if advance else None)
     ops.sync()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     res = dict(ms_per_step=(t1 - t0) * 1e3 / steps, batch=batch, device=ops.device_name())
     a_bytes = attention_bytes(shape, batch, keys)
     res.update(attn_bytes=a_bytes, stage_bytes=n_hosted * (a_bytes + layer_weight_bytes(shape)))
+    if advance:                                 # keys grow by one per step: the bytes of the run are the sum over its steps
+        res["stage_bytes"] = sum(n_hosted * (attention_bytes(shape, batch, keys + k) + layer_weight_bytes(shape)) for k in range(steps)) // steps
+        res["gemm_route"] = gemm_route(calls0)
+        st.close()
+        return res
     if events and fused:
         # pass 2: the same steps with HIP events around every attention launch (an event record holds
         # the next kernel back by a few microseconds, so this pass is not the one the step is timed on)
@@ -299,6 +328,7 @@ def decode_bench(workload, steps, warmup, fused=True, cpu=True, events=True):
             "attn_ms_per_layer": att_s * 1e3, "layer_ms": layer_s * 1e3,
         }
         del w, layers
+    res["gemm_route"] = gemm_route(calls0)
     st.close()
     return res
 
@@ -365,6 +395,7 @@ def decode_line(workload, steps, warmup, attn_variant="auto", cpu=True):
                      "kernel": "attn_decode (split-K fused decode attention)", "launches_timed": g["attn_launches"],
                      "algorithmic_bytes_per_launch": g["attn_bytes"]},
         "cpu_baseline": g.get("cpu_baseline"),
+        "gemm_route": g["gemm_route"],
     }
 
 
@@ -376,6 +407,7 @@ def concept_path(workload, steps, warmup):
     g = decode_bench(workload, steps, warmup, fused=False, cpu=False, events=False)
     return {"ms_per_step": round(g["ms_per_step"], 4), "stage_tokens_per_s": round(g["batch"] / (g["ms_per_step"] * 1e-3), 1),
             "stage_roofline_frac": round(g["stage_bytes"] / (HBM_PEAK_GBPS * 1e9) * 1e3 / g["ms_per_step"], 4),
+            "gemm_route": g["gemm_route"],
             "note": "unfused attention ops + score buffer, separate projection / element-wise ops, per-op host tables"}
 
 
@@ -389,6 +421,7 @@ def prefill_bench(steps, warmup, cpu=True):
     name, first, n_hosted, batch, T = "llama2-13b-4k", 10, 10, 8, 2048
     shape = SHAPES[name]
     ops.init(0)
+    calls0 = library_calls()
     st = S.Stage(name, "f16", first, n_hosted, batch, batch, seed=3)
     rng = np.random.default_rng(3)
     # the boundary's host buffers, page-locked like the states' own buffers
@@ -460,6 +493,7 @@ def prefill_bench(steps, warmup, cpu=True):
                      "kernel": "whole prefill pass incl. host transfers (projection GEMMs + causal attention flops / step time)",
                      "algorithmic_flops_per_step": flops},
         "cpu_baseline": cpu_res,
+        "gemm_route": gemm_route(calls0),
     }
 
 
@@ -476,6 +510,7 @@ def churn_bench(steps, warmup, cpu=True):
     shape = SHAPES[name]
     ops.init(0)
     L = _lib.lib()
+    calls0 = library_calls()
     st = S.Stage(name, "f16", first, n_hosted, slots, slots, seed=5)
     rng = np.random.default_rng(5)
     start_pos = rng.integers(16, 4096, slots)
@@ -573,13 +608,46 @@ def churn_bench(steps, warmup, cpu=True):
                      "frac": round(decode_bytes / t_decode / 1e9 / HBM_PEAK_GBPS, 4),
                      "traffic": None, "kernel": "whole decode step (cached K/V read once + weights once) / decode time"},
         "cpu_baseline": cpu_res,
+        "gemm_route": gemm_route(calls0),
     }
+
+
+def with_own_kernels(others):
+    """When a run was asked to send products to the vendor's GEMM library, the same prefill and churn steps once more on
+    the kernels of this library, so that the line carries both (`ms_per_step_own_kernels`)."""
+    from glinthawk_amd import _lib
+    L = _lib.lib()
+    rows = int(L.gh_gemm_library_rows())
+    if rows == 0:
+        return
+    _lib.check(L.gh_gemm_set_library_rows(0))
+    try:
+        for key, again in (("cfg3", lambda: prefill_bench(3, 1, False)), ("cfg5", lambda: churn_bench(16, 3, False))):
+            if key in others and others[key]["gemm_route"]["route"] == "vendor":
+                others[key]["ms_per_step_own_kernels"] = again()["ms_per_step"]
+    finally:
+        _lib.check(L.gh_gemm_set_library_rows(rows))
+
+
+def full_configs(cpu):
+    """The configurations other than the headline at the run lengths they are stated with (the default run keeps them short)."""
+    g = decode_bench("llama2-7b-b32-ctx1024", 128, 3, cpu=False, events=False, advance=True)
+    cfg2 = {"workload": "llama2-7b-b32-ctx1024", "steps": 128, "keys_per_context": "1024..1151, one more per step",
+            "ms_per_step": round(g["ms_per_step"], 4), "stage_tokens_per_s": round(g["batch"] / (g["ms_per_step"] * 1e-3), 1),
+            "stage_roofline_frac": round(g["stage_bytes"] / (HBM_PEAK_GBPS * 1e9) * 1e3 / g["ms_per_step"], 4), "gemm_route": g["gemm_route"]}
+    cfg3 = brief(prefill_bench(3, 1, cpu))
+    cfg3["decode_steps"] = 64
+    cfg5 = brief(churn_bench(512, 3, cpu))
+    by_keys = cfg5.pop("decode_ms_by_mean_keys")
+    cfg5["decode_ms_by_mean_keys_every_32nd_step"] = by_keys[::32]
+    return {"full_configs": {"cfg2": cfg2, "cfg3": cfg3, "cfg5": cfg5}, "n_gpus": 1, "data": "synthetic", "dtype": "f16"}
 
 
 def brief(line):
     """What the headline line keeps of another configuration's line."""
     keep = ("value", "unit", "ms_per_step", "steps", "warmup", "stage_tokens_per_s", "stage_roofline_frac", "attn_kernel_ms", "decode_ms_per_step",
-            "decode_tokens_per_s", "prefill_ms_per_step", "prefill_tokens_per_s", "mean_keys_per_slot", "decode_ms_by_mean_keys")
+            "decode_tokens_per_s", "prefill_ms_per_step", "prefill_tokens_per_s", "mean_keys_per_slot", "decode_ms_by_mean_keys", "gemm_route",
+            "ms_per_step_own_kernels")
     out = {"workload": line["config"]["workload"], "metric": line["metric"]}
     out.update({k: line[k] for k in keep if k in line})
     r = line["roofline"]
@@ -604,7 +672,11 @@ def main():
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="also run a plain D2D copy of this many MiB (reference point for profiler byte counters)")
     ap.add_argument("--library-rows", type=int, default=-1,
-                    help="measurement hook: rows from which plain products go to the vendor's GEMM library (0: never; default: the library's own setting)")
+                    help="measurement hook: rows from which plain products go to the vendor's GEMM library (0: never; default: the library's own setting, "
+                         "which is never unless GLINT_LIBRARY_ROWS says otherwise)")
+    ap.add_argument("--full-configs", action="store_true",
+                    help="the other configurations at their stated run lengths instead of the headline line: 128 decode steps at 1024..1151 keys "
+                         "(7B shape), the 8 x 2048 prefill with its 64 decode steps (13B shape), 512 churn steps (70B shape); takes some minutes")
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -625,6 +697,9 @@ def main():
         from glinthawk_amd import _lib, ops
         ops.init(0)
         _lib.check(_lib.lib().gh_attn_set_auto_variant({"generic": 1, "valu": 2, "mfma": 3}[args.attn_variant]))
+    if args.full_configs:
+        print(json.dumps(full_configs(cpu)))
+        return
     if args.workload == "llama2-13b-prefill-8x2048":
         print(json.dumps(prefill_bench(args.steps, args.warmup, cpu)))
         return
@@ -642,11 +717,13 @@ def main():
         cp = concept_path(args.workload, min(args.steps, 10), 2)
         line["concept_path_ms_per_step"] = cp["ms_per_step"]
         line["concept_path"] = cp
-        line["other"] = {
-            "cfg2": brief(decode_line("llama2-7b-b32-ctx1024", min(args.steps, 20), 3, "auto", cpu)),
-            "cfg3": brief(prefill_bench(3, 1, cpu)),
-            "cfg5": brief(churn_bench(16, 3, cpu)),
+        others = {
+            "cfg2": decode_line("llama2-7b-b32-ctx1024", min(args.steps, 20), 3, "auto", cpu),
+            "cfg3": prefill_bench(3, 1, cpu),
+            "cfg5": churn_bench(16, 3, cpu),
         }
+        with_own_kernels(others)
+        line["other"] = {k: brief(v) for k, v in others.items()}
     print(json.dumps(line))
 
 

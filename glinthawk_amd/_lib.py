@@ -73,6 +73,7 @@ SIGNATURES = {
     "gh_stream_wait_event": (_i, [_vp, _vp]),
     "gh_malloc": (_i, [C.POINTER(_vp), _u64]),
     "gh_free": (_i, [_vp]),
+    "gh_allocation_count": (_u64, []),
     "gh_host_malloc": (_i, [C.POINTER(_vp), _u64]),
     "gh_host_free": (_i, [_vp]),
     "gh_memcpy": (_i, [_vp, _vp, _u64, _i, _i, _vp]),
@@ -95,6 +96,8 @@ SIGNATURES = {
     "gh_argmax": (_i, [_vp, _vp, _vp, _u64, _u64, _i, _vp]),
     "gh_gemm_set_tuning": (_i, [_i, _i, _i]),
     "gh_gemm_set_library_rows": (_i, [_u64]),
+    "gh_gemm_library_rows": (_u64, []),
+    "gh_gemm_library_calls": (_u64, []),
     "gh_matmul_fuses_many_rows": (_i, [_u64, _u64, _u64, _i]),
     "gh_gemm_stream_plan": (_i, [_u64, _u64, _u64, _vp, _vp, _vp]),
     "gh_matmul": (_i, [_vp, _vp, _vp, _u64, _u64, _u64, _i, _vp]),

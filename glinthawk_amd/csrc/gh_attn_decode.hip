@@ -367,9 +367,10 @@ __global__ __launch_bounds__( 256 ) void attn_decode_valu_kernel( const __half* 
                                                                   uint32_t n_kv_heads,
                                                                   uint32_t chunk,
                                                                   uint32_t max_splits,
+                                                                  uint32_t seq_len,
                                                                   float scale_log2e )
 {
-  const WaveJob job = wave_job( layer_rows, pos, n_kv_heads, chunk, max_splits );
+  const WaveJob job = wave_job( layer_rows, pos, n_kv_heads, chunk, max_splits, seq_len );
   if ( !job.valid ) {
     return; // wave-uniform; the kernel has no block-level barrier
   }
@@ -589,11 +590,12 @@ __global__ __launch_bounds__( 256 ) void attn_decode_mfma_kernel( const __half* 
                                                                   uint32_t n_kv_heads,
                                                                   uint32_t chunk,
                                                                   uint32_t max_splits,
+                                                                  uint32_t seq_len,
                                                                   float scale_log2e )
 {
   __shared__ uint4 s_k[4][16 * 16]; // per wave: 16 tokens x 16 chunks of 16 bytes
 
-  const WaveJob job = wave_job( layer_rows, pos, n_kv_heads, chunk, max_splits );
+  const WaveJob job = wave_job( layer_rows, pos, n_kv_heads, chunk, max_splits, seq_len );
   if ( !job.valid ) {
     return; // wave-uniform; only wave-private LDS is used, no block barrier
   }
@@ -982,7 +984,7 @@ void launch_valu( dim3 grid, hipStream_t st, const void* q, const void* const* r
                   const gh_shape* s, const Plan& p, float scale )
 {
   attn_decode_valu_kernel<G><<<grid, 256, 0, st>>>( static_cast<const __half*>( q ), reinterpret_cast<const __half* const*>( rows ), pos, part,
-                                                   static_cast<__half*>( xb ), s->n_kv_heads, p.chunk, p.max_splits, scale );
+                                                   static_cast<__half*>( xb ), s->n_kv_heads, p.chunk, p.max_splits, s->seq_len, scale );
 }
 
 template<int G>
@@ -990,7 +992,7 @@ void launch_mfma( dim3 grid, hipStream_t st, const void* q, const void* const* r
                   const gh_shape* s, const Plan& p, float scale )
 {
   attn_decode_mfma_kernel<G><<<grid, 256, 0, st>>>( static_cast<const __half*>( q ), reinterpret_cast<const __half* const*>( rows ), pos, part,
-                                                   static_cast<__half*>( xb ), s->n_kv_heads, p.chunk, p.max_splits, scale );
+                                                   static_cast<__half*>( xb ), s->n_kv_heads, p.chunk, p.max_splits, s->seq_len, scale );
 }
 
 // where the plan and the partials of the balanced variant lie in its workspace
@@ -1245,6 +1247,9 @@ int gh_attn_decode_static( const void* q, const void* const* layer_rows_dev, con
   const int device = initialised_device();
   GH_REQUIRE( device >= 0, "gh_attn_decode_static: the library is not initialised; call gh_init() first (this entry point allocates nothing)" );
   GH_REQUIRE( device < MAX_DEVICES && g_static_scratch[device] != nullptr, "gh_attn_decode_static: no scratch array on device %d", device );
+  int current = -1; // every GPU holds its own copy of the array at its own address: the kernels must run where that address is valid
+  GH_REQUIRE( hipGetDevice( &current ) == hipSuccess && current == device,
+              "gh_attn_decode_static: the calling thread's current device is %d, the library was initialised on device %d", current, device );
   if ( batch == 0 ) {
     return GH_OK;
   }

@@ -31,7 +31,8 @@ __device__ __forceinline__ WaveJob wave_job( const __half* const* layer_rows,
                                              const uint32_t* pos,
                                              uint32_t n_kv_heads,
                                              uint32_t chunk,
-                                             uint32_t max_splits )
+                                             uint32_t max_splits,
+                                             uint32_t seq_len )
 {
   WaveJob j;
   const uint32_t wave = threadIdx.x >> 6;
@@ -43,7 +44,9 @@ __device__ __forceinline__ WaveJob wave_job( const __half* const* layer_rows,
   j.ctx = bid / max_splits;
   j.h = hg * 4 + wave;
   j.base = layer_rows[j.ctx];
-  const uint32_t n_tok = min( pos[j.ctx] + 1, max_splits * chunk ); // never beyond what the host sized the grid and the partials for
+  // never beyond what the host sized the grid and the partials for, nor beyond the rows a context has (chunks are rounded up, so
+  // max_splits * chunk may exceed seq_len; the positions come from device memory and are not checked by the host)
+  const uint32_t n_tok = min( min( pos[j.ctx] + 1, max_splits * chunk ), seq_len );
   j.t_begin = j.split * chunk;
   j.t_end = min( n_tok, j.t_begin + chunk );
   j.valid = j.h < n_kv_heads && j.base != nullptr && j.t_begin < n_tok;

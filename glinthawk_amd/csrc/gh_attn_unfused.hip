@@ -77,7 +77,7 @@ __global__ __launch_bounds__( 256 ) void attn_scores_mfma_kernel( const __half* 
 {
   __shared__ uint4 s_k[4][2][16 * 16]; // per wave: two tiles of 16 tokens x 16 chunks of 16 bytes
 
-  const WaveJob job = wave_job( layer_rows, pos, n_kv_heads, chunk, max_splits );
+  const WaveJob job = wave_job( layer_rows, pos, n_kv_heads, chunk, max_splits, seq_len );
   if ( !job.valid ) {
     return; // wave-uniform; only wave-private LDS is used, no block barrier
   }
@@ -162,7 +162,7 @@ __global__ __launch_bounds__( 256 ) void attn_scores_valu_kernel( const __half* 
                                                                   uint32_t max_splits,
                                                                   float scale )
 {
-  const WaveJob job = wave_job( layer_rows, pos, n_kv_heads, chunk, max_splits );
+  const WaveJob job = wave_job( layer_rows, pos, n_kv_heads, chunk, max_splits, seq_len );
   if ( !job.valid ) {
     return;
   }
@@ -311,7 +311,7 @@ __global__ __launch_bounds__( 256 ) void attn_pv_mfma_kernel( const __half* __re
                                                               uint32_t chunk,
                                                               uint32_t max_splits )
 {
-  const WaveJob job = wave_job( layer_rows, pos, n_kv_heads, chunk, max_splits );
+  const WaveJob job = wave_job( layer_rows, pos, n_kv_heads, chunk, max_splits, seq_len );
   if ( !job.valid ) {
     return;
   }
@@ -424,7 +424,7 @@ __global__ __launch_bounds__( 256 ) void attn_pv_valu_kernel( const __half* __re
                                                               uint32_t chunk,
                                                               uint32_t max_splits )
 {
-  const WaveJob job = wave_job( layer_rows, pos, n_kv_heads, chunk, max_splits );
+  const WaveJob job = wave_job( layer_rows, pos, n_kv_heads, chunk, max_splits, seq_len );
   if ( !job.valid ) {
     return;
   }

@@ -92,6 +92,7 @@ enum { SCRATCH_GEMM_PARTIALS = 0, SCRATCH_CONVERT = 1, SCRATCH_ATTN_PV = 2, SCRA
 int stream_scratch( hipStream_t stream, int which, uint64_t bytes, uint64_t min_bytes, void** out );
 // gh_gemm_lib.hip: a plain f16 product through the vendor's GEMM library; *done = false: declined, nothing queued
 int gemm_library( void* xout, const void* x, const void* w, uint64_t s, uint64_t r, uint64_t b, hipStream_t st, bool* done );
+bool gemm_library_available( uint64_t s, uint64_t r, uint64_t b );
 bool gemm_library_wanted( uint64_t s, uint64_t r, uint64_t b, gh_dtype dt, const void* x, const void* w, const void* xout );
 bool gemm_library_wanted_wide( uint64_t s, uint64_t r, uint64_t b, gh_dtype dt, const void* x, const void* w, const void* xout );
 

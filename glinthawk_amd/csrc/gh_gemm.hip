@@ -44,9 +44,9 @@ int g_force_kernel = 0; // 0 auto, 1 small tiled kernel of this file, 2 streamin
 uint64_t library_rows_default()
 {
   const char* env = getenv( "GLINT_LIBRARY_ROWS" );
-  return env != nullptr && *env != '\0' ? strtoull( env, nullptr, 10 ) : 768;
+  return env != nullptr && *env != '\0' ? strtoull( env, nullptr, 10 ) : 0;
 }
-uint64_t g_library_rows = library_rows_default(); // plain products of this many rows and more go to the vendor's GEMM library (measurement hook: gh_gemm_set_library_rows)
+uint64_t g_library_rows = library_rows_default(); // 0: never; else plain products of this many rows and more go to the vendor's GEMM library (gh_gemm_set_library_rows)
 
 typedef _Float16 f16x8 __attribute__( ( ext_vector_type( 8 ) ) );
 typedef float f32x4 __attribute__( ( ext_vector_type( 4 ) ) );
@@ -446,6 +446,8 @@ int gh_gemm_set_library_rows( uint64_t rows )
   g_library_rows = rows;
   return GH_OK;
 }
+
+uint64_t gh_gemm_library_rows( void ) { return g_library_rows; }
 
 int gh_matmul_fuses_many_rows( uint64_t s, uint64_t r, uint64_t b, gh_dtype dt )
 {

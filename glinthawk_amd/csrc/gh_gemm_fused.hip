@@ -447,7 +447,7 @@ int gh_matmul_accum( void* residual, const void* x, const void* w, uint64_t s, u
   bool done = false;
   // many rows (prompt tokens), the product by the vendor's library where the dispatcher sends plain products there: the rounded
   // product, then the reference's own next ops on it (accum, rmsnorm) -- the same roundings as fused
-  if ( gemm_library_wanted( s, r, b, dt, x, w, residual ) ) {
+  if ( gemm_library_wanted( s, r, b, dt, x, w, residual ) && gemm_library_available( s, r, b ) ) { // the product's buffer only when it will be used
     void* product = nullptr;
     if ( int rc = stream_scratch( st, SCRATCH_PRODUCT, b * r * sizeof( __half ), 64ull << 20, &product ) ) {
       return rc;
@@ -530,7 +530,7 @@ int gh_matmul_silu_gate( void* hb, const void* x, const void* w13, uint64_t s, u
   // Some hundred rows, short of where every plain product goes to the vendor's library: [w1; w3] as one product of that library, whose
   // kernels cut a wide product finer than whole tiles (70B shape, 256 rows: 207 us against 262 for the route below), then the gate
   // over the two halves of each row.  The same roundings: each factor to DType, then the gate.
-  if ( gemm_library_wanted_wide( s, 2 * hidden_dim, b, dt, x, w13, hb ) && hidden_dim % 8 == 0 ) {
+  if ( gemm_library_wanted_wide( s, 2 * hidden_dim, b, dt, x, w13, hb ) && hidden_dim % 8 == 0 && gemm_library_available( s, 2 * hidden_dim, b ) ) {
     void* both = nullptr;
     if ( int rc = stream_scratch( st, SCRATCH_PRODUCT, b * 2 * hidden_dim * sizeof( __half ), 64ull << 20, &both ) ) {
       return rc;

@@ -12,6 +12,7 @@
 #include <dlfcn.h>
 #include <hipblaslt/hipblaslt.h>
 
+#include <atomic>
 #include <map>
 #include <mutex>
 #include <tuple>
@@ -45,9 +46,10 @@ struct Product
 };
 
 constexpr uint64_t LIB_WORKSPACE = 64ull << 20;
-constexpr size_t MAX_PRODUCTS = 4096; // shapes whose descriptors and algorithm are kept
+constexpr size_t MAX_PRODUCTS = 256; // shapes whose descriptors and algorithm are kept (a stage has a handful)
 
 std::mutex g_lib_mutex;
+std::atomic<uint64_t> g_library_calls { 0 }; // products the library has run
 Api g_api;
 std::map<std::tuple<uint64_t, uint64_t, uint64_t>, Product> g_products; // (s, r, b); kept until the process ends
 
@@ -130,16 +132,29 @@ const Product& product_for( uint64_t s, uint64_t r, uint64_t b )
 
 } // namespace
 
+// Whether gemm_library() would run this product: the library opens and has an algorithm for the shape.  Lets a caller that needs a
+// buffer for the product allocate it only then.
+bool gemm_library_available( uint64_t s, uint64_t r, uint64_t b )
+{
+  std::lock_guard<std::mutex> lock( g_lib_mutex );
+  return open_library() && product_for( s, r, b ).ok;
+}
+
 // xout(b, r) = x(b, s) . w(r, s)^T, f16 storage, fp32 sums rounded once.  *done = false: declined (no library, no algorithm):
 // nothing was queued.
 int gemm_library( void* xout, const void* x, const void* w, uint64_t s, uint64_t r, uint64_t b, hipStream_t st, bool* done )
 {
   *done = false;
-  std::lock_guard<std::mutex> lock( g_lib_mutex );
-  if ( !open_library() ) {
-    return GH_OK;
+  Product p;
+  {
+    // the lock covers the table of descriptors only: a product's descriptors are never changed or dropped once made, and the
+    // library's handle may be used from several threads at once, so stage threads do not queue behind each other's products
+    std::lock_guard<std::mutex> lock( g_lib_mutex );
+    if ( !open_library() ) {
+      return GH_OK;
+    }
+    p = product_for( s, r, b );
   }
-  const Product& p = product_for( s, r, b );
   if ( !p.ok ) {
     return GH_OK;
   }
@@ -155,8 +170,11 @@ int gemm_library( void* xout, const void* x, const void* w, uint64_t s, uint64_t
     return fail( GH_ERR_DEVICE, "gemm_library: hipblasLtMatmul failed with status %d for %llu x %llu x %llu", (int)status, (unsigned long long)b,
                  (unsigned long long)s, (unsigned long long)r );
   }
+  g_library_calls++;
   *done = true;
   return GH_OK;
 }
 
 } // namespace gh
+
+extern "C" uint64_t gh_gemm_library_calls( void ) { return gh::g_library_calls.load(); }

@@ -4,6 +4,7 @@
 #include "gh_common.h"
 
 #include <algorithm>
+#include <atomic>
 #include <cstdarg>
 #include <mutex>
 #include <vector>
@@ -46,6 +47,9 @@ struct ScratchBuffer
 };
 std::vector<ScratchBuffer> g_scratch;
 
+// every allocation this library makes (device, page-locked host, physical blocks of the paged arena), for gh_allocation_count()
+std::atomic<uint64_t> g_allocations { 0 };
+
 // ---- attention kernel timer ----------------------------------------------------------------
 constexpr int TIMER_SLOTS = 8192;
 int g_timing = 0; // 0 off; 1 events in front of, between and behind the two kernels; 2 only in front of and behind the pair
@@ -87,6 +91,7 @@ int check_buffer_bounds()
 {
   uint32_t* buf = nullptr;
   GH_HIP( hipMalloc( reinterpret_cast<void**>( &buf ), 4096 + 64 * 4 ) );
+  g_allocations++;
   uint32_t* out = buf + 1024;
   GH_HIP( hipMemset( buf, 0x5a, 4096 + 64 * 4 ) );
   buffer_bounds_probe_kernel<<<1, 64>>>( buf, out, 2048 ); // descriptor: 1024 bytes; the loads land at 2048.. of a 4096-byte block
@@ -129,6 +134,7 @@ static int init_locked( int device )
   for ( int i = 0; i < STAGE_SLOTS; i++ ) {
     GH_HIP( hipHostMalloc( reinterpret_cast<void**>( &g_slots[i].pinned ), STAGE_SLOT_BYTES, hipHostMallocDefault ) );
     GH_HIP( hipMalloc( reinterpret_cast<void**>( &g_slots[i].device ), STAGE_SLOT_BYTES ) );
+    g_allocations += 2;
     GH_HIP( hipEventCreateWithFlags( &g_slots[i].done, hipEventDisableTiming ) );
   }
   g_device = device;
@@ -236,6 +242,7 @@ int stream_scratch( hipStream_t stream, int which, uint64_t bytes, uint64_t min_
     }
     const uint64_t want = std::max( bytes, min_bytes );
     GH_HIP( hipMalloc( &buf->ptr, want ) );
+    g_allocations++;
     buf->bytes = want;
   }
   *out = buf->ptr;
@@ -317,8 +324,33 @@ int gh_stream_create( gh_stream* out )
 int gh_stream_destroy( gh_stream stream )
 {
   GH_REQUIRE( stream != nullptr, "gh_stream_destroy: the default stream is not the caller's" );
-  GH_HIP( hipStreamSynchronize( as_stream( stream ) ) );
-  GH_HIP( hipStreamDestroy( as_stream( stream ) ) );
+  hipStream_t st = as_stream( stream );
+  GH_HIP( hipStreamSynchronize( st ) );
+  {
+    // What the library keeps for this stream goes with it: the grow-only scratch buffers (nothing queued reads them after the
+    // synchronise above) and the staging slots' memory of having been filled on it -- a later stream may get the same handle
+    // value and must neither inherit the buffers' contents nor be handed a table that was copied on the old stream.
+    std::lock_guard<std::mutex> lock( g_mutex );
+    for ( size_t i = 0; i < g_scratch.size(); ) {
+      if ( g_scratch[i].stream == st ) {
+        if ( g_scratch[i].ptr != nullptr ) {
+          GH_HIP( hipFree( g_scratch[i].ptr ) );
+        }
+        g_scratch.erase( g_scratch.begin() + (long)i );
+      } else {
+        i++;
+      }
+    }
+    for ( StageSlot& slot : g_slots ) {
+      if ( slot.stream == st ) {
+        slot.stream = nullptr;
+        slot.bytes = 0;
+        slot.staged = false;
+        slot.in_flight = false; // its event, if recorded, lies behind the synchronise above
+      }
+    }
+  }
+  GH_HIP( hipStreamDestroy( st ) );
   return GH_OK;
 }
 
@@ -399,8 +431,11 @@ int gh_malloc( void** out, uint64_t bytes )
     return GH_OK;
   }
   GH_HIP( hipMalloc( out, bytes ) );
+  g_allocations++;
   return GH_OK;
 }
+
+uint64_t gh_allocation_count( void ) { return g_allocations.load(); }
 
 int gh_free( void* ptr )
 {
@@ -421,6 +456,7 @@ int gh_host_malloc( void** out, uint64_t bytes )
     return GH_OK;
   }
   GH_HIP( hipHostMalloc( out, bytes, hipHostMallocDefault ) );
+  g_allocations++;
   return GH_OK;
 }
 
@@ -536,6 +572,7 @@ int gh_vmm_commit( gh_vmm* r, uint64_t offset, uint64_t len )
   }
   hipMemGenericAllocationHandle_t handle;
   GH_HIP( hipMemCreate( &handle, len, &prop, 0 ) );
+  g_allocations++;
   void* at = static_cast<char*>( r->base ) + offset;
   hipError_t err = hipMemMap( at, len, 0, handle, 0 );
   if ( err != hipSuccess ) {

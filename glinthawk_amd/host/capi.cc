@@ -47,6 +47,7 @@ struct StageBase
   virtual int release_context( uint32_t id ) = 0;
   virtual void paging_info( size_t row, size_t layer, uint64_t out[3] ) = 0;
   virtual void sync() = 0;
+  virtual void copy_bytes( void* dst, const void* src, uint64_t bytes, int kind ) = 0;
   virtual void time_device_spans( bool on ) = 0;
   virtual void device_spans( double* ms, uint64_t* spans ) = 0;
   virtual int prefill( uint32_t batch, const uint32_t* context_ids, const uint32_t* start_pos, uint32_t n_tokens, uint32_t first_layer,
@@ -234,6 +235,11 @@ struct StageImpl : StageBase
     }
   }
   void sync() override { model.ops().synchronize(); }
+  // the instantiation the reference's concept names: convert_and_copy<void, void>, a copy of `bytes` bytes
+  void copy_bytes( void* dst, const void* src, uint64_t bytes, int kind ) override
+  {
+    model.ops().template convert_and_copy<void, void>( dst, src, bytes, static_cast<CopyType>( kind ) );
+  }
   void time_device_spans( bool on ) override { model.time_device_spans( on ); }
   void device_spans( double* ms, uint64_t* spans ) override
   {
@@ -561,6 +567,7 @@ int glint_stage_release_context( void* h, uint32_t id ) { return static_cast<Sta
 void glint_stage_paging_info( void* h, uint32_t row, uint32_t layer, uint64_t out[3] ) { static_cast<StageBase*>( h )->paging_info( row, layer, out ); }
 void* glint_stage_scratch( void* h, int which ) { return static_cast<StageBase*>( h )->scratch( which ); }
 void glint_stage_sync( void* h ) { static_cast<StageBase*>( h )->sync(); }
+void glint_stage_copy_bytes( void* h, void* dst, const void* src, uint64_t bytes, int kind ) { static_cast<StageBase*>( h )->copy_bytes( dst, src, bytes, kind ); }
 // device time of forward() without the copies over the host boundary: on / off, then total milliseconds and steps since the last read
 void glint_stage_time_device_spans( void* h, int on ) { static_cast<StageBase*>( h )->time_device_spans( on != 0 ); }
 void glint_stage_device_spans( void* h, double* ms, uint64_t* spans ) { static_cast<StageBase*>( h )->device_spans( ms, spans ); }

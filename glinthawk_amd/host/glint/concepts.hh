@@ -44,6 +44,7 @@ concept OperationsConcept = requires( const T t,
 
 template<typename T, typename DType, typename Settings>
 concept AdditionalLlamaOperationsConcept = requires( const T t,
+                                                     void* ptr_void,
                                                      DType* ptr,
                                                      const DType* cptr,
                                                      const uint64_t size,
@@ -58,7 +59,7 @@ concept AdditionalLlamaOperationsConcept = requires( const T t,
   { t.attention_softmax( ptr, int_arr, ptr, size ) } -> std::same_as<void>;
   { t.apply_rope( size, int_arr, cptr, cptr, ptr, tc ) } -> std::same_as<void>;
   { t.copy_kv_cache( tc, cptr, size ) } -> std::same_as<void>;
-  { t.template convert_and_copy<DType, DType>( ptr, cptr, size, cpt ) } -> std::same_as<void>;
+  { t.template convert_and_copy<void, void>( ptr_void, ptr_void, size, cpt ) } -> std::same_as<void>;
 };
 
 template<typename T, typename DType, typename Settings>

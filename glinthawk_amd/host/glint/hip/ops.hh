@@ -7,6 +7,7 @@
 
 #include <memory>
 #include <string>
+#include <type_traits>
 #include <vector>
 
 #include "glint/config.hh"
@@ -153,7 +154,7 @@ public:
   void copy( DType* dst, const DType* src, const uint64_t len_bytes, const CopyType type, const bool async = false ) const
   {
     GLINT_GH( gh_memcpy( dst, src, len_bytes, gh_kind( type ), async ? 1 : 0, stream_ ) );
-    if ( !async ) {
+    if ( !async && len_bytes > 0 ) { // a copy of nothing returns without waiting for the stream
       drains_++;
     }
   }
@@ -308,10 +309,18 @@ public:
     GLINT_GH( gh_kv_append_host( token_table( token_contexts, batch_size ), state_kv, batch_size, Config::kv_dim, gh_type<DType>(), this->stream_ ) );
   }
 
+  // <void, void> is the instantiation the reference's concept names (models/llama2/ops/concept.hh:36): the element is
+  // then a byte (sizeof( void ) is 1 in the reference's GNU dialect, arch/amd64/llama2/ops.hh:361-362), i.e. a plain
+  // synchronous copy of `size` bytes.
   template<typename DTypeDst, typename DTypeSrc>
   void convert_and_copy( DTypeDst* dst, const DTypeSrc* src, const uint64_t size, const CopyType type ) const
   {
-    GLINT_GH( gh_convert_and_copy( dst, gh_type<DTypeDst>(), src, gh_type<DTypeSrc>(), size, gh_kind( type ), this->stream_ ) );
+    if constexpr ( std::is_void_v<DTypeDst> && std::is_void_v<DTypeSrc> ) {
+      GLINT_GH( gh_memcpy( dst, src, size, gh_kind( type ), 0, this->stream_ ) );
+    } else {
+      static_assert( !std::is_void_v<DTypeDst> && !std::is_void_v<DTypeSrc>, "convert_and_copy: void on one side only" );
+      GLINT_GH( gh_convert_and_copy( dst, gh_type<DTypeDst>(), src, gh_type<DTypeSrc>(), size, gh_kind( type ), this->stream_ ) );
+    }
   }
 
   // Extension used by the stage driver: attention_0_gemm + attention_softmax + attention_2_gemm in

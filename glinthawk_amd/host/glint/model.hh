@@ -553,6 +553,8 @@ public:
         next_tokens[i] = argmax_pos_[i];
       }
     } else {
+      // Also the end of the uploads of a pipelined call: the stage's stream waited for every run's upload event before that run's
+      // first kernel, so once it is empty the caller's input buffer is free again, whether or not anything was downloaded.
       ops_.synchronize();
     }
   }

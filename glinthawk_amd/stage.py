@@ -61,6 +61,7 @@ def host_lib() -> C.CDLL:
             "glint_stage_paging_info": (None, [vp, u32, u32, C.POINTER(u64)]),
             "glint_stage_scratch": (vp, [vp, C.c_int]),
             "glint_stage_sync": (None, [vp]),
+            "glint_stage_copy_bytes": (None, [vp, vp, vp, u64, C.c_int]),
             "glint_stage_time_device_spans": (None, [vp, C.c_int]),
             "glint_stage_device_spans": (None, [vp, C.POINTER(C.c_double), C.POINTER(u64)]),
             "glint_stage_prefill": (C.c_int, [vp, u32, vp, vp, u32, u32, vp, vp, vp, vp]),
@@ -254,6 +255,11 @@ class Stage:
 
     def sync(self) -> None:
         host_lib().glint_stage_sync(self._h)
+
+    def copy_bytes(self, dst: int, src: int, n_bytes: int, kind: int) -> None:
+        """The ops class's convert_and_copy<void, void>: a synchronous copy of n_bytes bytes (kind: 0 host to device,
+        1 device to host, 2 device to device, 3 host to host)."""
+        host_lib().glint_stage_copy_bytes(self._h, dst, src, n_bytes, kind)
 
     def time_device_spans(self, on: bool) -> None:
         """Times forward() on the device, first kernel to last, without the copies of the state over the host boundary."""

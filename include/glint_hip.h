@@ -102,6 +102,10 @@ int gh_event_elapsed_ms( gh_event begin, gh_event end, float* ms );
 /* Operations::device_allocate / DeviceUniquePtr deleter (arch/cuda/common/ops.cuh:27-35,748-756) */
 int gh_malloc( void** out, uint64_t bytes );
 int gh_free( void* ptr );
+/* host-only: allocations (device memory, page-locked host memory, physical blocks of the paged arena) this library has made since the
+ * process started, its own scratch buffers included; no counterpart in the reference.  Lets a caller that must not allocate check
+ * that a call did not. */
+uint64_t gh_allocation_count( void );
 /* pinned host memory for the staging buffers of a caller (hipHostMalloc) */
 int gh_host_malloc( void** out, uint64_t bytes );
 int gh_host_free( void* ptr );
@@ -151,12 +155,16 @@ int gh_argmax( uint32_t* out_host, uint32_t* out_dev, const void* v, uint64_t n,
  * streaming kernel's K split is balanced for (<= 0 keeps the current value; the default is the device's own count); weight rows per work-group of the
  * 256-token tile kernel: 256, 384, or 0 for the library's choice */
 int gh_gemm_set_tuning( int kernel, int target_workgroups, int tile_rows );
-/* Plain f16 products (gh_matmul, the two of gh_matmul_pair, the product inside gh_matmul_accum and gh_matmul_silu_gate where no
+/* Opt-in: plain f16 products (gh_matmul, the two of gh_matmul_pair, the product inside gh_matmul_accum and gh_matmul_silu_gate where no
  * kernel of this library fuses it) of `rows` activation rows and more go to the vendor's GEMM library, as every product of the
- * reference's GPU target does (cublasGemmEx, arch/cuda/common/ops.cuh:666-700); 0: never; from half as many rows on for weight matrices that are not much wider than tall.  Default 768 (measured: from there on the library's kernels are the faster ones for nearly every shape of the 13B and
- * 70B models; below, the split-K tile kernel and the fused epilogues of this library are).  A forced kernel
- * (gh_gemm_set_tuning) also keeps the library out.  GLINT_LIBRARY_ROWS in the environment replaces the default. */
+ * reference's GPU target does (cublasGemmEx, arch/cuda/common/ops.cuh:666-700); from half as many rows on for weight matrices that
+ * are not much wider than tall.  Default 0: never, every product runs on the kernels of this library.  A forced kernel
+ * (gh_gemm_set_tuning) also keeps the vendor library out.  GLINT_LIBRARY_ROWS in the environment replaces the default. */
 int gh_gemm_set_library_rows( uint64_t rows );
+uint64_t gh_gemm_library_rows( void ); /* the row count in force */
+/* host-only: how many products the vendor's GEMM library has run for this process so far (a declined product -- library or
+ * algorithm missing -- is not counted and runs on the kernels of this library): lets a test or a benchmark say which route ran */
+uint64_t gh_gemm_library_calls( void );
 /* host-only query: 1 when gh_matmul_accum runs a product of this shape (16-byte aligned operands) in the large tile kernel with the residual added
  * in its epilogue, i.e. without fp32 partial sums of (b, r): the caller's test for taking the fused call on many rows */
 int gh_matmul_fuses_many_rows( uint64_t s, uint64_t r, uint64_t b, gh_dtype dt );

@@ -155,6 +155,7 @@ def test_config3_llama13b_prefill_8x2048_then_decode(product_route):
             assert a <= 2e-2 and r <= 2e-3, f"13B prefill: cache row of context {i}, token {t}: max_abs {a:.2e}, mean_rel {r:.2e}"
             caches[i][t] = saved[k]              # later rows are checked against what the GPU holds
     assert worst > 0.0
+    product_route.check()                        # the prefill's plain products ran where the route says
 
     # (c) decode steps on the caches the prefill left (MHA: the dot2/DPP kernel over 2049.. keys)
     for step in range(3):

@@ -137,3 +137,24 @@ def test_attention_stage_takes_a_state_of_the_other_type(fused):
         assert_close(out_b, want, what=f"attention from an fp32 state, step {step}")
     a.close()
     b.close()
+
+
+def test_convert_and_copy_of_void_is_a_byte_copy():
+    """The instantiation the reference's concept names, convert_and_copy<void, void>
+    (models/llama2/ops/concept.hh:36): its element is a byte (arch/amd64/llama2/ops.hh:361-362 with
+    sizeof(void) == 1), so `size` bytes travel unchanged, whatever their number, in every direction."""
+    st = S.Stage("test-tiny", "f16", 0, 1, 2, 2)
+    rng = np.random.default_rng(5)
+    for n in (1, 7, 4099):                                           # odd counts: no element type divides them
+        src = rng.integers(0, 256, n, dtype=np.uint8)
+        dev = torch.zeros(n + 2, dtype=torch.uint8, device="cuda")
+        dev2 = torch.zeros(n + 2, dtype=torch.uint8, device="cuda")
+        back = np.zeros(n + 2, dtype=np.uint8)
+        st.copy_bytes(dev.data_ptr(), src.ctypes.data, n, GH_H2D)
+        st.copy_bytes(dev2.data_ptr(), dev.data_ptr(), n, GH_D2D)
+        st.copy_bytes(back.ctypes.data, dev2.data_ptr(), n, GH_D2H)
+        assert np.array_equal(back[:n], src) and not back[n:].any()   # nothing beyond `size` bytes
+        again = np.zeros(n, dtype=np.uint8)
+        st.copy_bytes(again.ctypes.data, src.ctypes.data, n, GH_H2H)
+        assert np.array_equal(again, src)
+    st.close()

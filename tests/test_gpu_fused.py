@@ -47,6 +47,8 @@ def test_matmul_accum_and_norm(dt, b, s, r, product_route):
     o_res = res.float().cpu().numpy()
     O.accum(o_res, O.matmul(x.float().cpu().numpy(), w.float().cpu().numpy()))
     assert_close(got_norm.float().cpu().numpy(), O.rmsnorm(o_res, nw.float().cpu().numpy()), what="fused accum+rmsnorm")
+    # the plain product of the separate ops and the product inside each of the two fused calls
+    product_route.check(3 if dt == torch.float16 and product_route.wanted(b, s, r) else 0)
 
 
 @pytest.mark.parametrize("dt", [torch.float16, torch.float32])
@@ -54,7 +56,7 @@ def test_matmul_accum_and_norm(dt, b, s, r, product_route):
                                         # enough row tiles for one launch without a K split: both factors in one kernel
                                         (64, 512, 16384), (5, 256, 16404), (33, 1024, 28672),
                                         (5, 256, 16386)])     # rows not a multiple of 4: the two-kernel route
-def test_matmul_silu_gate(dt, b, s, hidden):
+def test_matmul_silu_gate(dt, b, s, hidden, product_route):
     g = torch.Generator(device="cuda").manual_seed(2)
     x = torch.randn((b, s), generator=g, device="cuda").to(dt)
     w13 = (torch.randn((2 * hidden, s), generator=g, device="cuda") / s ** 0.5).to(dt)
@@ -71,6 +73,10 @@ def test_matmul_silu_gate(dt, b, s, hidden):
         want = O.matmul(xh, np.ascontiguousarray(wh[:hidden]))
         O.silu(want, O.matmul(xh, np.ascontiguousarray(wh[hidden:])))
         assert_close(got.float().cpu().numpy(), want, what="fused w1, w3, silu")
+    # some hundred rows and a wide [w1; w3]: one product of the vendor library, then the gate over the two halves of each row
+    wide = dt == torch.float16 and 128 <= b < product_route.ROWS and 2 * hidden >= 16384 and s % 8 == 0 and hidden % 8 == 0
+    plain = 2 if dt == torch.float16 and product_route.wanted(b, s, hidden) else 0        # the two separate products above
+    product_route.check(plain + (1 if wide else 0))
 
 
 @pytest.mark.parametrize("dt", [torch.float16, torch.float32])

@@ -283,6 +283,7 @@ def test_matmul_token_split_one_hot(b, s, r, product_route):
     x[torch.arange(b, device="cuda"), cols] = 1
     got = ops.matmul(x, w)
     assert torch.equal(got, w[:, cols].t().contiguous())
+    product_route.check(1)
 
 
 # two products that share their activations (wq and wkv): few rows take the two-call route, many rows one launch of the large tile
@@ -309,6 +310,8 @@ def test_matmul_pair(dt, b, s, ra, rb, product_route):
     want = xr.float() @ wr.float().t()
     err = (torch.cat([got_a, got_b], dim=1).float() - want).abs()
     assert err.max().item() < 2e-2 and (err.mean() / want.abs().mean()).item() < 1e-3
+    both = dt == "f16" and product_route.wanted(b, s, ra) and product_route.wanted(b, s, rb)   # else one launch of the tile kernel, or two plain calls
+    product_route.check(4 if both else 0)
 
 
 def test_matmul_many_rows_repeatable(product_route):
@@ -321,6 +324,7 @@ def test_matmul_many_rows_repeatable(product_route):
     ops.matmul(torch.flip(x, dims=[0]).contiguous(), w)
     again = ops.matmul(x, w)
     assert torch.equal(first, again)
+    product_route.check(3)
     want = x.float() @ w.float().t()
     err = (first.float() - want).abs()
     assert err.max().item() < 2e-2 and (err.mean() / want.abs().mean()).item() < 1e-3
@@ -423,6 +427,42 @@ def test_rope_cache_row_not_16_byte_aligned():
     # nothing outside the K halves moved
     assert np.array_equal(got[0, :1], rows[0, :1]) and np.array_equal(got[0, 1 + shape.kv_dim:], rows[0, 1 + shape.kv_dim:])
     assert np.array_equal(got[1, shape.kv_dim:], rows[1, shape.kv_dim:])
+
+
+# The positions of the device-table entry points never pass through the host, so the kernels bound them themselves: a position at
+# or beyond seq_len reads no cache row past the context's last one and writes no score past the end of its row, also where the
+# token ranges of the launch are rounded up beyond seq_len (seq_len not a multiple of the range granularity).
+@pytest.mark.parametrize("shape", [Shape(dim=1024, n_layers=1, n_heads=8, n_kv_heads=1, hidden_dim=64, seq_len=1000),     # gqa 8: MFMA kernels
+                                   Shape(dim=512, n_layers=1, n_heads=4, n_kv_heads=4, hidden_dim=64, seq_len=1000)],    # MHA: dot2 kernels
+                         ids=["gqa8", "mha"])
+def test_unfused_attention_ops_bound_a_bad_position_by_seq_len(shape):
+    batch, guard = 3, 4096
+    arena = Arena(shape, batch + 1, torch.float16, seed=41)                 # the context behind the last one is the guard: all NaN
+    arena.dev[batch].fill_(float("nan"))
+    rng = np.random.default_rng(42)
+    dq = torch.from_numpy(rng.standard_normal((batch, shape.dim)).astype(np.float16)).cuda()
+    rows = ops.row_table([arena.layer_ptr(i) for i in range(batch)])
+    n_att = batch * shape.n_heads * shape.seq_len
+    good = torch.tensor([999, 999, 5], dtype=torch.int32, device="cuda")
+    bad = torch.tensor([999, 1010, 5], dtype=torch.int32, device="cuda")    # context 1: beyond its 1000 rows
+    outs = []
+    for pos in (good, bad):
+        buf = torch.full((n_att + guard,), 3.0, dtype=torch.float16, device="cuda")
+        att = buf[:n_att].view(batch, shape.n_heads, shape.seq_len)
+        ops.attn_scores(dq, rows, att, pos, shape)
+        ops.sync()
+        assert torch.all(buf[n_att:] == 3.0)                                # nothing written behind the last row of scores
+        assert torch.isfinite(att.float()).all()                            # no row of the guard context was read
+        outs.append(att.clone())
+        ops.attn_softmax(att, pos, shape)
+        xb = torch.full((batch + 1, shape.dim), 5.0, dtype=torch.float16, device="cuda")
+        ops.attn_pv(att, rows, xb[:batch], pos, shape)
+        ops.sync()
+        assert torch.all(buf[n_att:] == 3.0) and torch.all(xb[batch] == 5.0)
+        assert torch.isfinite(xb[:batch].float()).all()
+        outs.append(xb[:batch].clone())
+    # the bad position behaves as the last valid one, and the other contexts are what they are without it
+    assert torch.equal(outs[0], outs[2]) and torch.equal(outs[1], outs[3])
 
 
 # ------------------------------------------------------------------ unfused attention ops

@@ -105,3 +105,39 @@ def test_static_scratch_entry_point_refuses_what_does_not_fit():
     ops.attn_decode(q, rows, pos, xb, 1023, wide)
     ops.sync()
     assert float(xb.float().abs().max()) == 0.0                                                   # all-zero V rows
+
+
+def test_static_scratch_entry_point_allocates_nothing():
+    """The property the entry point exists for.  Around a call on a shape and batch this process has not run before (a plan of its
+    own, several splits): the library's count of its own allocations stands still and so does the driver's count of free device
+    memory; the same call through the workspace entry point is what the result is compared with, afterwards."""
+    ops.init(0)
+    L = _lib.lib()
+    shape = Shape(dim=1536, n_layers=1, n_heads=12, n_kv_heads=3, hidden_dim=64, seq_len=1536)     # head 128, gqa 4; used nowhere else
+    positions = [1535, 1201, 77, 640, 1024, 3]
+    batch = len(positions)
+    splits, need = plan_bytes(batch, max(positions), shape)
+    assert splits > 1 and 0 < need <= 16 << 20
+    arena = Arena(shape, batch, torch.float16, seed=51)
+    rng = np.random.default_rng(52)
+    q = torch.from_numpy(rng.standard_normal((batch, shape.dim)).astype(np.float16)).cuda()
+    rows = ops.row_table([arena.layer_ptr(i) for i in range(batch)])
+    pos = torch.tensor(positions, dtype=torch.int32, device="cuda")
+    got = torch.full((batch, shape.dim), 7.0, dtype=torch.float16, device="cuda")
+    want = got.clone()
+    # the code object is on the device and the launch path warm before anything is counted (a first launch loads code)
+    warm = Shape(dim=1024, n_layers=1, n_heads=8, n_kv_heads=2, hidden_dim=64, seq_len=1024)
+    run_both(warm, torch.float16, [1023, 5], seed=53)
+    torch.cuda.synchronize()
+    allocations = int(L.gh_allocation_count())
+    free_before, _ = torch.cuda.mem_get_info()
+    rc = decode_static(q, rows, pos, got, max(positions), shape)
+    ops.sync()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert rc == 0, L.gh_last_error()
+    assert int(L.gh_allocation_count()) == allocations          # no hipMalloc / hipHostMalloc / hipMemCreate of the library's
+    assert free_after == free_before                            # and none of anybody else's on its behalf
+    ops.attn_decode(q, rows, pos, want, max(positions), shape)
+    ops.sync()
+    assert torch.equal(got, want)
+    assert int(L.gh_allocation_count()) == allocations          # (the workspace above is torch's, not the library's)
