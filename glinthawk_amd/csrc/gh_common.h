@@ -88,7 +88,7 @@ public:
 // ---- library-owned device scratch ---------------------------------------------------------------
 // Grow-only buffer for purpose `which`, private to `stream`: work queued on different streams never
 // shares one.  Growing waits for that stream only.  `min_bytes` is the size of the first allocation.
-enum { SCRATCH_GEMM_PARTIALS = 0, SCRATCH_CONVERT = 1, SCRATCH_ATTN_PV = 2, SCRATCH_GATE_FACTOR = 3, SCRATCH_LIBRARY = 4, SCRATCH_PRODUCT = 5 };
+enum { SCRATCH_GEMM_PARTIALS = 0, SCRATCH_CONVERT = 1, SCRATCH_ATTN_PV = 2, SCRATCH_GATE_FACTOR = 3, SCRATCH_LIBRARY = 4, SCRATCH_PRODUCT = 5, SCRATCH_GEMM_PIECES = 6 };
 int stream_scratch( hipStream_t stream, int which, uint64_t bytes, uint64_t min_bytes, void** out );
 // gh_gemm_lib.hip: a plain f16 product through the vendor's GEMM library; *done = false: declined, nothing queued
 int gemm_library( void* xout, const void* x, const void* w, uint64_t s, uint64_t r, uint64_t b, hipStream_t st, bool* done );

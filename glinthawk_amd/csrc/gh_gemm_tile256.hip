@@ -82,6 +82,33 @@ struct TileOrder
   uint32_t rest_rows, rest_share;      // left-over row tiles; tiles of them per XCD
 };
 
+// Which tile work-group blockIdx.x takes; false: none (padding of the last patches).
+__device__ __forceinline__ bool tile_of_workgroup( const TileOrder& ord, uint32_t& row_tile, uint32_t& token_tile )
+{
+  const uint32_t xcd = blockIdx.x & 7; // work-groups go to the XCDs in turn
+  const uint32_t idx = blockIdx.x >> 3;
+  if ( idx < ord.main_per_xcd ) {
+    const uint32_t per_patch = ord.gm * ord.gn;
+    const uint32_t patch = idx / per_patch, in_patch = idx % per_patch;
+    const uint32_t patch_m = patch / ord.patches_n, patch_n = patch % ord.patches_n;
+    const uint32_t own_row = patch_m * ord.gm + in_patch / ord.gn;
+    row_tile = own_row * 8 + xcd;
+    token_tile = patch_n * ord.gn + in_patch % ord.gn;
+    return own_row < ord.rows_per_xcd && token_tile < ord.token_tiles;
+  }
+  const uint32_t mine = idx - ord.main_per_xcd;
+  const uint32_t u = xcd * ord.rest_share + mine;
+  if ( mine >= ord.rest_share || u >= ord.rest_rows * ord.token_tiles ) {
+    return false;
+  }
+  const uint32_t per_patch_col = ord.rest_rows * 8; // the last one may be narrower
+  const uint32_t patch_col = u / per_patch_col, in_col = u % per_patch_col;
+  const uint32_t width = min( 8u, ord.token_tiles - patch_col * 8 );
+  row_tile = ord.rows_per_xcd * 8 + in_col / width;
+  token_tile = patch_col * 8 + in_col % width;
+  return true;
+}
+
 constexpr int T256_THREADS = 512;
 
 // What a work-group does with its sums: xout = DType(sum); the reference's next op on top of that,
@@ -111,30 +138,9 @@ __global__ __launch_bounds__( T256_THREADS, 1 ) void gemm_tile256_kernel( __half
   constexpr int TM = 128 * NA; // weight rows per work-group: 4 waves x NA x 32
   __shared__ uint4 s_x0[TN2 * 8], s_x1[TN2 * 8]; // 2 x 32 KiB
   __shared__ uint4 s_w0[TM * 8], s_w1[TM * 8];   // 2 x 32 KiB, or 2 x 48 KiB: all 160 KiB of the CU
-  const uint32_t xcd = blockIdx.x & 7; // work-groups go to the XCDs in turn
-  const uint32_t idx = blockIdx.x >> 3;
   uint32_t row_tile, token_tile;
-  if ( idx < ord.main_per_xcd ) {
-    const uint32_t per_patch = ord.gm * ord.gn;
-    const uint32_t patch = idx / per_patch, in_patch = idx % per_patch;
-    const uint32_t patch_m = patch / ord.patches_n, patch_n = patch % ord.patches_n;
-    const uint32_t own_row = patch_m * ord.gm + in_patch / ord.gn;
-    row_tile = own_row * 8 + xcd;
-    token_tile = patch_n * ord.gn + in_patch % ord.gn;
-    if ( own_row >= ord.rows_per_xcd || token_tile >= ord.token_tiles ) {
-      return; // padding of the last patches (whole work-group)
-    }
-  } else {
-    const uint32_t mine = idx - ord.main_per_xcd;
-    const uint32_t u = xcd * ord.rest_share + mine;
-    if ( mine >= ord.rest_share || u >= ord.rest_rows * ord.token_tiles ) {
-      return;
-    }
-    const uint32_t per_patch_col = ord.rest_rows * 8; // the last one may be narrower
-    const uint32_t patch_col = u / per_patch_col, in_col = u % per_patch_col;
-    const uint32_t width = min( 8u, ord.token_tiles - patch_col * 8 );
-    row_tile = ord.rows_per_xcd * 8 + in_col / width;
-    token_tile = patch_col * 8 + in_col % width;
+  if ( !tile_of_workgroup( ord, row_tile, token_tile ) ) {
+    return; // padding of the last patches (whole work-group)
   }
   const uint32_t wave = __builtin_amdgcn_readfirstlane( threadIdx.x >> 6 );
   const uint32_t lane = threadIdx.x & 63;
@@ -411,7 +417,447 @@ __global__ __launch_bounds__( T256_THREADS, 1 ) void gemm_tile256_kernel( __half
   }
 }
 
+// The same 256 x 256 tile with FOUR waves of 128 x 128 (2 x 2), one wave per SIMD: 16 accumulators of v_mfma_f32_32x32x16_f16,
+// 256 registers, which the compiler keeps in the accumulation half of the register file (512 registers per lane with one wave per
+// SIMD), so the 256 ordinary registers are free for operands and addresses.  Against 64 x 128 per wave a 16-k group of a wave
+// needs 8 fragment reads for 16 MFMAs instead of 6 for 8: a third less LDS traffic per flop, half as many waves at the barrier.
+//
+//   schedule    With one wave per SIMD nothing else fills a stall, so the loop is laid out instruction by instruction
+//               (sched_group_barrier).  A step is four groups of 16 MFMAs.  Beside the first 8 MFMAs of a group go the 8 fragment
+//               reads of the NEXT group (two fragment sets in turn).  The barrier that ends the step stands in front of its last
+//               group: behind it the wave requests the first fragments of the next stage and still has 16 MFMAs in hand while
+//               they arrive.
+//   operands    global -> registers -> LDS, two steps ahead: the 16 loads of step j + 2 go out four to a group all through step
+//               j, and the 16 registers loaded during step j - 1 (step j + 1) are written to the other stage beside the first
+//               three groups of step j.  Every memory instruction of the loop is spread evenly between the MFMAs; that is what
+//               counts.  Measured at 16384 x 8192 x 8192 (matrix pipes busy of 4 per CU, clock): without any loads 3.74, 1.87 GHz,
+//               1.8-1.9 PFLOP/s; 16 loads back to back at the head of a step and never waited for 2.92 (the wave cannot issue
+//               MFMAs while its memory instructions queue for the address unit); loads straight to LDS one step ahead, in
+//               two bursts, 2.57, 1.04-1.07 PFLOP/s; the same spread evenly 1.28-1.30; as built here 3.48 at 1.29 GHz, 1.30
+//               PFLOP/s (the vendor library's kernel on the same box: 3.71 at 1.39 GHz, 1.31-1.52; the eight-wave kernel above
+//               3.05 at 1.35 GHz, 1.13-1.26).  Under this load the part runs at the clock its power budget allows.
+//   loop shape  one loop of two steps with a single exit: with the exit test between the steps (an odd number of steps) the
+//               compiler moved accumulators between the two register halves inside the loop (hundreds of copies per
+//               step and spills), so the kernel takes K ranges of an even number of 64-k steps only.
+//   work        either one tile per work-group in the tile order above, or (gemm_w4_streamk_kernel) one work-group per CU that
+//               walks an equal share of ALL the 64-k steps of the product, tile after tile: a product of 416 tiles on 256 CUs
+//               then takes 1.6 tiles' time instead of 2.  Tiles that a share covers whole are finished on the spot; the two
+//               pieces at the ends of a share leave fp32 sums in a buffer and gemm_w4_fixup_kernel adds the pieces of each
+//               divided tile in ascending order of the share (a fixed order: results repeat bit for bit).
+constexpr int T4_THREADS = 256;
+
+struct W4Stages
+{
+  uint4 *w0, *x0, *w1, *x1; // four separate arrays: see gemm_tile256_kernel
+};
+
+// acc = w[tile rows] . x[tile tokens]^T over n_steps (even) steps of 64 k, both descriptors starting at the range's first k.
+__device__ __forceinline__ void w4_multiply( f32x16 ( &acc )[4][4], const __amdgpu_buffer_rsrc_t w_rsrc, const __amdgpu_buffer_rsrc_t x_rsrc, uint32_t ld_bytes,
+                                             uint32_t n_steps, const W4Stages& st )
+{
+  const uint32_t wave = __builtin_amdgcn_readfirstlane( threadIdx.x >> 6 );
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t wr = wave >> 1, wc = wave & 1;
+  const uint32_t fr = lane & 31, g2 = lane >> 5;
+  // thread t holds slot t % 8 of row t / 8 (+ 32 i): it fetches the chunk that the swizzle keeps in that slot
+  const uint32_t voff = ( threadIdx.x >> 3 ) * ld_bytes + ( ( threadIdx.x & 7 ) ^ ( ( threadIdx.x >> 4 ) & 7 ) ) * 16;
+  const uint32_t slot0 = 8 * wave * 8 + lane; // this thread's uint4 in the wave's 8 rows
+#pragma unroll
+  for ( int rt = 0; rt < 4; rt++ ) {
+#pragma unroll
+    for ( int t = 0; t < 4; t++ ) {
+#pragma unroll
+      for ( int e = 0; e < 16; e++ ) {
+        acc[rt][t][e] = 0.f;
+      }
+    }
+  }
+  struct Frags
+  {
+    f16x8 a[4], bb[4];
+  };
+  Frags f0, f1;
+  uint4 ra[16], rq[16]; // W0 X0 W1 X1 ... W7 X7 of a step (32 rows of the tile each), two steps in turn
+  auto read_k16 = [&]( Frags& f, const uint4* wt, const uint4* xt, int kk ) __attribute__( ( always_inline ) ) {
+    const uint32_t ch = 2 * kk + g2;
+#pragma unroll
+    for ( int i = 0; i < 4; i++ ) {
+      f.a[i] = __builtin_bit_cast( f16x8, wt[swz( 128 * wr + 32 * i + fr, ch )] );
+      f.bb[i] = __builtin_bit_cast( f16x8, xt[swz( 128 * wc + 32 * i + fr, ch )] );
+    }
+  };
+  auto mfma_k16 = [&]( const Frags& f ) __attribute__( ( always_inline ) ) {
+#pragma unroll
+    for ( int t = 0; t < 4; t++ ) {
+#pragma unroll
+      for ( int rt = 0; rt < 4; rt++ ) {
+        acc[rt][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16( f.a[rt], f.bb[t], acc[rt][t], 0, 0, 0 );
+      }
+    }
+  };
+  auto load_part = [&]( uint4* set, uint32_t kb, int from, int to ) __attribute__( ( always_inline ) ) {
+#pragma unroll
+    for ( int l = 0; l < 16; l++ ) {
+      if ( l >= from && l < to ) {
+        set[l] = __builtin_bit_cast( uint4, __builtin_amdgcn_raw_buffer_load_b128( ( l & 1 ) == 0 ? w_rsrc : x_rsrc, voff, 32 * ( l >> 1 ) * ld_bytes + kb, 0 ) );
+      }
+    }
+  };
+  auto store_part = [&]( const uint4* set, uint4* wn, uint4* xn, int from, int to ) __attribute__( ( always_inline ) ) {
+#pragma unroll
+    for ( int l = 0; l < 16; l++ ) {
+      if ( l >= from && l < to ) {
+        ( ( l & 1 ) == 0 ? wn : xn )[slot0 + 32 * ( l >> 1 ) * 8] = set[l];
+      }
+    }
+  };
+  // order of a group: MFMA i with an LDS read (i < 8), a load (i = 1, 5, 9, 13) and an LDS write (the first n_st of i = 2, 4, 7, 10, 12, 15)
+  auto order = [&]( int n_st ) __attribute__( ( always_inline ) ) {
+    int done = 0;
+#pragma unroll
+    for ( int i = 0; i < 16; i++ ) {
+      __builtin_amdgcn_sched_group_barrier( 0x008, 1, 0 ); // one MFMA
+      if ( i < 8 ) {
+        __builtin_amdgcn_sched_group_barrier( 0x100, 1, 0 ); // one LDS read
+      }
+      if ( ( i & 3 ) == 1 ) {
+        __builtin_amdgcn_sched_group_barrier( 0x020, 1, 0 ); // one load
+      }
+      if ( ( i == 2 || i == 4 || i == 7 || i == 10 || i == 12 || i == 15 ) && done < n_st ) {
+        __builtin_amdgcn_sched_group_barrier( 0x200, 1, 0 ); // one LDS write
+        done++;
+      }
+    }
+  };
+  // f0 holds the first group of stage (wt, xt) on entry and that of stage (wn, xn) on exit; `loaded` holds the operands of step
+  // j + 1, `loading` receives those of step j + 2 (behind the last step: the start of the next rows, bounded by the descriptors,
+  // never multiplied)
+  auto step = [&]( const uint4* wt, const uint4* xt, uint4* wn, uint4* xn, uint4* loading, const uint4* loaded, uint32_t j ) __attribute__( ( always_inline ) ) {
+    const uint32_t kb = ( j + 2 ) * TKS * 2;
+    read_k16( f1, wt, xt, 1 );
+    load_part( loading, kb, 0, 4 );
+    store_part( loaded, wn, xn, 0, 6 );
+    mfma_k16( f0 );
+    order( 6 );
+    __builtin_amdgcn_sched_barrier( 0 );
+    read_k16( f0, wt, xt, 2 );
+    load_part( loading, kb, 4, 8 );
+    store_part( loaded, wn, xn, 6, 11 );
+    mfma_k16( f1 );
+    order( 5 );
+    __builtin_amdgcn_sched_barrier( 0 );
+    read_k16( f1, wt, xt, 3 );
+    load_part( loading, kb, 8, 12 );
+    store_part( loaded, wn, xn, 11, 16 );
+    mfma_k16( f0 );
+    order( 5 );
+    __builtin_amdgcn_sched_barrier( 0 );
+    __syncthreads(); // the next stage is written, and every wave has read the last fragments of this one
+    __builtin_amdgcn_sched_barrier( 0 );
+    read_k16( f0, wn, xn, 0 );
+    load_part( loading, kb, 12, 16 );
+    mfma_k16( f1 );
+    order( 0 );
+    __builtin_amdgcn_sched_barrier( 0 );
+  };
+  load_part( ra, 0, 0, 16 );
+  load_part( rq, TKS * 2, 0, 16 );
+  store_part( ra, st.w0, st.x0, 0, 16 );
+  __syncthreads();
+  read_k16( f0, st.w0, st.x0, 0 );
+  for ( uint32_t j = 0; j < n_steps; j += 2 ) {
+    step( st.w0, st.x0, st.w1, st.x1, ra, rq, j );
+    step( st.w1, st.x1, st.w0, st.x0, rq, ra, j + 1 );
+  }
+}
+
+// acc[rt][t][v]: row = tile_row0 + 128*wr + 32*rt + 8*(v/4) + 4*(lane/32) + v%4, token = tile_col0 + 128*wc + 32*t + lane%32.
+// Output of a whole tile: through LDS (token-major, the four stage arrays as four regions of 64 tokens x 256 rows) as whole row
+// segments where r % 8 == 0, else (and for the fp32 sums of a K split) from the registers.
+struct W4Out
+{
+  __half* xout;
+  __half* xout2;    // rows from r_first on go here, as rows 0.. of a (b, r - r_first) matrix
+  float* partial;   // EPI_PARTIAL: (splits, b, r)
+  uint32_t r, b, r_first, split;
+};
+
+template<int EPI>
+__device__ __forceinline__ void w4_store_tile( f32x16 ( &acc )[4][4], const W4Out& o, uint32_t tile_row0, uint32_t tile_col0, const W4Stages& st )
+{
+  const uint32_t wave = __builtin_amdgcn_readfirstlane( threadIdx.x >> 6 );
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t wr = wave >> 1, wc = wave & 1;
+  const uint32_t fr = lane & 31, g2 = lane >> 5;
+  constexpr bool PARTIAL = EPI == EPI_PARTIAL;
+  if ( !PARTIAL && ( o.r & 7 ) == 0 ) {
+    __syncthreads(); // (the fragments requested behind the last barrier are not used; nothing is in flight into the arrays any more)
+    constexpr uint32_t CHUNKS = TM2 / 8; // 16-byte chunks per token
+    constexpr uint32_t SWZ_MASK = 31;
+#pragma unroll
+    for ( int t = 0; t < 4; t++ ) {
+      uint2* out = reinterpret_cast<uint2*>( wc == 0 ? ( t < 2 ? st.x0 : st.x1 ) : ( t < 2 ? st.w0 : st.w1 ) );
+      const uint32_t token = 32 * ( t & 1 ) + fr;
+#pragma unroll
+      for ( int rt = 0; rt < 4; rt++ ) {
+#pragma unroll
+        for ( int q4 = 0; q4 < 4; q4++ ) {
+          union
+          {
+            uint2 raw;
+            __half h[4];
+          } v;
+#pragma unroll
+          for ( int e = 0; e < 4; e++ ) {
+            v.h[e] = __float2half_rn( acc[rt][t][4 * q4 + e] );
+          }
+          const uint32_t chunk = 16 * wr + 4 * rt + q4;
+          out[( token * CHUNKS + ( chunk ^ ( token & SWZ_MASK ) ) ) * 2 + g2] = v.raw;
+        }
+      }
+    }
+    __syncthreads();
+#pragma unroll 4
+    for ( int it = 0; it < 32; it++ ) {
+      const uint4* region = it < 8 ? st.x0 : it < 16 ? st.x1 : it < 24 ? st.w0 : st.w1;
+      const uint32_t j = ( it % 8 ) * T4_THREADS + threadIdx.x;
+      const uint32_t token = j / CHUNKS, slot = j % CHUNKS;
+      const uint32_t chunk = slot ^ ( token & SWZ_MASK );
+      const uint32_t col = tile_col0 + 64 * ( it / 8 ) + token, row = tile_row0 + 8 * chunk;
+      if ( col < o.b && row < o.r ) {
+        const bool second = row >= o.r_first; // two products that share their activations in one launch (r_first % 8 == 0)
+        uint4* dst = reinterpret_cast<uint4*>( second ? o.xout2 + (uint64_t)col * ( o.r - o.r_first ) + ( row - o.r_first ) : o.xout + (uint64_t)col * o.r_first + row );
+        union
+        {
+          uint4 raw;
+          __half h[8];
+        } y, old;
+        y.raw = region[j];
+        if ( EPI == EPI_ACCUM ) { // the op that follows the product, on the rounded product
+          old.raw = *dst;
+#pragma unroll
+          for ( int e = 0; e < 8; e++ ) {
+            y.h[e] = __float2half_rn( __half2float( old.h[e] ) + __half2float( y.h[e] ) );
+          }
+        }
+        *dst = y.raw;
+      }
+    }
+    return;
+  }
+#pragma unroll
+  for ( int t = 0; t < 4; t++ ) {
+    const uint32_t col = tile_col0 + 128 * wc + 32 * t + fr;
+    if ( col >= o.b ) {
+      continue;
+    }
+#pragma unroll
+    for ( int rt = 0; rt < 4; rt++ ) {
+#pragma unroll
+      for ( int q4 = 0; q4 < 4; q4++ ) {
+        const uint32_t row = tile_row0 + 128 * wr + 32 * rt + 8 * q4 + 4 * g2;
+        const bool whole = row + 3 < o.r && ( o.r & 3 ) == 0;
+        if ( PARTIAL ) {
+          float* dst = o.partial + ( (uint64_t)o.split * o.b + col ) * o.r + row;
+          if ( whole ) {
+            *reinterpret_cast<float4*>( dst ) = make_float4( acc[rt][t][4 * q4], acc[rt][t][4 * q4 + 1], acc[rt][t][4 * q4 + 2], acc[rt][t][4 * q4 + 3] );
+          } else {
+            for ( int e = 0; e < 4; e++ ) {
+              if ( row + e < o.r ) {
+                dst[e] = acc[rt][t][4 * q4 + e];
+              }
+            }
+          }
+        } else {
+          __half* dst = o.xout + (uint64_t)col * o.r + row; // (one output only: the launch refuses two with r % 8 != 0)
+          if ( whole ) {
+            union
+            {
+              uint2 raw;
+              __half h[4];
+            } v;
+#pragma unroll
+            for ( int e = 0; e < 4; e++ ) {
+              v.h[e] = __float2half_rn( acc[rt][t][4 * q4 + e] );
+            }
+            *reinterpret_cast<uint2*>( dst ) = v.raw;
+          } else {
+            for ( int e = 0; e < 4; e++ ) {
+              if ( row + e < o.r ) {
+                dst[e] = __float2half_rn( acc[rt][t][4 * q4 + e] );
+              }
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
+// grid as gemm_tile256_kernel: 8 x (padded tiles of one XCD) by K splits; k_len % 128 == 0, s % 128 == 0
+template<int EPI>
+__global__ __launch_bounds__( T4_THREADS, 1 ) void gemm_tile256w4_kernel( __half* __restrict__ xout,
+                                                                        float* __restrict__ partial,
+                                                                        const __half* __restrict__ x,
+                                                                        const __half* __restrict__ w,
+                                                                        uint32_t s,
+                                                                        uint32_t r,
+                                                                        uint32_t b,
+                                                                        uint32_t k_len,
+                                                                        __half* __restrict__ xout2,
+                                                                        uint32_t r_first,
+                                                                        TileOrder ord )
+{
+  __shared__ uint4 s_x0[TN2 * 8], s_x1[TN2 * 8];
+  __shared__ uint4 s_w0[TM2 * 8], s_w1[TM2 * 8];
+  uint32_t row_tile, token_tile;
+  if ( !tile_of_workgroup( ord, row_tile, token_tile ) ) {
+    return;
+  }
+  const uint32_t tile_row0 = row_tile * TM2, tile_col0 = token_tile * TN2;
+  const uint32_t ld_bytes = s * 2;
+  const uint32_t w_rows = min( (uint32_t)TM2, r - tile_row0 ), x_cols = min( (uint32_t)TN2, b - tile_col0 );
+  const uint32_t k0 = blockIdx.y * k_len; // this split's k range starts here; the descriptors start there too and end with the tile's last row
+  const __amdgpu_buffer_rsrc_t w_rsrc
+    = __builtin_amdgcn_make_buffer_rsrc( const_cast<__half*>( w + (uint64_t)tile_row0 * s + k0 ), 0, (int)( w_rows * ld_bytes - k0 * 2 ), 0x00020000 );
+  const __amdgpu_buffer_rsrc_t x_rsrc
+    = __builtin_amdgcn_make_buffer_rsrc( const_cast<__half*>( x + (uint64_t)tile_col0 * s + k0 ), 0, (int)( x_cols * ld_bytes - k0 * 2 ), 0x00020000 );
+  const W4Stages st { s_w0, s_x0, s_w1, s_x1 };
+  f32x16 acc[4][4];
+  w4_multiply( acc, w_rsrc, x_rsrc, ld_bytes, min( k_len, s - k0 ) / TKS, st );
+  const W4Out o { xout, xout2, partial, r, b, r_first, blockIdx.y };
+  w4_store_tile<EPI>( acc, o, tile_row0, tile_col0, st );
+}
+
+// Equal shares of all the 64-k steps of a product.  Tile t (token fastest: t = row tile x token tiles + token tile) owns the steps
+// [t * steps, (t + 1) * steps) of the product's list; share g takes [g * share, (g + 1) * share) of it, an even number of steps.
+// Shares are dealt to the work-groups so that the 32 of an XCD (work-groups x, x + 8, ...) hold neighbouring shares: their tiles
+// are a few neighbouring row tiles over all their token tiles and share their operands in that XCD's L2.
+struct StreamK
+{
+  uint32_t tiles, token_tiles, steps, share, shares;
+  float* pieces; // (shares, 2) pieces of 256 x 256 fp32 sums in register order: [wave][rt][t][v / 4][lane][v % 4]
+};
+constexpr uint64_t PIECE_FLOATS = (uint64_t)TM2 * TN2;
+
+__device__ __forceinline__ uint32_t streamk_share_of_workgroup( const StreamK& sk )
+{
+  const uint32_t per_xcd = ( sk.shares + 7 ) / 8; // work-group g runs on XCD g % 8
+  return ( blockIdx.x & 7 ) * per_xcd + ( blockIdx.x >> 3 );
+}
+
+// grid: 8 * ceil(shares / 8) work-groups, one per CU
+template<int EPI>
+__global__ __launch_bounds__( T4_THREADS, 1 ) void gemm_w4_streamk_kernel( __half* __restrict__ xout,
+                                                                         const __half* __restrict__ x,
+                                                                         const __half* __restrict__ w,
+                                                                         uint32_t s,
+                                                                         uint32_t r,
+                                                                         uint32_t b,
+                                                                         __half* __restrict__ xout2,
+                                                                         uint32_t r_first,
+                                                                         StreamK sk )
+{
+  __shared__ uint4 s_x0[TN2 * 8], s_x1[TN2 * 8];
+  __shared__ uint4 s_w0[TM2 * 8], s_w1[TM2 * 8];
+  const uint32_t g = streamk_share_of_workgroup( sk );
+  const uint64_t total = (uint64_t)sk.tiles * sk.steps;
+  const uint64_t begin = (uint64_t)g * sk.share;
+  if ( g >= sk.shares || begin >= total ) {
+    return;
+  }
+  const uint64_t end = min( total, begin + sk.share );
+  const W4Stages st { s_w0, s_x0, s_w1, s_x1 };
+  const uint32_t ld_bytes = s * 2;
+  const uint32_t first_tile = (uint32_t)( begin / sk.steps );
+  const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for ( uint64_t at = begin; at < end; ) {
+    const uint32_t tile = (uint32_t)( at / sk.steps );
+    const uint32_t step0 = (uint32_t)( at - (uint64_t)tile * sk.steps );
+    const uint32_t n_steps = (uint32_t)min( (uint64_t)( sk.steps - step0 ), end - at );
+    const uint32_t tile_row0 = ( tile / sk.token_tiles ) * TM2, tile_col0 = ( tile % sk.token_tiles ) * TN2;
+    const uint32_t w_rows = min( (uint32_t)TM2, r - tile_row0 ), x_cols = min( (uint32_t)TN2, b - tile_col0 );
+    const uint32_t k0 = step0 * TKS;
+    const __amdgpu_buffer_rsrc_t w_rsrc
+      = __builtin_amdgcn_make_buffer_rsrc( const_cast<__half*>( w + (uint64_t)tile_row0 * s + k0 ), 0, (int)( w_rows * ld_bytes - k0 * 2 ), 0x00020000 );
+    const __amdgpu_buffer_rsrc_t x_rsrc
+      = __builtin_amdgcn_make_buffer_rsrc( const_cast<__half*>( x + (uint64_t)tile_col0 * s + k0 ), 0, (int)( x_cols * ld_bytes - k0 * 2 ), 0x00020000 );
+    f32x16 acc[4][4];
+    w4_multiply( acc, w_rsrc, x_rsrc, ld_bytes, n_steps, st );
+    if ( n_steps == sk.steps ) { // a whole tile: finished here
+      const W4Out o { xout, xout2, nullptr, r, b, r_first, 0 };
+      w4_store_tile<EPI>( acc, o, tile_row0, tile_col0, st );
+    } else { // a piece: its sums as they lie in the registers, 1 KiB per wave and store
+      float* piece = sk.pieces + ( (uint64_t)g * 2 + ( tile == first_tile ? 0 : 1 ) ) * PIECE_FLOATS + (uint64_t)wave * ( PIECE_FLOATS / 4 );
+#pragma unroll
+      for ( int rt = 0; rt < 4; rt++ ) {
+#pragma unroll
+        for ( int t = 0; t < 4; t++ ) {
+#pragma unroll
+          for ( int q4 = 0; q4 < 4; q4++ ) {
+            *reinterpret_cast<float4*>( piece + ( ( ( rt * 4 + t ) * 4 + q4 ) * 64 + lane ) * 4 )
+              = make_float4( acc[rt][t][4 * q4], acc[rt][t][4 * q4 + 1], acc[rt][t][4 * q4 + 2], acc[rt][t][4 * q4 + 3] );
+          }
+        }
+      }
+    }
+    __syncthreads(); // the stage arrays serve the next tile
+    at += n_steps;
+  }
+}
+
+// One work-group per tile: nothing to do for a tile that one share covered whole; else the pieces of the tile added in ascending
+// order of the share, then the same output path as a tile finished in the multiply kernel.
+template<int EPI>
+__global__ __launch_bounds__( T4_THREADS, 1 ) void gemm_w4_fixup_kernel( __half* __restrict__ xout, uint32_t r, uint32_t b, __half* __restrict__ xout2, uint32_t r_first,
+                                                                       StreamK sk )
+{
+  __shared__ uint4 s_x0[TN2 * 8], s_x1[TN2 * 8];
+  __shared__ uint4 s_w0[TM2 * 8], s_w1[TM2 * 8];
+  const uint32_t tile = blockIdx.x;
+  const uint64_t t_begin = (uint64_t)tile * sk.steps, t_end = t_begin + sk.steps;
+  const uint32_t g_first = (uint32_t)( t_begin / sk.share ), g_last = (uint32_t)( ( t_end - 1 ) / sk.share );
+  if ( g_first == g_last ) {
+    return;
+  }
+  const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  f32x16 acc[4][4];
+#pragma unroll
+  for ( int rt = 0; rt < 4; rt++ ) {
+#pragma unroll
+    for ( int t = 0; t < 4; t++ ) {
+#pragma unroll
+      for ( int e = 0; e < 16; e++ ) {
+        acc[rt][t][e] = 0.f;
+      }
+    }
+  }
+  for ( uint32_t g = g_first; g <= g_last; g++ ) {
+    const uint32_t first_tile = (uint32_t)( (uint64_t)g * sk.share / sk.steps );
+    const float* piece = sk.pieces + ( (uint64_t)g * 2 + ( tile == first_tile ? 0 : 1 ) ) * PIECE_FLOATS + (uint64_t)wave * ( PIECE_FLOATS / 4 );
+#pragma unroll
+    for ( int rt = 0; rt < 4; rt++ ) {
+#pragma unroll
+      for ( int t = 0; t < 4; t++ ) {
+#pragma unroll
+        for ( int q4 = 0; q4 < 4; q4++ ) {
+          const float4 v = *reinterpret_cast<const float4*>( piece + ( ( ( rt * 4 + t ) * 4 + q4 ) * 64 + lane ) * 4 );
+          acc[rt][t][4 * q4] += v.x;
+          acc[rt][t][4 * q4 + 1] += v.y;
+          acc[rt][t][4 * q4 + 2] += v.z;
+          acc[rt][t][4 * q4 + 3] += v.w;
+        }
+      }
+    }
+  }
+  const W4Stages st { s_w0, s_x0, s_w1, s_x1 };
+  const W4Out o { xout, xout2, nullptr, r, b, r_first, 0 };
+  w4_store_tile<EPI>( acc, o, ( tile / sk.token_tiles ) * TM2, ( tile % sk.token_tiles ) * TN2, st );
+}
+
 int g_tile_rows = 0; // 0: by tile256_rows(); 256 or 384: forced
+// measurement hook (tile rows): 256 or 384 force the eight-wave kernel, 128 the four-wave one with one tile per work-group, 129 the
+// four-wave one over equal shares of all steps; 0: the four-wave kernel wherever it applies, equal shares where whole tiles fit badly
 
 // Rounds of one work-group per CU that an XCD (32 CUs) runs for its share of the tiles.
 uint64_t rounds_per_xcd( uint64_t r, uint64_t b, uint64_t tile_rows )
@@ -430,8 +876,43 @@ uint32_t tile256_rows( uint64_t s, uint64_t r, uint64_t b )
   if ( g_tile_rows == 256 || g_tile_rows == 384 ) {
     return (uint32_t)g_tile_rows;
   }
+  if ( g_tile_rows == 128 || g_tile_rows == 129 ) {
+    return 256;
+  }
   const uint64_t round_cost_pct = s >= 7168 ? 143 : 136;
   return round_cost_pct * rounds_per_xcd( r, b, 384 ) < 97 * rounds_per_xcd( r, b, 256 ) ? 384 : 256; // 3 % in hand for 256
+}
+
+// Whether a product runs over equal shares of all its steps, and how: worth it when whole tiles would leave the last round of
+// one tile per CU partly empty.  `force`: whenever the shape allows.
+bool streamk_plan( uint64_t s, uint64_t r, uint64_t b, bool force, StreamK* sk )
+{
+  const uint64_t cus = (uint64_t)cu_count();
+  const uint64_t row_tiles = ( r + TM2 - 1 ) / TM2, token_tiles = ( b + TN2 - 1 ) / TN2;
+  const uint64_t tiles = row_tiles * token_tiles, steps = s / TKS;
+  if ( tiles == 0 || steps < 4 || steps % 2 != 0 || tiles > 0xffffffull ) {
+    return false;
+  }
+  const uint64_t rounds = ( tiles + cus - 1 ) / cus;
+  const uint64_t share = ( ( tiles * steps + 2 * cus - 1 ) / ( 2 * cus ) ) * 2; // even
+  // in steps of one CU: whole tiles take rounds x steps; shares take `share` plus the pieces' way through memory (one step's
+  // time for a piece written and one for a piece read is generous) and a second launch
+  // Measured (3328 tokens, 70B shapes): shares that start in the middle of tiles walk K out of step with their neighbours, so an
+  // operand strip is no longer fetched into the XCD's L2 once for all the tiles that use it at that moment, and the multiply
+  // runs at about three quarters of its rate in whole tiles; the pieces cost a launch and 2 x 256 KiB of traffic each on top.
+  // 520 tiles (2.03 rounds, 3 as whole tiles): 493 against 543 us; 416 tiles (1.63 rounds): 452 against 392 us.  So only where
+  // whole tiles waste more than 30 % of their rounds.
+  const bool pays = 100 * ( share + 6 ) < 70 * rounds * steps && share >= 8;
+  if ( !force && !pays ) {
+    return false;
+  }
+  sk->tiles = (uint32_t)tiles;
+  sk->token_tiles = (uint32_t)token_tiles;
+  sk->steps = (uint32_t)steps;
+  sk->share = (uint32_t)std::max<uint64_t>( share, 2 );
+  sk->shares = (uint32_t)( ( tiles * steps + sk->share - 1 ) / sk->share );
+  sk->pieces = nullptr;
+  return true;
 }
 
 } // namespace
@@ -525,7 +1006,40 @@ int gemm_tile256_launch( __half* xout, float* partial, const __half* x, const __
   if ( splits == 1 ) {
     k_len = (uint32_t)s;
   }
-  const uint32_t tile_rows = splits > 1 ? 256 : tile256_rows( s, r, b );
+  // four waves of 128 x 128 where the K range of every split is an even number of 64-k steps
+  const bool even_steps = s % ( 2 * TKS ) == 0 && k_len % ( 2 * TKS ) == 0;
+  // Measured against the eight-wave kernel (same box, same run): a round of four-wave tiles takes 0.92-0.97 of a round of
+  // eight-wave 256-row tiles where the chip is full (16384 tokens: 70B shapes 1.29-1.32 against 1.20-1.29 PFLOP/s, 13B wq 1.22
+  // against 1.16, w2 1.31 against 1.22), and more where it is not (1024 tokens x 8192 x 8192, half a round: 179 against 146 us --
+  // with idle CUs the part is not held back by its power budget, and two waves per SIMD cover a tile's start and end better).
+  const uint64_t cus = (uint64_t)cu_count();
+  const uint64_t tiles256 = ( ( r + TM2 - 1 ) / TM2 ) * ( ( b + TN2 - 1 ) / TN2 );
+  const uint64_t cost384 = s >= 7168 ? 143 : 136;
+  const bool four_pays = 2 * tiles256 >= 3 * cus && 94 * rounds_per_xcd( r, b, 256 ) <= cost384 * rounds_per_xcd( r, b, 384 );
+  const bool four_waves = even_steps && ( g_tile_rows == 128 || g_tile_rows == 129 || ( g_tile_rows == 0 && splits == 1 && four_pays ) );
+  GH_REQUIRE( ( g_tile_rows != 128 && g_tile_rows != 129 ) || even_steps, "gh_matmul: the four-wave tile kernel needs K ranges that are multiples of 128" );
+  const int epi_sk = epilogue;
+  if ( four_waves && splits == 1 && partial == nullptr && ( epi_sk == EPI_STORE || epi_sk == EPI_ACCUM ) && ( epi_sk != EPI_ACCUM || r % 8 == 0 ) ) {
+    StreamK sk;
+    if ( streamk_plan( s, r, b, g_tile_rows == 129, &sk ) ) {
+      void* pieces = nullptr;
+      if ( int rc = stream_scratch( st, SCRATCH_GEMM_PIECES, (uint64_t)sk.shares * 2 * PIECE_FLOATS * sizeof( float ), 0, &pieces ) ) {
+        return rc;
+      }
+      sk.pieces = static_cast<float*>( pieces );
+      const unsigned wgs = 8 * ( ( sk.shares + 7 ) / 8 );
+      if ( epi_sk == EPI_STORE ) {
+        gemm_w4_streamk_kernel<EPI_STORE><<<wgs, T4_THREADS, 0, st>>>( xout, x, w, (uint32_t)s, (uint32_t)r, (uint32_t)b, xout2, (uint32_t)r_first, sk );
+        gemm_w4_fixup_kernel<EPI_STORE><<<sk.tiles, T4_THREADS, 0, st>>>( xout, (uint32_t)r, (uint32_t)b, xout2, (uint32_t)r_first, sk );
+      } else {
+        gemm_w4_streamk_kernel<EPI_ACCUM><<<wgs, T4_THREADS, 0, st>>>( xout, x, w, (uint32_t)s, (uint32_t)r, (uint32_t)b, xout2, (uint32_t)r_first, sk );
+        gemm_w4_fixup_kernel<EPI_ACCUM><<<sk.tiles, T4_THREADS, 0, st>>>( xout, (uint32_t)r, (uint32_t)b, xout2, (uint32_t)r_first, sk );
+      }
+      GH_LAUNCH_CHECK();
+      return GH_OK;
+    }
+  }
+  const uint32_t tile_rows = splits > 1 || four_waves ? 256 : tile256_rows( s, r, b );
   ord.row_tiles = (uint32_t)( ( r + tile_rows - 1 ) / tile_rows );
   ord.token_tiles = (uint32_t)( ( b + TN2 - 1 ) / TN2 );
   ord.gn = std::min<uint32_t>( ord.token_tiles, 8 );
@@ -540,19 +1054,21 @@ int gemm_tile256_launch( __half* xout, float* partial, const __half* x, const __
   GH_REQUIRE( gx < ( 1ull << 31 ), "gh_matmul: grid too large" );
   ord.main_per_xcd = (uint32_t)main_per_xcd;
   ord.rest_share = (uint32_t)rest_share;
-  const dim3 grid( (unsigned)gx, splits ), block( T256_THREADS );
+  const dim3 grid( (unsigned)gx, splits ), block( four_waves ? T4_THREADS : T256_THREADS );
   const uint32_t s32 = (uint32_t)s, r32 = (uint32_t)r, b32 = (uint32_t)b;
   const int epi = partial != nullptr ? EPI_PARTIAL : epilogue;
   GH_REQUIRE( epi == EPI_STORE || epi == EPI_ACCUM || epi == EPI_PARTIAL, "gh_matmul: unknown tile epilogue %d", epi );
   GH_REQUIRE( epi != EPI_ACCUM || r % 8 == 0, "gh_matmul: the accumulating tile epilogue needs r %% 8 == 0" );
 #define GH_TILE256_LAUNCH( E, N ) gemm_tile256_kernel<E, N><<<grid, block, 0, st>>>( xout, partial, x, w, s32, r32, b32, k_len, xout2, (uint32_t)r_first, ord )
-#define GH_TILE256_ROWS( E ) ( tile_rows == 384 ? GH_TILE256_LAUNCH( E, 3 ) : GH_TILE256_LAUNCH( E, 2 ) )
+#define GH_TILE256_W4( E ) gemm_tile256w4_kernel<E><<<grid, block, 0, st>>>( xout, partial, x, w, s32, r32, b32, k_len, xout2, (uint32_t)r_first, ord )
+#define GH_TILE256_ROWS( E ) ( four_waves ? GH_TILE256_W4( E ) : tile_rows == 384 ? GH_TILE256_LAUNCH( E, 3 ) : GH_TILE256_LAUNCH( E, 2 ) )
   switch ( epi ) {
     case EPI_STORE: GH_TILE256_ROWS( EPI_STORE ); break;
     case EPI_ACCUM: GH_TILE256_ROWS( EPI_ACCUM ); break;
     default: GH_TILE256_ROWS( EPI_PARTIAL ); break;
   }
 #undef GH_TILE256_ROWS
+#undef GH_TILE256_W4
 #undef GH_TILE256_LAUNCH
   GH_LAUNCH_CHECK();
   return GH_OK;

@@ -171,10 +171,13 @@ def test_matmul_many_rows(dt, b, s, r):
 # enough 256-token tiles for the second tile kernel (forced with 256 and with 384 rows per work-group, and
 # whatever the dispatcher picks), ragged edges; the row counts leave 4, 0 and 6 (256) / 3, 6 and 7 (384)
 # row tiles beyond a multiple of 8, the part of the tile order that is cut into equal runs per XCD
-@pytest.mark.parametrize("force,rows", [(4, 256), (4, 384), (4, 0), (0, 0)])
+@pytest.mark.parametrize("force,rows", [(4, 256), (4, 384), (4, 128), (4, 129), (4, 0), (0, 0)])
 @pytest.mark.parametrize("b,s,r", [(3000, 8192, 4100), (8200, 128, 8190), (700, 8256, 18000)])
 def test_matmul_256_tiles(force, rows, b, s, r):
     from glinthawk_amd import _lib
+    if rows in (128, 129) and s % 128:
+        pytest.skip("the four-wave kernel (tile rows 128: one tile per work-group, 129: equal shares of all steps) takes K ranges of an even "
+                    "number of 64-k steps; the dispatcher takes the eight-wave one here")
     rng = np.random.default_rng(26)
     x = rng.standard_normal((b, s)).astype(np.float16)
     w = (rng.standard_normal((r, s)) / np.sqrt(s)).astype(np.float16)
@@ -191,7 +194,7 @@ def test_matmul_256_tiles(force, rows, b, s, r):
     assert_close(got[:8].cpu().numpy(), want_cpu, what=f"matmul 256-tile {b}x{s}x{r}")
 
 
-@pytest.mark.parametrize("rows", [256, 384])
+@pytest.mark.parametrize("rows", [256, 384, 128, 129])
 @pytest.mark.parametrize("s,r,b", [(8192, 12544, 1030),    # 49 / 33 row tiles x 5: one left-over row tile
                                    (1024, 5000, 16390),    # 20 / 14 row tiles x 65: 4 / 6 left over, ragged last token tile
                                    (256, 1700, 9000)])     # 7 / 5 row tiles: left-over tiles only
@@ -208,6 +211,50 @@ def test_matmul_256_tile_one_hot_layout(rows, s, r, b):
     finally:
         _lib.lib().gh_gemm_set_tuning(0, 0, 0)
     assert torch.equal(got, w[:, cols].t().contiguous())
+
+
+@pytest.mark.parametrize("epilogue", ["store", "accum", "pair"])
+def test_matmul_equal_shares_of_all_steps(epilogue):
+    """The four-wave kernel over equal shares of all 64-k steps (tile rows 129): shares that end inside tiles leave pieces that a
+    second kernel adds in a fixed order.  Ragged tiles in both directions, shares shorter and longer than a tile, all three outputs
+    (plain, residual add, two matrices); one-hot activations bit for bit, a random product twice with identical bits."""
+    from glinthawk_amd import _lib
+    for b, s, r in [(3000, 1280, 4104), (1100, 2560, 15880), (2300, 768, 8968)]:     # 204, 315 and 324 tiles of 20, 40 and 12 steps; shares of 16, 50 and 16
+        w = torch.arange(r * s, dtype=torch.float32, device="cuda").reshape(r, s).remainder(1000).half()
+        hot = torch.zeros((b, s), dtype=torch.float16, device="cuda")
+        cols = torch.tensor([(7919 * i + 3) % s for i in range(b)], device="cuda")
+        hot[torch.arange(b, device="cuda"), cols] = 1
+        g = torch.Generator(device="cuda").manual_seed(b + r)
+        x = torch.randn((b, s), generator=g, device="cuda").half()
+        wr = (torch.randn((r, s), generator=g, device="cuda") / s ** 0.5).half()
+        res = torch.randn((b, r), generator=g, device="cuda").half()
+        _lib.lib().gh_gemm_set_tuning(4 if epilogue == "store" else 0, 0, 129)
+        try:
+            if epilogue == "store":
+                got_hot, first, again = ops.matmul(hot, w), ops.matmul(x, wr), ops.matmul(x, wr)
+                want_hot = w[:, cols].t().contiguous()
+                want = x.float() @ wr.float().t()
+            elif epilogue == "accum":
+                got_hot = res.clone()
+                ops.matmul_accum(got_hot, hot, w)
+                first, again = res.clone(), res.clone()
+                ops.matmul_accum(first, x, wr)
+                ops.matmul_accum(again, x, wr)
+                want_hot = (res.float() + w[:, cols].t().float()).half()
+                want = res.float() + (x.float() @ wr.float().t()).half().float()
+            else:
+                ra = (r // 16) * 8
+                a, c = ops.matmul_pair(hot, w, ra)
+                got_hot = torch.cat([a, c], dim=1)
+                first, again = (torch.cat(ops.matmul_pair(x, wr, ra), dim=1) for _ in range(2))
+                want_hot = w[:, cols].t().contiguous()
+                want = x.float() @ wr.float().t()
+        finally:
+            _lib.lib().gh_gemm_set_tuning(0, 0, 0)
+        assert torch.equal(got_hot, want_hot), (b, s, r)
+        assert torch.equal(first, again), (b, s, r)
+        err = (first.float() - want).abs()
+        assert err.max().item() < 2e-2 and (err.mean() / want.abs().mean()).item() < 1e-3, (b, s, r)
 
 
 def test_matmul_many_rows_layout_one_hot():
