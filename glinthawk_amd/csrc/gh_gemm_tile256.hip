@@ -1015,7 +1015,8 @@ int gemm_tile256_launch( __half* xout, float* partial, const __half* x, const __
   const uint64_t cus = (uint64_t)cu_count();
   const uint64_t tiles256 = ( ( r + TM2 - 1 ) / TM2 ) * ( ( b + TN2 - 1 ) / TN2 );
   const uint64_t cost384 = s >= 7168 ? 143 : 136;
-  const bool four_pays = 2 * tiles256 >= 3 * cus && 94 * rounds_per_xcd( r, b, 256 ) <= cost384 * rounds_per_xcd( r, b, 384 );
+  // Most of a round is enough: 224 tiles (w1 and w3 of the 70B shape at 256 tokens) 221 against 254 us, at 512 tokens 428 against 484.
+  const bool four_pays = 4 * tiles256 >= 3 * cus && 94 * rounds_per_xcd( r, b, 256 ) <= cost384 * rounds_per_xcd( r, b, 384 );
   const bool four_waves = even_steps && ( g_tile_rows == 128 || g_tile_rows == 129 || ( g_tile_rows == 0 && splits == 1 && four_pays ) );
   GH_REQUIRE( ( g_tile_rows != 128 && g_tile_rows != 129 ) || even_steps, "gh_matmul: the four-wave tile kernel needs K ranges that are multiples of 128" );
   const int epi_sk = epilogue;
