@@ -57,6 +57,7 @@
 #include "gh_common.h"
 
 #include <algorithm>
+#include <cstdlib>
 
 namespace gh {
 
@@ -855,7 +856,13 @@ __global__ __launch_bounds__( T4_THREADS, 1 ) void gemm_w4_fixup_kernel( __half*
   w4_store_tile<EPI>( acc, o, ( tile / sk.token_tiles ) * TM2, ( tile % sk.token_tiles ) * TN2, st );
 }
 
-int g_tile_rows = 0; // 0: by tile256_rows(); 256 or 384: forced
+// GLINT_TILE_ROWS in the environment sets the start value (for the command-line profilers, which have no other way in)
+int tile_rows_default()
+{
+  const char* env = getenv( "GLINT_TILE_ROWS" );
+  return env != nullptr && *env != '\0' ? atoi( env ) : 0;
+}
+int g_tile_rows = tile_rows_default(); // 0: by the cost rules below; 256 or 384: the eight-wave kernel with that many rows; 128, 129: below
 // measurement hook (tile rows): 256 or 384 force the eight-wave kernel, 128 the four-wave one with one tile per work-group, 129 the
 // four-wave one over equal shares of all steps; 0: the four-wave kernel wherever it applies, equal shares where whole tiles fit badly
 

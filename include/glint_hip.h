@@ -152,8 +152,9 @@ int gh_argmax( uint32_t* out_host, uint32_t* out_dev, const void* v, uint64_t n,
 /* Operations::matmul<s,r> / untemplated_matmul  arch/amd64/common/ops.hh:74-93,212-271 :
  * xout(b, r) = sum_p w(r, p) * x(b, p); w row-major (r, s); fp32 accumulate */
 /* tuning hook: kernel 0 auto / 1 small tiled / 2 streaming (decode) / 3 128x128 tile / 4 256-token tile (many rows); the number of compute units the
- * streaming kernel's K split is balanced for (<= 0 keeps the current value; the default is the device's own count); weight rows per work-group of the
- * 256-token tile kernel: 256, 384, or 0 for the library's choice */
+ * streaming kernel's K split is balanced for (<= 0 keeps the current value; the default is the device's own count); the 256-token tile kernel: 256 or
+ * 384 weight rows per work-group of eight waves, 128 = four waves of 128 x 128 with one tile per work-group, 129 = four waves over equal shares of
+ * all K steps with the fix-up kernel, 0 = the library's choice (GLINT_TILE_ROWS in the environment sets the start value) */
 int gh_gemm_set_tuning( int kernel, int target_workgroups, int tile_rows );
 /* Opt-in: plain f16 products (gh_matmul, the two of gh_matmul_pair, the product inside gh_matmul_accum and gh_matmul_silu_gate where no
  * kernel of this library fuses it) of `rows` activation rows and more go to the vendor's GEMM library, as every product of the
