@@ -1,9 +1,10 @@
 // Plain products of many activation rows through the vendor's GEMM library (hipBLASLt), as the reference's GPU target sends
 // every product through its vendor library (cublasGemmEx, arch/cuda/common/ops.cuh:666-700: op(W) = T, op(x) = N,
 // m = r, n = b, k = s, fp32 compute type).  Same operands, same layout, same call here: xout(b, r) row-major is the
-// column-major C(m = r, n = b).  On this part the library's kernels reach 1.22-1.50 PFLOP/s at 3328 and more rows where the
-// tile kernels of this library reach 1.11-1.25, so the dispatcher hands it the products that are nothing but a product; what
-// is fused with an epilogue, split along K or shaped for decode stays on the kernels of this library.
+// column-major C(m = r, n = b).  An opt-in route (gh_gemm_set_library_rows, off by default): on this part the library's kernels
+// reach 1.22-1.50 PFLOP/s at 3328 and more rows where the tile kernels of this library reach 1.13-1.34, so a caller may hand it
+// the products that are nothing but a product; what is fused with an epilogue, split along K or shaped for decode stays on the
+// kernels of this library either way.
 //
 // The library is opened at the first such product, not linked: without it (or without an algorithm for a shape) the call is
 // declined and the dispatcher goes on to its own tile kernels.
