@@ -290,8 +290,11 @@ def decode_bench(workload, steps, warmup, fused=True, cpu=True, events=True, adv
         _lib.check(L.gh_attn_timing_read(C.byref(k_ms), C.byref(m_ms), C.byref(n)))
         L.gh_attn_timing_enable(0)
         launches = max(1, n.value)
+        # waves per work-group when the splits of a context are added up inside the attention kernel's work-groups: then there is
+        # no merge kernel, and what lies between the second and the third event is the events' own cost
+        join = ops.attn_decode_join_waves(batch, keys - 1, shape)
         res.update(ms_per_step_with_events=(t3 - t2) * 1e3 / steps, attn_kernel_ms=k_ms.value / launches,
-                   attn_merge_ms=m_ms.value / launches, attn_launches=int(n.value))
+                   attn_merge_ms=None if join else m_ms.value / launches, attn_launches=int(n.value), attn_split_join=join)
         # the attention op as it runs in production, its two kernels back to back: one event in front of the pair, one behind
         L.gh_attn_timing_enable(2)
         L.gh_attn_timing_reset()
@@ -389,7 +392,8 @@ def decode_line(workload, steps, warmup, attn_variant="auto", cpu=True):
                    "attn_variant": attn_variant},
         "attn_op_ms": round(attn_op_ms, 5),
         "attn_kernel_ms": round(g["attn_kernel_ms"], 5),
-        "attn_merge_ms": round(g["attn_merge_ms"], 5),
+        "attn_merge_ms": None if g["attn_merge_ms"] is None else round(g["attn_merge_ms"], 5),
+        "attn_split_join_waves": g["attn_split_join"],
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic, "traffic_source": traffic_note,
                      "kernel": "attn_decode (split-K fused decode attention)", "launches_timed": g["attn_launches"],
@@ -668,6 +672,9 @@ def main():
                     help="only the named workload: no concept-path run and no short runs of the other configurations")
     ap.add_argument("--attn-variant", default="auto", choices=["auto", "generic", "valu", "mfma"],
                     help="decode attention kernel the stage uses (measurement of the alternatives; auto = the library's choice)")
+    ap.add_argument("--attn-split-join", type=int, default=1, choices=[0, 1, 4, 8],
+                    help="measurement hook: how the splits of a context are added up in the decode attention (1: the library's choice; 0: always partial "
+                         "sums and the merge kernel; 4, 8: inside work-groups of that many waves where the plan has 2 or 4 splits)")
     ap.add_argument("--concept-path", action="store_true", help="time the named decode workload through the reference's op sequence only")
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="also run a plain D2D copy of this many MiB (reference point for profiler byte counters)")
@@ -693,6 +700,10 @@ def main():
         from glinthawk_amd import _lib, ops
         ops.init(0)
         _lib.check(_lib.lib().gh_gemm_set_library_rows(args.library_rows))
+    if args.attn_split_join != 1:
+        from glinthawk_amd import _lib, ops
+        ops.init(0)
+        _lib.check(_lib.lib().gh_attn_set_split_join(args.attn_split_join))
     if args.attn_variant != "auto":
         from glinthawk_amd import _lib, ops
         ops.init(0)

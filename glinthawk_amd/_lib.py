@@ -117,9 +117,11 @@ SIGNATURES = {
     "gh_attn_pv": (_i, [_vp, _vp, _vp, _u64, _vp, _shp, _i, _vp]),
     "gh_attn_pv_host": (_i, [_vp, _vp, _vp, _u64, _vp, _shp, _i, _vp]),
     "gh_attn_set_chunk": (_i, [_u32]),
+    "gh_attn_set_split_join": (_i, [_i]),
     "gh_attn_set_auto_variant": (_i, [_i]),
     "gh_attn_decode_workspace": (_u64, [_u64, _u32, _shp]),
     "gh_attn_decode_plan": (_i, [_u64, _u32, _shp, _i, _i, C.POINTER(_u32), C.POINTER(_u32), C.POINTER(_u64)]),
+    "gh_attn_decode_join_waves": (_u32, [_u64, _u32, _shp, _i, _i]),
     "gh_attn_decode": (_i, [_vp, _vp, _vp, _vp, _u64, _u32, _shp, _i, _vp, _u64, _i, _vp]),
     "gh_attn_decode_static_limit": (_u64, []),
     "gh_attn_decode_static": (_i, [_vp, _vp, _vp, _vp, _u64, _u32, _shp, _i, _i, _vp]),

@@ -38,6 +38,7 @@ static __device__ __align__( 256 ) float scratch[STATIC_SCRATCH_BYTES / sizeof( 
 float* g_static_scratch[MAX_DEVICES] = {};
 
 uint32_t g_chunk_override = 0;
+int g_split_join = 1; // 1: plans of 2 or 4 splits run on the kernels that add the splits up inside the work-group; 4, 8: with that many waves; 0: never
 int g_auto_variant = GH_ATTN_AUTO; // what GH_ATTN_AUTO resolves to when the shape allows it (gh_attn_set_auto_variant)
 
 struct Partials
@@ -209,6 +210,52 @@ __global__ __launch_bounds__( 256 ) void attn_merge_kernel( Partials part,
       xb[( (uint64_t)ctx * n_heads + head ) * head_size + d] = from_f32<T>( acc * ( 1.0f / l ) );
     }
   }
+}
+
+// =================================================================================================
+// joined splits: the splits of a (context, kv head) stream are the waves of ONE work-group, which adds them up itself
+//
+// With up to four splits per stream a work-group of four waves holds whole streams: wave = (stream of the work-group, split).
+// Every wave walks its token range as in the kernels above; then the waves leave their maxima, sums and accumulators in LDS, lane
+// for lane as they lie in the registers, and the wave of split 0 combines them in the order and with the arithmetic of
+// attn_merge_kernel (so the output is the same bit for bit) and stores the rounded result.  No partial sums in memory, no second
+// launch.
+// =================================================================================================
+struct JoinedJob
+{
+  const __half* base;
+  uint32_t ctx, h, split, t_begin, t_end;
+  uint32_t slot;     // which of the work-group's streams
+  uint32_t n_splits; // splits of this context that hold keys (0: nothing to do for the stream)
+  bool active;       // this wave has keys to walk
+};
+
+// splits = 2 or 4; a work-group is JOIN_WAVES (4 or 8) waves = (JOIN_WAVES / splits neighbouring kv heads) x splits, so that its waves
+// read pieces of the same cache rows that lie next to each other (with four waves on one head's four ranges a CU fetched 256-byte
+// pieces and the launch took 168-171 instead of 166 us at 64 contexts of 4096 keys).  Work-group b: head group b % n_groups,
+// context b / n_groups.
+template<uint32_t JOIN_WAVES>
+__device__ __forceinline__ JoinedJob joined_job( const __half* const* layer_rows, const uint32_t* pos, uint32_t n_kv_heads, uint32_t batch,
+                                                 uint32_t chunk, uint32_t splits, uint32_t seq_len )
+{
+  JoinedJob j;
+  const uint32_t wave = threadIdx.x >> 6;
+  const uint32_t heads_per_group = JOIN_WAVES / splits;
+  const uint32_t n_groups = ( n_kv_heads + heads_per_group - 1 ) / heads_per_group;
+  j.split = wave % splits;
+  j.slot = wave / splits;
+  const uint32_t ctx = blockIdx.x / n_groups;
+  const uint32_t h = ( blockIdx.x % n_groups ) * heads_per_group + j.slot;
+  const bool exists = ctx < batch && h < n_kv_heads;
+  j.ctx = exists ? ctx : 0;
+  j.h = exists ? h : 0;
+  j.base = exists ? layer_rows[j.ctx] : nullptr;
+  const uint32_t n_tok = j.base != nullptr ? min( min( pos[j.ctx] + 1, splits * chunk ), seq_len ) : 0;
+  j.n_splits = ( n_tok + chunk - 1 ) / chunk;
+  j.t_begin = j.split * chunk;
+  j.t_end = min( n_tok, j.t_begin + chunk );
+  j.active = j.t_begin < n_tok;
+  return j;
 }
 
 // =================================================================================================
@@ -409,6 +456,83 @@ __global__ __launch_bounds__( 256 ) void attn_decode_valu_kernel( const __half* 
         }
       }
     }
+  }
+}
+
+// the valu kernel with the splits of a stream joined inside the work-group (see joined_job)
+template<int G, uint32_t JOIN_WAVES>
+__global__ __launch_bounds__( 64 * JOIN_WAVES ) void attn_decode_valu_joined_kernel( const __half* __restrict__ q,
+                                                                         const __half* const* __restrict__ layer_rows,
+                                                                         const uint32_t* __restrict__ pos,
+                                                                         __half* __restrict__ xb,
+                                                                         uint32_t n_kv_heads,
+                                                                         uint32_t batch,
+                                                                         uint32_t chunk,
+                                                                         uint32_t splits,
+                                                                         uint32_t seq_len,
+                                                                         float scale_log2e )
+{
+  // per wave: what the 16 lanes of token row 0 hold -- 8 accumulators, the maximum and the sum of each of the G heads
+  __shared__ float s_join[JOIN_WAVES][10 * G][16];
+  const JoinedJob job = joined_job<JOIN_WAVES>( layer_rows, pos, n_kv_heads, batch, chunk, splits, seq_len );
+  const uint32_t wave = threadIdx.x >> 6;
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t c = lane & 15;
+  const uint32_t r = lane >> 4;
+  const uint32_t n_heads = n_kv_heads * G;
+
+  float m[G], l[G], acc[G][8];
+  if ( job.active ) {
+    valu_stream_range<G>( q, job.base, job.ctx, job.h, job.t_begin, job.t_end, job.split, n_kv_heads, scale_log2e, m, l, acc );
+    if ( job.split != 0 && r == 0 ) {
+#pragma unroll
+      for ( int g = 0; g < G; g++ ) {
+#pragma unroll
+        for ( int e = 0; e < 8; e++ ) {
+          s_join[wave][10 * g + e][c] = acc[g][e];
+        }
+        s_join[wave][10 * g + 8][c] = m[g];
+        s_join[wave][10 * g + 9][c] = l[g];
+      }
+    }
+  }
+  __syncthreads(); // reached by every wave of the work-group, with or without keys
+  if ( job.split != 0 || !job.active || r != 0 ) {
+    return; // split 0 holds keys whenever any split of the stream does
+  }
+#pragma unroll
+  for ( int g = 0; g < G; g++ ) {
+    float mm = m[g];
+    for ( uint32_t u = 1; u < job.n_splits; u++ ) {
+      mm = fmaxf( mm, s_join[wave + u][10 * g + 8][c] );
+    }
+    const float w0 = fast_exp2( m[g] - mm );
+    float lsum = l[g] * w0;
+    float out[8];
+#pragma unroll
+    for ( int e = 0; e < 8; e++ ) {
+      out[e] = acc[g][e] * w0;
+    }
+    for ( uint32_t u = 1; u < job.n_splits; u++ ) {
+      const float wu = fast_exp2( s_join[wave + u][10 * g + 8][c] - mm );
+      lsum = __builtin_fmaf( s_join[wave + u][10 * g + 9][c], wu, lsum );
+#pragma unroll
+      for ( int e = 0; e < 8; e++ ) {
+        out[e] = __builtin_fmaf( s_join[wave + u][10 * g + e][c], wu, out[e] );
+      }
+    }
+    const float inv = 1.0f / lsum;
+    union
+    {
+      uint4 raw;
+      __half h[8];
+    } o;
+#pragma unroll
+    for ( int e = 0; e < 8; e++ ) {
+      o.h[e] = __float2half_rn( out[e] * inv );
+    }
+    const uint64_t head = (uint64_t)job.ctx * n_heads + (uint64_t)job.h * G + g;
+    *reinterpret_cast<uint4*>( xb + head * HS + 8 * c ) = o.raw;
   }
 }
 
@@ -645,6 +769,98 @@ __global__ __launch_bounds__( 256 ) void attn_decode_mfma_kernel( const __half* 
         }
       }
     }
+  }
+}
+
+// the mfma kernel with the splits of a stream joined inside the work-group (see joined_job)
+template<int G, uint32_t JOIN_WAVES>
+__global__ __launch_bounds__( 64 * JOIN_WAVES ) void attn_decode_mfma_joined_kernel( const __half* __restrict__ q,
+                                                                         const __half* const* __restrict__ layer_rows,
+                                                                         const uint32_t* __restrict__ pos,
+                                                                         __half* __restrict__ xb,
+                                                                         uint32_t n_kv_heads,
+                                                                         uint32_t batch,
+                                                                         uint32_t chunk,
+                                                                         uint32_t splits,
+                                                                         uint32_t seq_len,
+                                                                         float scale_log2e )
+{
+  __shared__ uint4 s_k[JOIN_WAVES][16 * 16]; // per wave: 16 tokens x 16 chunks of 16 bytes
+  // per wave and lane: its 32 accumulators, then the maxima and the sums of its 4 heads; only the lanes whose heads exist (the first 4 G)
+  constexpr int JOIN_LANES = 4 * G < 16 ? 16 : 4 * G;
+  __shared__ float s_join[JOIN_WAVES][40][JOIN_LANES];
+  const JoinedJob job = joined_job<JOIN_WAVES>( layer_rows, pos, n_kv_heads, batch, chunk, splits, seq_len );
+  const uint32_t wave = threadIdx.x >> 6;
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t c = lane & 15;
+  const uint32_t g4 = lane >> 4;
+  const uint32_t n_heads = n_kv_heads * G;
+
+  f32x4 acc[8];
+  float mh[4], lh[4]; // of heads 4*g4 + i, to which this lane's accumulators acc[.][i] belong
+  if ( job.active ) {
+    float m, l;
+    mfma_stream_range<G>( q, job.base, job.ctx, job.h, job.t_begin, job.t_end, job.split, n_kv_heads, scale_log2e, s_k[wave], acc, m, l );
+    l += __shfl_xor( l, 16, WAVE );
+    l += __shfl_xor( l, 32, WAVE );
+#pragma unroll
+    for ( int i = 0; i < 4; i++ ) {
+      mh[i] = __shfl( m, (int)( 4 * g4 + i ), WAVE );
+      lh[i] = __shfl( l, (int)( 4 * g4 + i ), WAVE );
+    }
+    if ( job.split != 0 && 4 * g4 < G ) {
+#pragma unroll
+      for ( int i = 0; i < 4; i++ ) {
+#pragma unroll
+        for ( int nn = 0; nn < 8; nn++ ) {
+          s_join[wave][8 * i + nn][lane] = acc[nn][i];
+        }
+        s_join[wave][32 + i][lane] = mh[i];
+        s_join[wave][36 + i][lane] = lh[i];
+      }
+    }
+  }
+  __syncthreads(); // reached by every wave of the work-group, with or without keys
+  if ( job.split != 0 || !job.active ) {
+    return; // split 0 holds keys whenever any split of the stream does
+  }
+#pragma unroll
+  for ( int i = 0; i < 4; i++ ) {
+    const uint32_t hd = 4 * g4 + i;
+    if ( hd >= G ) {
+      continue;
+    }
+    float mm = mh[i];
+    for ( uint32_t u = 1; u < job.n_splits; u++ ) {
+      mm = fmaxf( mm, s_join[wave + u][32 + i][lane] );
+    }
+    const float w0 = fast_exp2( mh[i] - mm );
+    float lsum = lh[i] * w0;
+    float out[8];
+#pragma unroll
+    for ( int nn = 0; nn < 8; nn++ ) {
+      out[nn] = acc[nn][i] * w0;
+    }
+    for ( uint32_t u = 1; u < job.n_splits; u++ ) {
+      const float wu = fast_exp2( s_join[wave + u][32 + i][lane] - mm );
+      lsum = __builtin_fmaf( s_join[wave + u][36 + i][lane], wu, lsum );
+#pragma unroll
+      for ( int nn = 0; nn < 8; nn++ ) {
+        out[nn] = __builtin_fmaf( s_join[wave + u][8 * i + nn][lane], wu, out[nn] );
+      }
+    }
+    const float inv = 1.0f / lsum;
+    union
+    {
+      uint4 raw;
+      __half h[8];
+    } o;
+#pragma unroll
+    for ( int nn = 0; nn < 8; nn++ ) {
+      o.h[nn] = __float2half_rn( out[nn] * inv );
+    }
+    const uint64_t head = (uint64_t)job.ctx * n_heads + (uint64_t)job.h * G + hd;
+    *reinterpret_cast<uint4*>( xb + head * HS + 8 * c ) = o.raw;
   }
 }
 
@@ -919,7 +1135,55 @@ struct Plan
   uint32_t chunk;       // tokens per split
   uint32_t max_splits;  // splits of the longest context
   uint32_t split_bound; // upper bound of max_splits for any shorter longest context (sizes the workspace)
+  uint32_t join;        // > 0: the splits of a stream are waves of one work-group of this many waves, which adds them up itself
 };
+
+// The splits of a (context, kv head) stream as waves of one work-group (no partial sums in memory, no merge kernel), for the f16
+// head-128 kernels: how many splits and how many waves per work-group, by the number of streams per CU.  A work-group of W waves
+// holds W / splits neighbouring kv heads (its waves then read neighbouring pieces of the same cache rows: with one head per
+// work-group of 8 waves the walk itself is slower than what the merge kernel costs), and what counts beside that is how evenly the
+// work-groups fill the CUs: every range below ends where its work-groups would no longer fit the CUs in one go.  Measured on MI355X
+// (256 CUs), fused op in us, partial sums + merge kernel / the choice below.  70B shape (8 kv heads, MFMA kernel), contexts x 4096 keys:
+//   24: 81 / 74 (4 splits, 4 waves)   32: 87 / 81   40: 123 / 109 (4, 8)   48: 142 / 123   64: 164 / 155   66: 202 / 180 (2, 8)
+//   80: 224 / 196   104: 282 / 250   112: 293 / 266 (2, 4)   128: 362 / 308   144: 408 / 386 (4, 8)   160: 457 / 397   250: 716 / 605
+// 7B shape (32 kv heads with one query head each: the VALU kernel), contexts x 2048 keys:
+//   10: 62 / 56 (4, 8)   16: 85 / 80   17: 104.5 / 94 (2, 8)   26: 144 / 130   27: 146 / 133 (2, 4)   32: 167 / 157
+// and 32 x 1024 keys: 85.5 / 80.2.  13B shape (40 heads), x 2048 keys: 8: 62.4 / 60.8   12: 85 / 77   16: 108.5 / 109.6   21: 141 / 137.
+// This kernel with more than four streams per CU or with at most one: no joined choice ahead of the merge route (13B, 32
+// contexts: 204 / 212; 7B, 8 contexts: 44.5 / 45.8).
+struct JoinChoice
+{
+  uint32_t splits, waves; // waves == 0: none
+};
+JoinChoice join_choice( uint64_t streams, int variant, uint32_t n_tok )
+{
+  const uint64_t cus = (uint64_t)cu_count();
+  const uint64_t x8 = 8 * streams; // streams per CU in eighths
+  JoinChoice c { 0, 0 };
+  if ( x8 < 6 * cus ) {
+    return c;
+  } else if ( x8 <= 8 * cus ) {
+    c = variant == GH_ATTN_MFMA ? JoinChoice { 4, 4 } : c; // one work-group of 4 waves per stream, at most one per CU
+  } else if ( x8 < 10 * cus ) {
+    return c; // work-groups of 8 waves would reach little more than half of the CUs (-9 ... +6 %)
+  } else if ( x8 <= 16 * cus ) {
+    c = JoinChoice { 4, 8 }; // one work-group of 8 waves per two streams, at most one per CU
+  } else if ( x8 <= 26 * cus ) {
+    c = JoinChoice { 2, 8 }; // ... per four streams
+  } else if ( x8 <= 32 * cus ) {
+    c = JoinChoice { 2, 4 }; // two work-groups of 4 waves per CU
+  } else if ( x8 < 64 * cus ) {
+    c = variant == GH_ATTN_MFMA ? JoinChoice { 4, 8 } : c; // several rounds of work-groups
+  }
+  // splits are never shorter than 256 tokens
+  while ( c.waves != 0 && c.splits > 1 && (uint64_t)n_tok < 256ull * c.splits ) {
+    c.splits /= 2;
+  }
+  if ( c.splits < 2 ) {
+    c = JoinChoice { 0, 0 };
+  }
+  return c;
+}
 
 bool fast_ok( const gh_shape* s, gh_dtype dt ) { return dt == GH_F16 && s->head_size == HS; }
 bool valu_gqa_ok( uint32_t g ) { return g == 1 || g == 2 || g == 4 || g == 8; }
@@ -928,6 +1192,7 @@ bool mfma_gqa_ok( uint32_t g ) { return g == 2 || g == 4 || g == 8 || g == 16; }
 Plan make_plan( uint64_t batch, uint32_t max_pos, const gh_shape* s, gh_dtype dt, int variant )
 {
   Plan p;
+  p.join = 0;
   p.variant = variant;
   if ( variant == GH_ATTN_AUTO && g_auto_variant == GH_ATTN_GENERIC ) {
     p.variant = GH_ATTN_GENERIC;
@@ -963,6 +1228,14 @@ Plan make_plan( uint64_t batch, uint32_t max_pos, const gh_shape* s, gh_dtype dt
       chunk = 256;
     }
     split_cap = std::min<uint64_t>( splits, ( n_tok + 255 ) / 256 );
+    // the joined route where it pays: never more splits than the rule above gives, so the workspace bound holds either way
+    if ( g_split_join != 0 && p.variant != GH_ATTN_GENERIC ) {
+      const JoinChoice c = join_choice( streams, p.variant, n_tok );
+      if ( c.waves != 0 && c.splits <= splits ) {
+        chunk = ( n_tok + c.splits - 1 ) / c.splits;
+        p.join = g_split_join == 4 || g_split_join == 8 ? (uint32_t)g_split_join : c.waves;
+      }
+    }
   }
   chunk = ( chunk + 15 ) / 16 * 16;
   p.chunk = chunk;
@@ -971,6 +1244,13 @@ Plan make_plan( uint64_t batch, uint32_t max_pos, const gh_shape* s, gh_dtype dt
     p.max_splits = 1;
   }
   p.split_bound = (uint32_t)std::max<uint64_t>( p.max_splits, split_cap );
+  // a split length given from outside (tests, measurements), or a forced work-group size: joined whenever the plan has 2 or 4 splits
+  if ( g_split_join != 0 && p.variant != GH_ATTN_GENERIC && ( g_chunk_override != 0 || g_split_join == 4 || g_split_join == 8 ) ) {
+    p.join = g_split_join == 4 || g_split_join == 8 ? (uint32_t)g_split_join : 8u;
+  }
+  if ( !( p.max_splits == 2 || p.max_splits == 4 ) || p.max_splits > p.join ) {
+    p.join = 0;
+  }
   return p;
 }
 
@@ -993,6 +1273,32 @@ void launch_mfma( dim3 grid, hipStream_t st, const void* q, const void* const* r
 {
   attn_decode_mfma_kernel<G><<<grid, 256, 0, st>>>( static_cast<const __half*>( q ), reinterpret_cast<const __half* const*>( rows ), pos, part,
                                                    static_cast<__half*>( xb ), s->n_kv_heads, p.chunk, p.max_splits, s->seq_len, scale );
+}
+
+template<int G>
+void launch_valu_joined( uint32_t waves, dim3 grid, hipStream_t st, const void* q, const void* const* rows, const uint32_t* pos, void* xb, const gh_shape* s,
+                         const Plan& p, uint32_t batch, float scale )
+{
+  if ( waves == 4 ) {
+    attn_decode_valu_joined_kernel<G, 4><<<grid, 256, 0, st>>>( static_cast<const __half*>( q ), reinterpret_cast<const __half* const*>( rows ), pos,
+                                                               static_cast<__half*>( xb ), s->n_kv_heads, batch, p.chunk, p.max_splits, s->seq_len, scale );
+  } else {
+    attn_decode_valu_joined_kernel<G, 8><<<grid, 512, 0, st>>>( static_cast<const __half*>( q ), reinterpret_cast<const __half* const*>( rows ), pos,
+                                                               static_cast<__half*>( xb ), s->n_kv_heads, batch, p.chunk, p.max_splits, s->seq_len, scale );
+  }
+}
+
+template<int G>
+void launch_mfma_joined( uint32_t waves, dim3 grid, hipStream_t st, const void* q, const void* const* rows, const uint32_t* pos, void* xb, const gh_shape* s,
+                         const Plan& p, uint32_t batch, float scale )
+{
+  if ( waves == 4 ) {
+    attn_decode_mfma_joined_kernel<G, 4><<<grid, 256, 0, st>>>( static_cast<const __half*>( q ), reinterpret_cast<const __half* const*>( rows ), pos,
+                                                               static_cast<__half*>( xb ), s->n_kv_heads, batch, p.chunk, p.max_splits, s->seq_len, scale );
+  } else {
+    attn_decode_mfma_joined_kernel<G, 8><<<grid, 512, 0, st>>>( static_cast<const __half*>( q ), reinterpret_cast<const __half* const*>( rows ), pos,
+                                                               static_cast<__half*>( xb ), s->n_kv_heads, batch, p.chunk, p.max_splits, s->seq_len, scale );
+  }
 }
 
 // where the plan and the partials of the balanced variant lie in its workspace
@@ -1081,6 +1387,13 @@ int gh_attn_set_auto_variant( int variant )
   return GH_OK;
 }
 
+int gh_attn_set_split_join( int on )
+{
+  GH_REQUIRE( on == 0 || on == 1 || on == 4 || on == 8, "gh_attn_set_split_join: %d is not 0, 1, 4 or 8", on );
+  g_split_join = on;
+  return GH_OK;
+}
+
 int gh_attn_set_chunk( uint32_t tokens_per_split )
 {
   g_chunk_override = tokens_per_split;
@@ -1117,9 +1430,17 @@ int gh_attn_decode_plan( uint64_t batch, uint32_t max_pos, const gh_shape* shape
     *max_splits = plan.max_splits;
   }
   if ( partial_bytes ) {
-    *partial_bytes = plan.max_splits > 1 ? partial_floats( batch, shape, plan.max_splits ) * sizeof( float ) : 0;
+    *partial_bytes = plan.max_splits > 1 && plan.join == 0 ? partial_floats( batch, shape, plan.max_splits ) * sizeof( float ) : 0;
   }
   return GH_OK;
+}
+
+uint32_t gh_attn_decode_join_waves( uint64_t batch, uint32_t max_pos, const gh_shape* shape, gh_dtype dt, int variant )
+{
+  if ( shape == nullptr || batch == 0 || variant < GH_ATTN_AUTO || variant > GH_ATTN_MFMA ) {
+    return 0;
+  }
+  return make_plan( batch, max_pos, shape, dt, variant ).join;
 }
 
 // Shared by gh_attn_decode (partials in the caller's workspace, kernel timer on request) and
@@ -1150,8 +1471,10 @@ static int attn_decode_run( const char* who, const void* q, const void* const* l
   }
 
   const Plan plan = make_plan( batch, max_pos, shape, dt, variant );
+  const uint32_t join = plan.join; // > 0: no partial sums in memory, no merge kernel
+  const bool joined = join > 0;
   Partials part { nullptr, nullptr };
-  if ( plan.max_splits > 1 ) {
+  if ( plan.max_splits > 1 && !joined ) {
     const uint64_t need = partial_floats( batch, shape, plan.max_splits ) * sizeof( float );
     GH_REQUIRE( workspace != nullptr, "%s: workspace required (%llu bytes)", who, (unsigned long long)need );
     if ( workspace_bytes < need ) {
@@ -1183,6 +1506,26 @@ static int attn_decode_run( const char* who, const void* q, const void* const* l
                                                              pos_dev, part, static_cast<float*>( xb ), shape->n_kv_heads, shape->gqa_size,
                                                              shape->head_size, plan.chunk, plan.max_splits, scale );
     }
+  } else if ( joined ) {
+    const uint32_t heads_per_group = join / plan.max_splits;
+    const uint64_t n_blocks = batch * ( ( shape->n_kv_heads + heads_per_group - 1 ) / heads_per_group );
+    GH_REQUIRE( n_blocks <= 0x7fffffffull, "gh_attn_decode: grid too large" );
+    const dim3 grid( (unsigned)n_blocks );
+    if ( plan.variant == GH_ATTN_VALU ) {
+      switch ( shape->gqa_size ) {
+        case 1: launch_valu_joined<1>( join, grid, st, q, layer_rows_dev, pos_dev, xb, shape, plan, (uint32_t)batch, scale ); break;
+        case 2: launch_valu_joined<2>( join, grid, st, q, layer_rows_dev, pos_dev, xb, shape, plan, (uint32_t)batch, scale ); break;
+        case 4: launch_valu_joined<4>( join, grid, st, q, layer_rows_dev, pos_dev, xb, shape, plan, (uint32_t)batch, scale ); break;
+        default: launch_valu_joined<8>( join, grid, st, q, layer_rows_dev, pos_dev, xb, shape, plan, (uint32_t)batch, scale ); break;
+      }
+    } else {
+      switch ( shape->gqa_size ) {
+        case 2: launch_mfma_joined<2>( join, grid, st, q, layer_rows_dev, pos_dev, xb, shape, plan, (uint32_t)batch, scale ); break;
+        case 4: launch_mfma_joined<4>( join, grid, st, q, layer_rows_dev, pos_dev, xb, shape, plan, (uint32_t)batch, scale ); break;
+        case 8: launch_mfma_joined<8>( join, grid, st, q, layer_rows_dev, pos_dev, xb, shape, plan, (uint32_t)batch, scale ); break;
+        default: launch_mfma_joined<16>( join, grid, st, q, layer_rows_dev, pos_dev, xb, shape, plan, (uint32_t)batch, scale ); break;
+      }
+    }
   } else {
     const uint64_t n_blocks = batch * plan.max_splits * ( ( shape->n_kv_heads + 3 ) / 4 );
     GH_REQUIRE( n_blocks <= 0x7fffffffull, "gh_attn_decode: grid too large" );
@@ -1210,7 +1553,7 @@ static int attn_decode_run( const char* who, const void* q, const void* const* l
     }
   }
 
-  if ( plan.max_splits > 1 ) {
+  if ( plan.max_splits > 1 && !joined ) {
     const dim3 grid( shape->n_heads, (unsigned)batch );
     const unsigned threads = shape->head_size <= 64 ? 64 : ( shape->head_size <= 128 ? 128 : 256 );
     if ( dt == GH_F16 ) {

@@ -221,6 +221,12 @@ def attn_decode_workspace(batch: int, max_pos: int, shape: Shape) -> int:
     return int(lib().gh_attn_decode_workspace(batch, max_pos, C.byref(s)))
 
 
+def attn_decode_join_waves(batch: int, max_pos: int, shape: Shape, dt: int = GH_F16, variant: int = GH_ATTN_AUTO) -> int:
+    """Waves per work-group if the call's splits are added up inside the work-groups, 0 if partial sums and the merge kernel are used."""
+    s = shape.c()
+    return int(lib().gh_attn_decode_join_waves(batch, max_pos, C.byref(s), dt, variant))
+
+
 def attn_decode(q, layer_rows: torch.Tensor, pos: torch.Tensor, xb, max_pos: int, shape: Shape,
                 workspace: Optional[torch.Tensor] = None, variant: int = GH_ATTN_AUTO) -> None:
     s = shape.c()
@@ -285,6 +291,11 @@ def attn_prefill(q, layer_rows: torch.Tensor, start_pos: torch.Tensor, xb, n_tok
 
 def attn_set_chunk(tokens: int) -> None:
     check(lib().gh_attn_set_chunk(tokens), "gh_attn_set_chunk")
+
+
+def attn_set_split_join(mode) -> None:
+    """0 / False: partial sums + merge kernel; 1 / True: the library's choice; 4, 8: joined with that many waves per work-group."""
+    check(lib().gh_attn_set_split_join(int(mode)), "gh_attn_set_split_join")
 
 
 def pinned_empty(shape, dtype):

@@ -248,14 +248,23 @@ typedef enum gh_attn_variant
 
 /* tokens per split of the fused kernel; 0 (default) lets the library choose from the batch shape */
 int gh_attn_set_chunk( uint32_t tokens_per_split );
+/* measurement / test hook.  1 (default): a plan of 2 or 4 splits on the f16 head-128 kernels whose waves are all resident at once makes the splits of a
+ * (context, kv head) stream waves of one work-group, which adds them up itself: no partial sums in the workspace, no merge kernel, results within one
+ * rounding of the two-kernel route.  4, 8: that route with work-groups of 4 or 8 waves for every plan of 2 or 4 splits.  0: every split plan writes
+ * partial sums and runs the merge kernel. */
+int gh_attn_set_split_join( int on );
 /* measurement hook: which kernel GH_ATTN_AUTO picks where the shape permits it (GH_ATTN_AUTO restores the library's choice) */
 int gh_attn_set_auto_variant( int variant );
 /* bytes that serve every call with at most `batch` rows and positions up to `max_pos` (a smaller batch is cut into more splits per context, so the
  * largest need over all batch sizes in [1, batch] is returned) */
 uint64_t gh_attn_decode_workspace( uint64_t batch, uint32_t max_pos, const gh_shape* shape );
-/* host-only query: how gh_attn_decode would cut this call (tokens per split, splits of the longest context) and the workspace bytes it would use */
+/* host-only query: how gh_attn_decode would cut this call (tokens per split, splits of the longest context) and the workspace bytes it would use
+ * (0 for a plan whose splits are added up inside the work-groups) */
 int gh_attn_decode_plan( uint64_t batch, uint32_t max_pos, const gh_shape* shape, gh_dtype dt, int variant, uint32_t* tokens_per_split, uint32_t* max_splits,
                          uint64_t* partial_bytes );
+/* host-only query: waves per work-group if gh_attn_decode would add the splits of this call up inside its work-groups (no partial sums, no merge
+ * kernel: see gh_attn_set_split_join), 0 if it would write partial sums to the workspace and run the merge kernel, or needs no split at all */
+uint32_t gh_attn_decode_join_waves( uint64_t batch, uint32_t max_pos, const gh_shape* shape, gh_dtype dt, int variant );
 int gh_attn_decode( const void* q, const void* const* layer_rows_dev, const uint32_t* pos_dev, void* xb, uint64_t batch,
                     uint32_t max_pos, const gh_shape* shape, gh_dtype dt, void* workspace, uint64_t workspace_bytes,
                     int variant, gh_stream stream );

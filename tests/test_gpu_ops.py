@@ -2,12 +2,14 @@
 
 Bit-exact: KV append.  Everything floating point: the north-star tolerance (2e-2 max-abs, 1e-3
 mean-relative) against the oracle's fp32 path, and tighter self-consistency bounds where stated."""
+import ctypes as C
+
 import numpy as np
 import pytest
 import torch
 
 import oracle as O
-from glinthawk_amd import Shape, ops
+from glinthawk_amd import Shape, _lib, ops
 from glinthawk_amd._lib import GH_ATTN_AUTO, GH_ATTN_GENERIC, GH_ATTN_MFMA, GH_ATTN_VALU, GlintError
 from helpers import half_ulp_diff, Arena, assert_close, errors, oracle_cfg
 
@@ -648,7 +650,7 @@ def test_unfused_attention_ops_streaming_kernels(name, shape, pos, host_tables):
 
 
 # ------------------------------------------------------------------ fused decode attention
-def run_fused_case(shape, dt, variant, pos, present, chunk, seed=13, host_tables=False, std=1.0, balanced=False):
+def run_fused_case(shape, dt, variant, pos, present, chunk, seed=13, host_tables=False, std=1.0, balanced=False, join=1):
     batch = len(pos)
     cfg = oracle_cfg(shape)
     arena = Arena(shape, batch, tdt(dt), seed=seed, std=std)
@@ -658,6 +660,7 @@ def run_fused_case(shape, dt, variant, pos, present, chunk, seed=13, host_tables
     dq = torch.from_numpy(q).cuda()
     dxb = torch.full((batch, shape.dim), 5.0, dtype=tdt(dt), device="cuda")
     ops.attn_set_chunk(chunk)
+    ops.attn_set_split_join(join)
     try:
         if balanced:
             max_pos = max([p for p, ok in zip(pos, present) if ok] + [0])
@@ -674,6 +677,7 @@ def run_fused_case(shape, dt, variant, pos, present, chunk, seed=13, host_tables
         got = dxb.cpu().numpy()
     finally:
         ops.attn_set_chunk(0)
+        ops.attn_set_split_join(1)
 
     # oracle: the reference's fp32 CPU path on the same (exactly converted) inputs
     q32 = q.astype(np.float32)
@@ -719,6 +723,41 @@ def test_fused_mfma(shape, chunk):
     pos = [p for p in RAGGED if p < shape.seq_len] + [shape.seq_len - 1, 2]
     present = [True] * (len(pos) - 1) + [False]
     run_fused_case(shape, "f16", GH_ATTN_MFMA, pos, present, chunk)
+
+
+@pytest.mark.parametrize("waves", [4, 8])
+@pytest.mark.parametrize("splits", [2, 4])
+@pytest.mark.parametrize("variant,shape", [(GH_ATTN_VALU, MHA128), (GH_ATTN_VALU, MHA128_ODD), (GH_ATTN_VALU, GQA2), (GH_ATTN_VALU, GQA8),
+                                           (GH_ATTN_MFMA, GQA2), (GH_ATTN_MFMA, GQA4), (GH_ATTN_MFMA, GQA8), (GH_ATTN_MFMA, GQA16)],
+                         ids=["valu-mha", "valu-mha6", "valu-gqa2", "valu-gqa8", "mfma-gqa2", "mfma-gqa4", "mfma-gqa8", "mfma-gqa16"])
+def test_fused_splits_joined_inside_the_work_group(variant, shape, splits, waves):
+    """Plans of 2 or 4 splits: the splits of a (context, kv head) stream are waves of one work-group, which adds them up itself, in
+    work-groups of 4 or of 8 waves.  Contexts that reach into every split, into some, into the first only; an empty context in the
+    middle; head counts that do not fill the last work-group.  Against the oracle, and against the route with partial sums and the
+    merge kernel, which does the same arithmetic in another kernel (contraction may differ: one rounding)."""
+    top = shape.seq_len - 1
+    chunk = -(-(-(-shape.seq_len // splits)) // 16) * 16
+    pos = [top, 0, chunk - 1, chunk, chunk + 1, top - 1, 5, 2 * chunk - 1 if splits > 2 else 17, top, 3 * chunk + 1 if splits > 2 else chunk // 2, 40]
+    present = [True] * len(pos)
+    present[4] = False
+    ops.attn_set_chunk(chunk)
+    ops.attn_set_split_join(waves)
+    try:
+        c_shape, got_chunk, got_splits, need = shape.c(), C.c_uint32(0), C.c_uint32(0), C.c_uint64(1)
+        _lib.check(_lib.lib().gh_attn_decode_plan(len(pos), top, C.byref(c_shape), _lib.GH_F16, variant, C.byref(got_chunk), C.byref(got_splits), C.byref(need)))
+        assert (got_chunk.value, got_splits.value, need.value) == (chunk, splits, 0)        # no partial sums in the workspace
+        assert ops.attn_decode_join_waves(len(pos), top, shape, variant=variant) == waves
+        ops.attn_set_split_join(0)
+        assert ops.attn_decode_join_waves(len(pos), top, shape, variant=variant) == 0
+    finally:
+        ops.attn_set_chunk(0)
+        ops.attn_set_split_join(1)
+    joined, _ = run_fused_case(shape, "f16", variant, pos, present, chunk, seed=71, join=waves)
+    merged, _ = run_fused_case(shape, "f16", variant, pos, present, chunk, seed=71, join=0)
+    live = [i for i, ok in enumerate(present) if ok]
+    assert half_ulp_diff(joined[live], merged[live])[0] <= 1
+    # large scores: the splits' maxima lie far apart
+    run_fused_case(shape, "f16", variant, pos, present, chunk, seed=72, std=5.0, join=waves)
 
 
 @pytest.mark.parametrize("shape", [TINY, MHA128, GQA8], ids=["tiny", "mha", "gqa8"])

@@ -89,22 +89,33 @@ def test_static_scratch_entry_point_refuses_what_does_not_fit():
     ops.init(0)
     wide = Shape(dim=4096, n_layers=1, n_heads=32, n_kv_heads=2, hidden_dim=64, seq_len=1024)     # gqa 16
     batch = 300
-    splits, need = plan_bytes(batch, 1023, wide)
-    assert need > 16 << 20
     q = torch.zeros((batch, wide.dim), dtype=torch.float16, device="cuda")
     xb = torch.full((batch, wide.dim), 3.0, dtype=torch.float16, device="cuda")
     cache = torch.zeros((wide.seq_len, 2 * wide.kv_dim), dtype=torch.float16, device="cuda")      # every context reads the same rows
     rows = ops.row_table([cache.data_ptr()] * batch)
     pos = torch.full((batch,), 1023, dtype=torch.int32, device="cuda")
-    rc = decode_static(q, rows, pos, xb, 1023, wide)
-    assert rc == -5                                                                               # GH_ERR_WORKSPACE
-    assert b"gh_attn_decode_static" in _lib.lib().gh_last_error() and b"available" in _lib.lib().gh_last_error()
+    # As the library would run this call its splits are added up inside the work-groups: nothing goes into the array.  With
+    # that route switched off the plan's partial sums exceed it.
+    assert plan_bytes(batch, 1023, wide)[1] == 0 and ops.attn_decode_join_waves(batch, 1023, wide) > 0
+    ops.attn_set_split_join(0)
+    try:
+        splits, need = plan_bytes(batch, 1023, wide)
+        assert need > 16 << 20
+        rc = decode_static(q, rows, pos, xb, 1023, wide)
+        assert rc == -5                                                                           # GH_ERR_WORKSPACE
+        assert b"gh_attn_decode_static" in _lib.lib().gh_last_error() and b"available" in _lib.lib().gh_last_error()
+        ops.sync()
+        assert float(xb.float().min()) == 3.0                                                     # nothing was launched
+        # the same call through the workspace entry point is fine
+        ops.attn_decode(q, rows, pos, xb, 1023, wide)
+        ops.sync()
+        assert float(xb.float().abs().max()) == 0.0                                               # all-zero V rows
+    finally:
+        ops.attn_set_split_join(1)
+    xb.fill_(3.0)
+    assert decode_static(q, rows, pos, xb, 1023, wide) == 0
     ops.sync()
-    assert float(xb.float().min()) == 3.0                                                         # nothing was launched
-    # the same call through the workspace entry point is fine
-    ops.attn_decode(q, rows, pos, xb, 1023, wide)
-    ops.sync()
-    assert float(xb.float().abs().max()) == 0.0                                                   # all-zero V rows
+    assert float(xb.float().abs().max()) == 0.0
 
 
 def test_static_scratch_entry_point_allocates_nothing():
