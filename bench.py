@@ -292,7 +292,8 @@ def decode_bench(workload, steps, warmup, fused=True, cpu=True, events=True, adv
         launches = max(1, n.value)
         # waves per work-group when the splits of a context are added up inside the attention kernel's work-groups: then there is
         # no merge kernel, and what lies between the second and the third event is the events' own cost
-        join = ops.attn_decode_join_waves(batch, keys - 1, shape)
+        from glinthawk_amd import Shape
+        join = ops.attn_decode_join_waves(batch, keys - 1, Shape(**{k: shape[k] for k in ("dim", "n_layers", "n_heads", "n_kv_heads", "hidden_dim", "seq_len")}))
         res.update(ms_per_step_with_events=(t3 - t2) * 1e3 / steps, attn_kernel_ms=k_ms.value / launches,
                    attn_merge_ms=None if join else m_ms.value / launches, attn_launches=int(n.value), attn_split_join=join)
         # the attention op as it runs in production, its two kernels back to back: one event in front of the pair, one behind
