@@ -676,6 +676,8 @@ def main():
     ap.add_argument("--attn-split-join", type=int, default=1, choices=[0, 1, 4, 8],
                     help="measurement hook: how the splits of a context are added up in the decode attention (1: the library's choice; 0: always partial "
                          "sums and the merge kernel; 4, 8: inside work-groups of that many waves where the plan has 2 or 4 splits)")
+    ap.add_argument("--attn-chunk", type=int, default=0,
+                    help="measurement hook: keys per split of the decode attention (0: the library's plan)")
     ap.add_argument("--concept-path", action="store_true", help="time the named decode workload through the reference's op sequence only")
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="also run a plain D2D copy of this many MiB (reference point for profiler byte counters)")
@@ -705,6 +707,10 @@ def main():
         from glinthawk_amd import _lib, ops
         ops.init(0)
         _lib.check(_lib.lib().gh_attn_set_split_join(args.attn_split_join))
+    if args.attn_chunk > 0:
+        from glinthawk_amd import ops
+        ops.init(0)
+        ops.attn_set_chunk(args.attn_chunk)
     if args.attn_variant != "auto":
         from glinthawk_amd import _lib, ops
         ops.init(0)
