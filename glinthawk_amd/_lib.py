@@ -95,6 +95,7 @@ SIGNATURES = {
     "gh_silu": (_i, [_vp, _vp, _u64, _u64, _i, _vp]),
     "gh_argmax": (_i, [_vp, _vp, _vp, _u64, _u64, _i, _vp]),
     "gh_gemm_set_tuning": (_i, [_i, _i, _i]),
+    "gh_gemm_set_gate_waves": (_i, [_i]),
     "gh_gemm_set_library_rows": (_i, [_u64]),
     "gh_gemm_library_rows": (_u64, []),
     "gh_gemm_library_calls": (_u64, []),

@@ -22,6 +22,7 @@ void gemm_stream_plan( uint64_t s, uint64_t r, uint64_t b, uint32_t* splits_out,
 int gemm_stream_launch( __half* xout, float* partial, const __half* x, const __half* w, uint64_t s, uint64_t r, uint64_t b, uint32_t splits,
                         uint32_t k_per_split, uint32_t rows_per_wg, bool write_partials, hipStream_t st );
 void gemm_stream_tuning( int target_wgs, int depth );
+void gemm_stream_gate_waves( int waves );
 bool gemm_stream_gate_applicable( uint64_t s, uint64_t hidden, uint64_t b, const void* x, const void* w13, const void* hb );
 int gemm_stream_gate_launch( __half* hb, const __half* x, const __half* w13, uint64_t s, uint64_t hidden, uint64_t b, hipStream_t st );
 // 256 x 256 tile kernel for products with enough tiles (gh_gemm_tile256.hip)
@@ -438,6 +439,13 @@ int gh_gemm_set_tuning( int kernel, int target_workgroups, int tile_rows )
   g_force_kernel = kernel;
   gemm_stream_tuning( target_workgroups, 0 );
   gemm_tile256_tuning( tile_rows );
+  return GH_OK;
+}
+
+int gh_gemm_set_gate_waves( int waves )
+{
+  GH_REQUIRE( waves == 0 || waves == 4 || waves == 8, "gh_gemm_set_gate_waves: %d is not 0, 4 or 8", waves );
+  gemm_stream_gate_waves( waves );
   return GH_OK;
 }
 

@@ -81,26 +81,29 @@ __device__ __forceinline__ void stage_w_half( uint4* tile, const WSlab& s, int h
 }
 
 // activations of one register slab: 64 columns x 256 k.  v[h][i], thread t: column t/16 + 16*i, chunk t%16 of half h
+template<int W>
 struct XSlab
 {
-  uint4 v[2][4];
+  uint4 v[2][16 / W];
 };
 
 // `rsrc` starts at the work-group's first column; lane_offset = (t / 16) * row bytes + 16 * (t % 16)
-__device__ __forceinline__ void load_x_half( XSlab& dst, __amdgpu_buffer_rsrc_t rsrc, uint32_t lane_offset, uint32_t ld_bytes, uint32_t kb, int h )
+template<int W>
+__device__ __forceinline__ void load_x_half( XSlab<W>& dst, __amdgpu_buffer_rsrc_t rsrc, uint32_t lane_offset, uint32_t ld_bytes, uint32_t kb, int h )
 {
 #pragma unroll
-  for ( int i = 0; i < 4; i++ ) {
-    dst.v[h][i] = buffer_load16( rsrc, lane_offset + h * 2 * HALF_K, 16 * i * ld_bytes + kb );
+  for ( int i = 0; i < 16 / W; i++ ) {
+    dst.v[h][i] = buffer_load16( rsrc, lane_offset + h * 2 * HALF_K, 4 * W * i * ld_bytes + kb );
   }
 }
 
-__device__ __forceinline__ void stage_x_half( uint4* tile, const XSlab& t, int h )
+template<int W>
+__device__ __forceinline__ void stage_x_half( uint4* tile, const XSlab<W>& t, int h )
 {
   const uint32_t chunk = threadIdx.x & 15;
 #pragma unroll
-  for ( int i = 0; i < 4; i++ ) {
-    const uint32_t col = ( threadIdx.x >> 4 ) + 16 * i;
+  for ( int i = 0; i < 16 / W; i++ ) {
+    const uint32_t col = ( threadIdx.x >> 4 ) + 4 * W * i;
     tile[col * 16 + ( chunk ^ ( col & 15 ) )] = t.v[h][i];
   }
 }
@@ -132,8 +135,8 @@ constexpr int MODE_GATE = 2;  // w = [w1 rows | w3 rows], r = rows of each: stor
 // MODE_GATE: a work-group takes 64 output rows; waves 0, 1 stream them from w1, waves 2, 3 the same
 // rows from w3, so that the two factors of an output element sit in the same lane and accumulator
 // register of a wave pair and meet through LDS after the K loop (no K split in this mode).
-template<int MODE>
-__global__ __launch_bounds__( 256, 2 ) void gemm_stream_kernel( __half* __restrict__ xout,
+template<int MODE, int W = 4>
+__global__ __launch_bounds__( 64 * W, W == 4 ? 2 : 1 ) void gemm_stream_kernel( __half* __restrict__ xout,
                                                              float* __restrict__ partial,
                                                              const __half* __restrict__ x,
                                                              const __half* __restrict__ w,
@@ -145,7 +148,7 @@ __global__ __launch_bounds__( 256, 2 ) void gemm_stream_kernel( __half* __restri
                                                              uint32_t rows_per_wave )
 {
   __shared__ uint4 s_x[2][COLS * 16]; // 2 x 16 KiB
-  __shared__ uint4 s_w[4][32 * 16];   // 4 x 8 KiB, one per wave
+  __shared__ uint4 s_w[W][32 * 16];   // 8 KiB per wave
 
   const uint32_t wave = __builtin_amdgcn_readfirstlane( threadIdx.x >> 6 ); // provably uniform: keeps descriptors in SGPRs
   const uint32_t lane = threadIdx.x & 63;
@@ -157,13 +160,14 @@ __global__ __launch_bounds__( 256, 2 ) void gemm_stream_kernel( __half* __restri
     const uint32_t idx = blockIdx.x >> 3;
     col_slab = idx % n_col_slabs;
     row_block = ( idx / n_col_slabs ) * 8 + ( blockIdx.x & 7 );
-    if ( row_block * ( MODE == MODE_GATE ? 2 : 4 ) * rows_per_wave >= r ) {
+    if ( row_block * ( MODE == MODE_GATE ? W / 2 : W ) * rows_per_wave >= r ) {
       return; // padding of the grid to a multiple of 8 row blocks (whole work-group)
     }
   }
   // a wave owns rows_per_wave (<= 32, a multiple of 4) rows of its 32-row MFMA tile; the others read as zero and are not stored
-  const uint32_t row0 = MODE == MODE_GATE ? ( row_block * 2 + ( wave & 1 ) ) * rows_per_wave : ( row_block * 4 + wave ) * rows_per_wave; // output row
-  const uint32_t w_row0 = MODE == MODE_GATE ? ( wave >> 1 ) * r + row0 : row0;
+  constexpr uint32_t HALF_W = W / 2;
+  const uint32_t row0 = MODE == MODE_GATE ? ( row_block * HALF_W + ( wave % HALF_W ) ) * rows_per_wave : ( row_block * W + wave ) * rows_per_wave; // output row
+  const uint32_t w_row0 = MODE == MODE_GATE ? ( wave / HALF_W ) * r + row0 : row0;
   const uint32_t col0 = col_slab * COLS;
   const uint32_t k_begin = blockIdx.z * k_per_split;
   const uint32_t k_end = min( s, k_begin + k_per_split );
@@ -203,7 +207,7 @@ __global__ __launch_bounds__( 256, 2 ) void gemm_stream_kernel( __half* __restri
   const uint32_t n_slabs = ( k_end - k_begin ) / SLAB_K; // K ranges are multiples of SLAB_K
   uint32_t cur = ( ( row_block + blockIdx.z ) * 3u ) % n_slabs; // rotated start, see the header
   WSlab wr[2];
-  XSlab xr;
+  XSlab<W> xr;
   {
     const uint32_t kb = ( k_begin + cur * SLAB_K ) * 2;
     load_w_slab( wr[0], w_rsrc, w_lane, ld_bytes, kb );
@@ -238,20 +242,20 @@ __global__ __launch_bounds__( 256, 2 ) void gemm_stream_kernel( __half* __restri
   // acc[t][v]: row = 8*(v/4) + 4*(lane/32) + v%4 of the wave's 32, column = 32*t + lane%32
   const uint32_t g2 = lane >> 5;
   if ( MODE == MODE_GATE ) {
-    // waves 2, 3 hand DType(y3) to waves 0, 1 through the activation tile's LDS (16 KiB = 2 x 2 x 16 x 64 floats)
+    // the waves on w3 hand DType(y3) to the waves on w1 through the activation tiles' LDS (W / 2 x 2 x 16 x 64 floats: 16 or 32 KiB)
     float* gate = reinterpret_cast<float*>( s_x[0] );
     __syncthreads(); // every wave is done reading the activation tiles
-    if ( wave >= 2 ) {
+    if ( wave >= HALF_W ) {
 #pragma unroll
       for ( int t = 0; t < 2; t++ ) {
 #pragma unroll
         for ( int v = 0; v < 16; v++ ) {
-          gate[( ( ( wave & 1 ) * 2 + t ) * 16 + v ) * 64 + lane] = __half2float( __float2half_rn( acc[t][v] ) );
+          gate[( ( ( wave % HALF_W ) * 2 + t ) * 16 + v ) * 64 + lane] = __half2float( __float2half_rn( acc[t][v] ) );
         }
       }
     }
     __syncthreads();
-    if ( wave >= 2 ) {
+    if ( wave >= HALF_W ) {
       return;
     }
 #pragma unroll
@@ -336,6 +340,7 @@ __global__ __launch_bounds__( 256, 2 ) void gemm_stream_kernel( __half* __restri
 }
 
 int g_target_wgs = 0; // tuning override of the CU count the plan balances for (0: the device's)
+int g_gate_waves = 0;  // tuning override of the waves per work-group of the one-launch gate product (0: by the rule in its launcher; 4, 8)
 
 void launch( dim3 grid, hipStream_t st, bool split, __half* xout, float* partial, const __half* x, const __half* w, uint32_t s, uint32_t r, uint32_t b,
              uint32_t k_per_split, uint32_t n_col_slabs, uint32_t rows_per_wave )
@@ -432,13 +437,24 @@ int gemm_stream_gate_launch( __half* hb, const __half* x, const __half* w13, uin
   uint32_t splits = 1, k_per_split = 0, rows = 0;
   gemm_stream_plan( s, 2 * hidden, b, &splits, &k_per_split, &rows );
   GH_REQUIRE( splits == 1, "gh_matmul_silu_gate: the one-launch form does not split K" );
-  const uint32_t rows_per_wave = rows / 4; // two waves on w1, two on w3: rows / 2 output rows per work-group
-  const uint64_t row_blocks = ( hidden + 2 * rows_per_wave - 1 ) / ( 2 * rows_per_wave );
+  const uint32_t rows_per_wave = rows / 4; // half of the waves on w1, half on w3
+  // Where work-groups of four waves come two to a CU, one of eight takes their place: the same waves on the same rows, but one
+  // activation tile per slab for all eight instead of one per four.  The activations are a third of what a CU's L1 fetches with
+  // four waves and a fifth with eight, and that L1 is what bounds the stream: 70B w1+w3 at 64 rows, cold weights, 162-167 -> 145-158 us.
+  // (With a K split the work-groups would be too few, or the splits more: wo, wq+wkv and w2 gained nothing or lost.)
+  const uint64_t blocks_of_four = ( hidden + 2 * rows_per_wave - 1 ) / ( 2 * rows_per_wave );
+  const uint32_t waves = g_gate_waves != 0 ? (uint32_t)g_gate_waves : ( blocks_of_four >= 2ull * (uint64_t)cu_count() ? 8u : 4u );
+  const uint64_t row_blocks = ( hidden + ( waves / 2 ) * rows_per_wave - 1 ) / ( ( waves / 2 ) * rows_per_wave );
   const uint64_t col_slabs = ( b + COLS - 1 ) / COLS;
   const uint64_t gx = col_slabs == 1 ? row_blocks : ( row_blocks + 7 ) / 8 * 8 * col_slabs;
   GH_REQUIRE( gx < ( 1ull << 31 ), "gh_matmul_silu_gate: grid too large" );
-  gemm_stream_kernel<MODE_GATE><<<dim3( (unsigned)gx, 1, 1 ), 256, 0, st>>>( hb, nullptr, x, w13, (uint32_t)s, (uint32_t)hidden, (uint32_t)b, (uint32_t)s,
-                                                                         (uint32_t)col_slabs, rows_per_wave );
+  if ( waves == 8 ) {
+    gemm_stream_kernel<MODE_GATE, 8><<<dim3( (unsigned)gx, 1, 1 ), 512, 0, st>>>( hb, nullptr, x, w13, (uint32_t)s, (uint32_t)hidden, (uint32_t)b, (uint32_t)s,
+                                                                              (uint32_t)col_slabs, rows_per_wave );
+  } else {
+    gemm_stream_kernel<MODE_GATE><<<dim3( (unsigned)gx, 1, 1 ), 256, 0, st>>>( hb, nullptr, x, w13, (uint32_t)s, (uint32_t)hidden, (uint32_t)b, (uint32_t)s,
+                                                                           (uint32_t)col_slabs, rows_per_wave );
+  }
   GH_LAUNCH_CHECK();
   return GH_OK;
 }
@@ -450,5 +466,7 @@ void gemm_stream_tuning( int target_wgs, int depth )
   }
   (void)depth;
 }
+
+void gemm_stream_gate_waves( int waves ) { g_gate_waves = waves == 4 || waves == 8 ? waves : 0; }
 
 } // namespace gh

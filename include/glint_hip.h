@@ -156,6 +156,9 @@ int gh_argmax( uint32_t* out_host, uint32_t* out_dev, const void* v, uint64_t n,
  * 384 weight rows per work-group of eight waves, 128 = four waves of 128 x 128 with one tile per work-group, 129 = four waves over equal shares of
  * all K steps with the fix-up kernel, 0 = the library's choice (GLINT_TILE_ROWS in the environment sets the start value) */
 int gh_gemm_set_tuning( int kernel, int target_workgroups, int tile_rows );
+/* measurement / test hook: waves per work-group of the decode product that computes w1 and w3 in one launch and applies the SiLU gate itself
+ * (gh_matmul_silu_gate at up to 64 rows without a K split): 4, 8, or 0 = the library's choice (8 where work-groups of 4 would come two to a CU) */
+int gh_gemm_set_gate_waves( int waves );
 /* Opt-in: plain f16 products (gh_matmul, the two of gh_matmul_pair, the product inside gh_matmul_accum and gh_matmul_silu_gate where no
  * kernel of this library fuses it) of `rows` activation rows and more go to the vendor's GEMM library, as every product of the
  * reference's GPU target does (cublasGemmEx, arch/cuda/common/ops.cuh:666-700); from half as many rows on for weight matrices that

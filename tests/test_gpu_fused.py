@@ -5,7 +5,7 @@ import pytest
 import torch
 
 import oracle as O
-from glinthawk_amd import Shape, ops, stage as S
+from glinthawk_amd import Shape, _lib, ops, stage as S
 from helpers import Arena, assert_close, assert_half_parity, oracle_cfg
 from test_gpu_stage import SHAPES, OracleModel, d2h, load_weights, make_weights
 
@@ -57,6 +57,23 @@ def test_matmul_accum_and_norm(dt, b, s, r, product_route):
                                         (64, 512, 16384), (5, 256, 16404), (33, 1024, 28672),
                                         (5, 256, 16386)])     # rows not a multiple of 4: the two-kernel route
 def test_matmul_silu_gate(dt, b, s, hidden, product_route):
+    check_matmul_silu_gate(dt, b, s, hidden, product_route)
+
+
+@pytest.mark.parametrize("waves", [4, 8])
+@pytest.mark.parametrize("b,s,hidden", [(64, 512, 16384), (5, 256, 16404), (33, 1024, 28672), (64, 8192, 3584), (17, 768, 16500)])
+def test_matmul_silu_gate_one_launch_with_four_and_eight_waves(waves, b, s, hidden, product_route):
+    """The one-launch form (w1 and w3 rows of the same outputs in one work-group, gate in the epilogue) with work-groups of four
+    and of eight waves, whichever the library would pick for the shape: row counts that leave the last work-group and the last
+    wave partly empty, few and many columns."""
+    _lib.check(_lib.lib().gh_gemm_set_gate_waves(waves))
+    try:
+        check_matmul_silu_gate(torch.float16, b, s, hidden, product_route)
+    finally:
+        _lib.check(_lib.lib().gh_gemm_set_gate_waves(0))
+
+
+def check_matmul_silu_gate(dt, b, s, hidden, product_route):
     g = torch.Generator(device="cuda").manual_seed(2)
     x = torch.randn((b, s), generator=g, device="cuda").to(dt)
     w13 = (torch.randn((2 * hidden, s), generator=g, device="cuda") / s ** 0.5).to(dt)
