@@ -676,6 +676,8 @@ def main():
     ap.add_argument("--attn-split-join", type=int, default=1, choices=[0, 1, 4, 8],
                     help="measurement hook: how the splits of a context are added up in the decode attention (1: the library's choice; 0: always partial "
                          "sums and the merge kernel; 4, 8: inside work-groups of that many waves where the plan has 2 or 4 splits)")
+    ap.add_argument("--gate-waves", type=int, default=0, choices=[0, 4, 8],
+                    help="measurement hook: waves per work-group of the decode product that computes w1 and w3 in one launch (0: the library's choice)")
     ap.add_argument("--attn-chunk", type=int, default=0,
                     help="measurement hook: keys per split of the decode attention (0: the library's plan)")
     ap.add_argument("--concept-path", action="store_true", help="time the named decode workload through the reference's op sequence only")
@@ -711,6 +713,10 @@ def main():
         from glinthawk_amd import ops
         ops.init(0)
         ops.attn_set_chunk(args.attn_chunk)
+    if args.gate_waves:
+        from glinthawk_amd import _lib, ops
+        ops.init(0)
+        _lib.check(_lib.lib().gh_gemm_set_gate_waves(args.gate_waves))
     if args.attn_variant != "auto":
         from glinthawk_amd import _lib, ops
         ops.init(0)
