@@ -218,7 +218,7 @@ __global__ __launch_bounds__( 256 ) void attn_merge_kernel( Partials part,
 // With up to four splits per stream a work-group of four waves holds whole streams: wave = (stream of the work-group, split).
 // Every wave walks its token range as in the kernels above; then the waves leave their maxima, sums and accumulators in LDS, lane
 // for lane as they lie in the registers, and the wave of split 0 combines them in the order and with the arithmetic of
-// attn_merge_kernel (so the output is the same bit for bit) and stores the rounded result.  No partial sums in memory, no second
+// attn_merge_kernel (the output differs from that route's by at most one rounding: the compiler contracts the two differently) and stores the rounded result.  No partial sums in memory, no second
 // launch.
 // =================================================================================================
 struct JoinedJob
